@@ -1,0 +1,89 @@
+"""ctypes binding of libdiffulex_amd.so (declarations follow include/diffulex_amd.h).
+
+There is no fallback: if the library is missing the import of any operator
+raises, so a GPU run can never silently take another path.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from pathlib import Path
+
+LIB_PATH = Path(__file__).resolve().parent / "libdiffulex_amd.so"
+
+DFX_ABI_VERSION = 1
+DFX_OK = 0
+DFX_KV_BF16, DFX_KV_FP8_E4M3 = 0, 1
+DFX_MASK_FULL, DFX_MASK_BLOCK_CAUSAL = 0, 1
+DFX_INDEX_I32, DFX_INDEX_I64 = 0, 1
+
+EXPORTS = (
+    "dfx_abi_version", "dfx_status_string", "dfx_kv_store_unified", "dfx_kv_store_distinct",
+    "dfx_kv_load", "dfx_paged_attn_workspace_bytes", "dfx_paged_attn",
+)
+
+
+class AttnParams(C.Structure):
+    """Mirror of ``dfx_attn_params``."""
+    _fields_ = [
+        ("q", C.c_void_p), ("k_new", C.c_void_p), ("v_new", C.c_void_p),
+        ("k_cache", C.c_void_p), ("v_cache", C.c_void_p), ("out", C.c_void_p),
+        ("block_tables", C.c_void_p), ("context_lens", C.c_void_p),
+        ("cu_seqlens_q", C.c_void_p), ("cu_seqlens_new", C.c_void_p),
+        ("k_scale", C.c_void_p), ("v_scale", C.c_void_p),
+        ("workspace", C.c_void_p), ("workspace_bytes", C.c_int64),
+        ("q_stride_token", C.c_int64), ("q_stride_head", C.c_int64),
+        ("kn_stride_token", C.c_int64), ("kn_stride_head", C.c_int64),
+        ("vn_stride_token", C.c_int64), ("vn_stride_head", C.c_int64),
+        ("o_stride_token", C.c_int64), ("o_stride_head", C.c_int64),
+        ("cache_stride_page", C.c_int64), ("cache_stride_token", C.c_int64), ("cache_stride_head", C.c_int64),
+        ("block_table_stride", C.c_int64), ("n_pages", C.c_int64),
+        ("num_seqs", C.c_int32), ("num_q_heads", C.c_int32), ("num_kv_heads", C.c_int32), ("head_dim", C.c_int32),
+        ("page_size", C.c_int32), ("max_pages_per_seq", C.c_int32), ("max_seqlen_q", C.c_int32),
+        ("diffusion_block_size", C.c_int32), ("kv_dtype", C.c_int32), ("mask_mode", C.c_int32),
+        ("max_workgroups", C.c_int32), ("scale", C.c_float),
+    ]
+
+
+class DfxError(RuntimeError):
+    pass
+
+
+_lib = None
+
+
+def load() -> C.CDLL:
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not LIB_PATH.exists():
+        raise ImportError(
+            f"{LIB_PATH} is missing: build the gfx950 kernels first (python -m diffulex_amd.build). "
+            "diffulex_amd has no fallback path.")
+    lib = C.CDLL(str(LIB_PATH))
+    i64, i32, vp = C.c_int64, C.c_int, C.c_void_p
+    lib.dfx_abi_version.restype = i32
+    lib.dfx_abi_version.argtypes = []
+    lib.dfx_status_string.restype = C.c_char_p
+    lib.dfx_status_string.argtypes = [i32]
+    lib.dfx_kv_store_unified.restype = i32
+    lib.dfx_kv_store_unified.argtypes = [vp, vp, i64, i64, vp, vp, vp, i32, i64, i64, i32, i32, i32, vp, vp, vp]
+    lib.dfx_kv_store_distinct.restype = i32
+    lib.dfx_kv_store_distinct.argtypes = [vp, vp, i64, i64, vp, vp, C.POINTER(i64), C.POINTER(i64), vp, i32,
+                                          i64, i64, i32, i32, i32, i32, vp]
+    lib.dfx_kv_load.restype = i32
+    lib.dfx_kv_load.argtypes = [vp, vp, vp, vp, i64, i64, vp, vp, vp, i64, vp, vp, vp, vp, i32, i32, i64, i32,
+                                i32, i32, i64, i32, vp, vp, vp]
+    lib.dfx_paged_attn_workspace_bytes.restype = i64
+    lib.dfx_paged_attn_workspace_bytes.argtypes = [C.POINTER(AttnParams)]
+    lib.dfx_paged_attn.restype = i32
+    lib.dfx_paged_attn.argtypes = [C.POINTER(AttnParams), vp]
+    if lib.dfx_abi_version() != DFX_ABI_VERSION:
+        raise ImportError(f"{LIB_PATH} has ABI {lib.dfx_abi_version()}, expected {DFX_ABI_VERSION}: rebuild it")
+    _lib = lib
+    return lib
+
+
+def check(status: int, what: str) -> None:
+    if status != DFX_OK:
+        msg = load().dfx_status_string(int(status)).decode()
+        raise DfxError(f"{what}: {msg} ({status})")

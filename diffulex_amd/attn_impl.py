@@ -1,0 +1,50 @@
+"""The ``Attention`` module: the operator boundary the model layers call.
+
+Mirrors diffulex/attention/attn_impl.py:13-72: reshape, optional KV-cache store,
+prefill / decode dispatch, flatten heads.  ``k_cache`` / ``v_cache`` are assigned
+from outside (diffulex/engine/model_runner.py:239-243).
+"""
+from __future__ import annotations
+
+import torch
+import torch.nn as nn
+
+from . import metadata as _metadata
+from .dllm_flash_attn import dllm_flash_attn_decode, dllm_flash_attn_prefill
+from .kv_cache_kernels import store_kvcache_distinct_layout, store_kvcache_unified_layout
+
+
+class Attention(nn.Module):
+    def __init__(self, num_heads, head_dim, scale, num_kv_heads):
+        super().__init__()
+        self.num_heads = num_heads
+        self.head_dim = head_dim
+        self.scale = scale
+        self.num_kv_heads = num_kv_heads
+        self.k_cache = self.v_cache = torch.tensor([])
+        # looked up at call time so that a later set_fetch_fn_for_attn_metadata() is seen
+        self.fetch_attn_metadata = lambda: _metadata.fetch_attn_metadata()
+
+    def forward(self, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask=None) -> torch.Tensor:
+        q = q.view(q.shape[0], self.num_heads, self.head_dim)
+        k = k.view(k.shape[0], self.num_kv_heads, self.head_dim)
+        v = v.view(v.shape[0], self.num_kv_heads, self.head_dim)
+
+        attn_metadata = self.fetch_attn_metadata()
+        k_cache, v_cache = self.k_cache, self.v_cache
+        is_unified_layout = attn_metadata.kv_cache_layout == "unified"
+
+        if k_cache.numel() and v_cache.numel():
+            if attn_metadata.need_kv_cache_store:
+                store_kvcache = store_kvcache_unified_layout if is_unified_layout else store_kvcache_distinct_layout
+                store_kvcache(k, v, k_cache, v_cache, attn_metadata.slot_mapping, attn_metadata)
+
+        if attn_metadata.is_prefill:
+            o = dllm_flash_attn_prefill(q, k, v, self.scale, attn_metadata)
+        else:
+            if is_unified_layout:
+                o = dllm_flash_attn_decode(q, k, v, k_cache, v_cache, self.scale, attn_metadata)
+            else:
+                raise NotImplementedError("Distinct layout is not supported yet...")
+
+        return o.reshape(o.shape[0], self.num_heads * self.head_dim).contiguous()

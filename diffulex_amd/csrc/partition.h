@@ -1,0 +1,62 @@
+// Work partition of the paged-attention kernel, shared by the device code and by
+// host-side tests (plain C++, no HIP dependency).
+//
+// Work is measured in "units": one unit is one KV tile (kTileTokens tokens of one KV head of
+// one sequence) processed for one row tile of that sequence's queries.  Sequence s owns
+//     units(s) = n_tiles(s) * n_row_tiles(s)
+// consecutive units (row-tile major), the sequences follow each other, and the whole list is
+// repeated for every KV head.  The linear unit space [0, total) is cut into n_wg equal
+// ranges, one per persistent workgroup; wherever a cut falls inside a (sequence, head, row
+// tile) item the two sides produce partial results that a combine pass merges.
+#pragma once
+
+#include <stdint.h>
+
+#ifndef DFX_HD
+#define DFX_HD inline
+#endif
+
+namespace dfx {
+
+constexpr int kTileTokens = 64;
+
+DFX_HD int ceil_div(int a, int b) { return (a + b - 1) / b; }
+
+struct SeqShape {
+    int ctx;        // cached tokens
+    int q_len;      // query rows of the sequence
+    int new_len;    // fresh K/V rows
+    int n_ctx_tiles;
+    int n_tiles;    // KV tiles: context tiles then fresh tiles (never mixed in one tile)
+    int n_row_tiles;
+    int units;
+};
+
+DFX_HD SeqShape make_seq_shape(int ctx, int q_len, int new_len, int group, int rows_per_tile) {
+    SeqShape s;
+    s.ctx = ctx > 0 ? ctx : 0;
+    s.q_len = q_len > 0 ? q_len : 0;
+    s.new_len = new_len > 0 ? new_len : 0;
+    s.n_ctx_tiles = ceil_div(s.ctx, kTileTokens);
+    s.n_tiles = s.n_ctx_tiles + ceil_div(s.new_len, kTileTokens);
+    s.n_row_tiles = ceil_div(group * s.q_len, rows_per_tile);
+    s.units = s.n_tiles * s.n_row_tiles;
+    return s;
+}
+
+// First unit of workgroup w (w == n_wg gives total).
+DFX_HD int64_t wg_first_unit(int w, int64_t total, int n_wg) { return (static_cast<int64_t>(w) * total) / n_wg; }
+
+// The workgroup whose range contains unit u: the largest w with wg_first_unit(w) <= u.
+DFX_HD int wg_of_unit(int64_t u, int64_t total, int n_wg) {
+    return static_cast<int>(((u + 1) * n_wg - 1) / total);
+}
+
+// A workgroup writes at most two partial results: slot 2w for a piece that starts at the
+// first unit of its range, slot 2w+1 for a piece that starts later (it then necessarily
+// runs to the end of the range).
+DFX_HD int partial_slot(int w, int64_t piece_begin, int64_t wg_begin) {
+    return 2 * w + (piece_begin != wg_begin ? 1 : 0);
+}
+
+}  // namespace dfx

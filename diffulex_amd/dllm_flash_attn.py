@@ -1,0 +1,149 @@
+"""Block-diffusion attention operators (same names and arguments as
+diffulex_kernel/python/dllm_flash_attn.py:539-637), backed by one gfx950 kernel.
+
+Both decode modes of the reference run the same fused paged kernel here: it reads
+the cached prefix through the block table and the fresh K/V from the operands, so
+the "varlen" mode needs no ``load_kvcache`` gather and no second pass over K/V.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from typing import Optional
+
+import torch
+
+from . import _lib
+from .kv_cache_kernels import _FP8_DTYPES, _scales, _stream
+
+_workspaces = {}
+
+
+def _workspace(device: torch.device, stream: int, nbytes: int) -> torch.Tensor:
+    key = (device.index, stream)
+    ws = _workspaces.get(key)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=device)
+        _workspaces[key] = ws
+    return ws
+
+
+def paged_attention(q, k, v, k_cache, v_cache, scale, *, block_tables, context_lens, cu_seqlens_q,
+                    cu_seqlens_new, max_seqlen_q, mask_mode=_lib.DFX_MASK_FULL, diffusion_block_size=32,
+                    k_scale=None, v_scale=None, max_workgroups=0, out=None) -> torch.Tensor:
+    """Marshal tensors into ``dfx_attn_params`` and launch ``dfx_paged_attn`` on the
+    current stream.  q: [T, H_q, hd]; k, v: [T_new, H_kv, hd]; caches
+    [pages, page, H_kv, hd] or None."""
+    lib = _lib.load()
+    assert q.is_cuda and q.dtype == torch.bfloat16 and k.dtype == torch.bfloat16 and v.dtype == torch.bfloat16
+    assert q.dim() == 3 and k.dim() == 3 and v.shape == k.shape
+    assert q.stride(-1) == 1 and k.stride(-1) == 1 and v.stride(-1) == 1
+    T, H_q, hd = q.shape
+    H_kv = k.shape[1]
+    assert k.shape[2] == hd and H_q % H_kv == 0
+    num_seqs = cu_seqlens_q.numel() - 1
+    assert cu_seqlens_new.numel() == num_seqs + 1
+    for t in (cu_seqlens_q, cu_seqlens_new):
+        assert t.dtype == torch.int32 and t.is_cuda and t.is_contiguous()
+    if out is None:
+        out = torch.empty((T, H_q, hd), dtype=q.dtype, device=q.device)
+    p = _lib.AttnParams()
+    keep = ()
+    has_cache = k_cache is not None and k_cache.numel() > 0
+    if has_cache:
+        assert k_cache.shape == v_cache.shape and k_cache.dim() == 4
+        assert k_cache.shape[2] == H_kv and k_cache.shape[3] == hd
+        assert k_cache.stride() == v_cache.stride() and k_cache.stride(-1) == 1
+        assert block_tables is not None and block_tables.dtype == torch.int32 and block_tables.stride(-1) == 1
+        assert context_lens is not None and context_lens.dtype == torch.int32 and context_lens.is_contiguous()
+        assert block_tables.shape[0] == num_seqs and context_lens.numel() == num_seqs
+        kv_dtype, ksp, vsp, keep = _scales(k_cache, None, k_scale, v_scale, H_kv)
+        p.k_cache, p.v_cache = k_cache.data_ptr(), v_cache.data_ptr()
+        p.block_tables, p.context_lens = block_tables.data_ptr(), context_lens.data_ptr()
+        p.k_scale, p.v_scale = ksp, vsp
+        p.cache_stride_page, p.cache_stride_token, p.cache_stride_head = k_cache.stride()[:3]
+        p.block_table_stride = block_tables.stride(0)
+        p.n_pages, p.page_size = k_cache.shape[0], k_cache.shape[1]
+        p.max_pages_per_seq = block_tables.shape[1]
+        p.kv_dtype = kv_dtype
+    else:
+        p.kv_dtype = _lib.DFX_KV_BF16
+    p.q, p.k_new, p.v_new, p.out = q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr()
+    p.cu_seqlens_q, p.cu_seqlens_new = cu_seqlens_q.data_ptr(), cu_seqlens_new.data_ptr()
+    p.q_stride_token, p.q_stride_head = q.stride(0), q.stride(1)
+    p.kn_stride_token, p.kn_stride_head = k.stride(0), k.stride(1)
+    p.vn_stride_token, p.vn_stride_head = v.stride(0), v.stride(1)
+    p.o_stride_token, p.o_stride_head = out.stride(0), out.stride(1)
+    p.num_seqs, p.num_q_heads, p.num_kv_heads, p.head_dim = num_seqs, H_q, H_kv, hd
+    p.max_seqlen_q = int(max_seqlen_q)
+    p.diffusion_block_size = int(diffusion_block_size)
+    p.mask_mode = int(mask_mode)
+    p.max_workgroups = int(max_workgroups)
+    p.scale = float(scale)
+    need = lib.dfx_paged_attn_workspace_bytes(C.byref(p))
+    if need < 0:
+        _lib.check(int(need), "dfx_paged_attn_workspace_bytes")
+    stream = _stream()
+    ws = _workspace(q.device, stream, int(need))
+    p.workspace, p.workspace_bytes = ws.data_ptr(), ws.numel()
+    _lib.check(lib.dfx_paged_attn(C.byref(p), stream), "dfx_paged_attn")
+    return out
+
+
+def _max_seqlen_q(attn_metadata, cu_seqlens_q) -> int:
+    m = int(getattr(attn_metadata, "max_seqlen_q", 0) or 0)
+    if m <= 0:  # not supplied: one host read
+        m = int((cu_seqlens_q[1:] - cu_seqlens_q[:-1]).max().item())
+    return m
+
+
+def dllm_flash_attn_prefill(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float,
+                            attn_metadata) -> torch.Tensor:
+    """dllm_flash_attn.py:539-596: varlen self-attention of each sequence; every key visible
+    for ``attn_type == "full_attention"``, the block-causal mask
+    ``kv_j < (q_i // DBS + 1) * DBS`` for ``"block_attention"`` (dllm_flash_attn.py:109-116)."""
+    if attn_metadata.attn_type == "full_attention":
+        mask = _lib.DFX_MASK_FULL
+    elif attn_metadata.attn_type == "block_attention":
+        mask = _lib.DFX_MASK_BLOCK_CAUSAL
+    else:
+        raise ValueError(f"unknown attn_type {attn_metadata.attn_type!r}")
+    return paged_attention(
+        q, k, v, None, None, scale, block_tables=None, context_lens=None,
+        cu_seqlens_q=attn_metadata.cu_seqlens_q, cu_seqlens_new=attn_metadata.cu_seqlens_k,
+        max_seqlen_q=_max_seqlen_q(attn_metadata, attn_metadata.cu_seqlens_q), mask_mode=mask,
+        diffusion_block_size=attn_metadata.diffusion_block_size)
+
+
+def dllm_flash_attn_decode(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, k_cache: torch.Tensor,
+                           v_cache: torch.Tensor, scale: float, attn_metadata,
+                           k_scale: Optional[torch.Tensor] = None,
+                           v_scale: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """dllm_flash_attn.py:599-637.
+
+    ``decode_mode == "static"``: ``cu_seqlens_k`` indexes the fresh K/V rows
+    (strategy/block_diffusion/engine/model_runner.py:134-139).
+    ``decode_mode == "varlen"``: ``cu_seqlens_k`` spans context + fresh rows and the
+    fresh rows are addressed through ``cu_seqlens_q``
+    (strategy/d2f/engine/model_runner.py:161-167, kv_cache_kernels.py:186-227).
+    ``scale`` is honoured in both modes.  ``attn_metadata.decode_mask ==
+    "block_causal"`` (optional attribute) selects the block-causal mask among the
+    in-flight blocks; the default is the reference's behaviour, all fresh tokens visible.
+    """
+    if attn_metadata.decode_mode == "static":
+        cu_new = attn_metadata.cu_seqlens_k
+    elif attn_metadata.decode_mode == "varlen":
+        cu_new = attn_metadata.cu_seqlens_q
+    else:
+        raise ValueError(f"unknown decode_mode {attn_metadata.decode_mode!r}")
+    mask = _lib.DFX_MASK_FULL
+    if getattr(attn_metadata, "decode_mask", "full") == "block_causal":
+        mask = _lib.DFX_MASK_BLOCK_CAUSAL
+    if k_cache.dtype in _FP8_DTYPES:
+        k_scale = k_scale if k_scale is not None else getattr(attn_metadata, "k_scale", None)
+        v_scale = v_scale if v_scale is not None else getattr(attn_metadata, "v_scale", None)
+    return paged_attention(
+        q, k, v, k_cache, v_cache, scale, block_tables=attn_metadata.block_tables,
+        context_lens=attn_metadata.context_lens, cu_seqlens_q=attn_metadata.cu_seqlens_q,
+        cu_seqlens_new=cu_new, max_seqlen_q=_max_seqlen_q(attn_metadata, attn_metadata.cu_seqlens_q),
+        mask_mode=mask, diffusion_block_size=attn_metadata.diffusion_block_size,
+        k_scale=k_scale, v_scale=v_scale)

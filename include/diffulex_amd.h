@@ -1,0 +1,175 @@
+/*
+ * diffulex_amd: C ABI of the MI355X (gfx950) dLLM decoding hot path.
+ *
+ * One shared library, libdiffulex_amd.so, exports the functions below.  They
+ * take plain device pointers, element strides, sizes and a HIP stream; they
+ * never allocate, never synchronise with the host and never throw.  Every
+ * function returns 0 (DFX_OK) or a negative dfx_status; on a non-zero return
+ * nothing has been launched.
+ *
+ * "Replaces" names the reference (zhijie-group/Diffulex) interface whose device
+ * work the entry point takes over; paths are relative to the reference tree.
+ */
+#ifndef DIFFULEX_AMD_H_
+#define DIFFULEX_AMD_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define DFX_ABI_VERSION 1
+
+typedef void* dfx_stream_t; /* a hipStream_t; NULL is the default stream */
+
+typedef enum dfx_status {
+    DFX_OK = 0,
+    DFX_ERR_INVALID_ARG = -1, /* null pointer, negative size, misaligned pointer or stride */
+    DFX_ERR_UNSUPPORTED = -2, /* a shape this build has no kernel for (see each function) */
+    DFX_ERR_WORKSPACE = -3,   /* workspace missing or smaller than dfx_paged_attn_workspace_bytes */
+    DFX_ERR_LAUNCH = -4       /* the HIP runtime refused the launch */
+} dfx_status;
+
+typedef enum dfx_kv_dtype {
+    DFX_KV_BF16 = 0,    /* 2-byte elements, copied bit for bit (bf16; fp16 works for store/load) */
+    DFX_KV_FP8_E4M3 = 1 /* OCP e4m3fn codes with one fp32 scale per KV head */
+} dfx_kv_dtype;
+
+typedef enum dfx_mask_mode {
+    DFX_MASK_FULL = 0,        /* every fresh token of the sequence is visible to every query */
+    DFX_MASK_BLOCK_CAUSAL = 1 /* fresh token j visible to query i iff j < (i / dbs + 1) * dbs */
+} dfx_mask_mode;
+
+typedef enum dfx_index_type { DFX_INDEX_I32 = 0, DFX_INDEX_I64 = 1 } dfx_index_type;
+
+/* ABI version of the loaded library (== DFX_ABI_VERSION it was built with). */
+int dfx_abi_version(void);
+
+/* Static string for a dfx_status value. */
+const char* dfx_status_string(int status);
+
+/*
+ * Paged KV-cache store, unified layout.
+ * Replaces: store_kvcache_unified_layout + dllm_store_kvcache_kernel_unified
+ *           (diffulex_kernel/python/kv_cache_kernels.py:110-124, :11-32).
+ *
+ * key/value: [n_tokens, n_kv_heads, head_dim] bf16, innermost two dims dense,
+ * row stride key_stride / value_stride (elements).  Caches: [n_slots, n_kv_heads,
+ * head_dim] dense, n_slots = pages * page_size.  For each token t with
+ * slot = slot_mapping[t]: slot < 0 is skipped, otherwise cache[slot] = row t.
+ * slot >= n_slots is skipped as well (the reference would write out of bounds).
+ * Duplicate slots are a caller error (unordered writes), as in the reference.
+ *
+ * kv_dtype == DFX_KV_FP8_E4M3: caches hold 1-byte codes and each element is
+ * stored as RNE_e4m3fn(clamp(float(x) / scale[head], -448, 448)); k_scale and
+ * v_scale are fp32[n_kv_heads].  With DFX_KV_BF16 they must be NULL.
+ */
+int dfx_kv_store_unified(const void* key, const void* value, int64_t key_stride, int64_t value_stride,
+                         void* k_cache, void* v_cache, const void* slot_mapping, int slot_index_type,
+                         int64_t n_tokens, int64_t n_slots, int n_kv_heads, int head_dim, int kv_dtype,
+                         const float* k_scale, const float* v_scale, dfx_stream_t stream);
+
+/*
+ * Paged KV-cache store, "distinct" (vLLM-style) layout.
+ * Replaces: store_kvcache_distinct_layout + dllm_store_kvcache_kernel_distinct
+ *           (diffulex_kernel/python/kv_cache_kernels.py:86-107, :35-83).
+ *
+ * k_cache: [pages, H, head_dim / x, page_size, x], v_cache: [pages, H, head_dim,
+ * page_size], both 2-byte elements, addressed through the element strides given
+ * (kc_stride: pages, H, head_dim/x, page_size, x; vc_stride: pages, H, head_dim,
+ * page_size).  Element (h, d) of token t with slot s goes to
+ * k_cache[s / page_size, h, d / x, s % page_size, d % x] and
+ * v_cache[s / page_size, h, d, s % page_size].
+ */
+int dfx_kv_store_distinct(const void* key, const void* value, int64_t key_stride, int64_t value_stride,
+                          void* k_cache, void* v_cache, const int64_t kc_stride[5], const int64_t vc_stride[4],
+                          const void* slot_mapping, int slot_index_type, int64_t n_tokens, int64_t n_pages,
+                          int page_size, int x, int n_kv_heads, int head_dim, dfx_stream_t stream);
+
+/*
+ * Paged KV-cache load: gather every sequence's cached context through its block
+ * table and append its fresh K/V rows, into packed [total, n_kv_heads, head_dim]
+ * buffers of the cache's element type.
+ * Replaces: load_kvcache + load_kvcache_kernel
+ *           (diffulex_kernel/python/kv_cache_kernels.py:230-279, :127-227).
+ *
+ * Sequence s writes rows [cu_seqlens_k[s], cu_seqlens_k[s] + context_lens[s])
+ * from pages block_tables[s, 0..], page p contributing min(page_size,
+ * context - p * page_size) rows (a full last page IS copied, unlike the reference
+ * kernel), then seq_lens_new[s] rows from k_new/v_new starting at row
+ * cu_seqlens_q[s].  max_total_len bounds the rows of any one sequence (it sizes
+ * the launch; larger sequences would be truncated, smaller values waste nothing).
+ * Outputs are caller-allocated.  With DFX_KV_FP8_E4M3 the fresh rows (bf16) are
+ * quantised with k_scale/v_scale as in dfx_kv_store_unified.
+ */
+int dfx_kv_load(const void* k_cache, const void* v_cache, const void* k_new, const void* v_new,
+                int64_t k_new_stride, int64_t v_new_stride, void* k_out, void* v_out,
+                const int32_t* block_tables, int64_t block_table_stride, const int32_t* context_lens,
+                const int32_t* seq_lens_new, const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k,
+                int num_seqs, int max_pages_per_seq, int64_t n_pages, int page_size, int n_kv_heads,
+                int head_dim, int64_t max_total_len, int kv_dtype, const float* k_scale,
+                const float* v_scale, dfx_stream_t stream);
+
+/*
+ * Block-diffusion paged attention.
+ * Replaces: dllm_flash_attn_decode (both decode modes) and its TileLang kernels
+ *           (diffulex_kernel/python/dllm_flash_attn.py:599-637, :163-347, :350-536),
+ *           including the load_kvcache + flash_attn_varlen_func pair of the
+ *           "varlen" mode, and, with k_cache == NULL, dllm_flash_attn_prefill
+ *           (dllm_flash_attn.py:539-596, :23-160).
+ *
+ * For every sequence s, query rows q[cu_seqlens_q[s] .. cu_seqlens_q[s+1]) attend
+ * to (a) the context_lens[s] cached tokens reached through block_tables[s, :]
+ * and (b) the fresh rows k_new/v_new[cu_seqlens_new[s] .. cu_seqlens_new[s+1]),
+ * masked by mask_mode (query i and fresh token j are indices inside the
+ * sequence's own rows).  O = softmax(scale * Q K^T) V with fp32 accumulation,
+ * GQA by kv_head = q_head / (num_q_heads / num_kv_heads).
+ *
+ * Supported: head_dim 64 or 128; num_q_heads a multiple of num_kv_heads; any
+ * page_size >= 1; num_seqs <= 4095; scale > 0.  Strides are in elements; the
+ * innermost (head_dim) dimension of q, k_new, v_new, out and the caches is dense
+ * and every row start is 16-byte aligned.
+ */
+typedef struct dfx_attn_params {
+    const void* q;               /* [T_q, num_q_heads, head_dim] bf16 */
+    const void* k_new;           /* [T_new, num_kv_heads, head_dim] bf16 */
+    const void* v_new;
+    const void* k_cache;         /* [n_pages, page_size, num_kv_heads, head_dim]; NULL: no cached context */
+    const void* v_cache;
+    void* out;                   /* [T_q, num_q_heads, head_dim] bf16 */
+    const int32_t* block_tables; /* [num_seqs, block_table_stride]; entries < 0 are never dereferenced */
+    const int32_t* context_lens; /* [num_seqs]; NULL means 0 everywhere */
+    const int32_t* cu_seqlens_q;   /* [num_seqs + 1] */
+    const int32_t* cu_seqlens_new; /* [num_seqs + 1] offsets of the fresh K/V rows */
+    const float* k_scale;        /* fp32 [num_kv_heads], DFX_KV_FP8_E4M3 only */
+    const float* v_scale;
+    void* workspace;             /* >= dfx_paged_attn_workspace_bytes(), 256-byte aligned */
+    int64_t workspace_bytes;
+    int64_t q_stride_token, q_stride_head;
+    int64_t kn_stride_token, kn_stride_head; /* k_new */
+    int64_t vn_stride_token, vn_stride_head; /* v_new */
+    int64_t o_stride_token, o_stride_head;
+    int64_t cache_stride_page, cache_stride_token, cache_stride_head; /* same for k_cache and v_cache */
+    int64_t block_table_stride;
+    int64_t n_pages;
+    int32_t num_seqs, num_q_heads, num_kv_heads, head_dim;
+    int32_t page_size, max_pages_per_seq;
+    int32_t max_seqlen_q;        /* upper bound of any sequence's query rows */
+    int32_t diffusion_block_size;
+    int32_t kv_dtype;            /* dfx_kv_dtype of the caches (k_new/v_new are always bf16) */
+    int32_t mask_mode;           /* dfx_mask_mode */
+    int32_t max_workgroups;      /* 0: one per compute unit; >0 caps the persistent grid */
+    float scale;
+} dfx_attn_params;
+
+/* Bytes of scratch dfx_paged_attn needs for these shapes (depends on the sizes
+ * and max_workgroups only, never on device data). Negative: dfx_status. */
+int64_t dfx_paged_attn_workspace_bytes(const dfx_attn_params* params);
+
+int dfx_paged_attn(const dfx_attn_params* params, dfx_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DIFFULEX_AMD_H_ */

@@ -1,0 +1,103 @@
+// Host-side test hooks: expose the host/device helper code of diffulex_amd/csrc to the
+// CPU test-suite (compiled with the host compiler only; nothing here runs on a GPU).
+#include <cstdint>
+#include <vector>
+
+#include "../../diffulex_amd/csrc/fp8_e4m3.h"
+#include "../../diffulex_amd/csrc/partition.h"
+
+extern "C" {
+
+void hook_quantise_e4m3(const float* x, float scale, uint8_t* out, int64_t n) {
+    for (int64_t i = 0; i < n; ++i) out[i] = dfx::quantise_e4m3(x[i], scale);
+}
+
+void hook_e4m3_to_f32(const uint8_t* codes, float* out, int64_t n) {
+    for (int64_t i = 0; i < n; ++i) out[i] = dfx::e4m3fn_to_f32(codes[i]);
+}
+
+void hook_bf16_round(const float* x, uint16_t* out, int64_t n) {
+    for (int64_t i = 0; i < n; ++i) out[i] = dfx::f32_to_bf16_bits(x[i]);
+}
+
+// Replays the persistent kernel's walk over its unit range on the host.  For workgroup w it
+// appends one record per segment: {w, kv_head, seq, row_tile, tile0, tile1, complete, slot}.
+// ctx/q_len/new_len: per-sequence lengths.  Returns the number of records (<= cap).
+int64_t hook_walk_segments(const int* ctx, const int* q_len, const int* new_len, int num_seqs, int h_kv, int group,
+                           int rows_per_tile, int n_wg, int64_t* rec, int64_t cap) {
+    using namespace dfx;
+    std::vector<SeqShape> sh(num_seqs);
+    std::vector<int> prefix(num_seqs + 1, 0);
+    for (int s = 0; s < num_seqs; ++s) {
+        sh[s] = make_seq_shape(ctx[s], q_len[s], new_len[s], group, rows_per_tile);
+        prefix[s + 1] = prefix[s] + sh[s].units;
+    }
+    const int per_head = prefix[num_seqs];
+    const int64_t total = static_cast<int64_t>(per_head) * h_kv;
+    int64_t n = 0;
+    if (total == 0) return 0;
+    for (int w = 0; w < n_wg; ++w) {
+        const int64_t begin = wg_first_unit(w, total, n_wg), end = wg_first_unit(w + 1, total, n_wg);
+        if (begin >= end) continue;
+        int kvh = static_cast<int>(begin / per_head);
+        const int rem = static_cast<int>(begin - static_cast<int64_t>(kvh) * per_head);
+        int s = 0;
+        while (!(prefix[s] <= rem && rem < prefix[s + 1])) ++s;
+        int u = rem - prefix[s];
+        int64_t pos = begin;
+        while (pos < end) {
+            const int n_tiles = sh[s].n_tiles;
+            const int rt = u / n_tiles, tile0 = u - rt * n_tiles;
+            const int64_t seg_end = pos + (n_tiles - tile0) < end ? pos + (n_tiles - tile0) : end;
+            const int tile1 = tile0 + static_cast<int>(seg_end - pos);
+            const bool complete = tile0 == 0 && tile1 == n_tiles;
+            if (n < cap) {
+                int64_t* r = rec + n * 8;
+                r[0] = w; r[1] = kvh; r[2] = s; r[3] = rt; r[4] = tile0; r[5] = tile1; r[6] = complete;
+                r[7] = partial_slot(w, pos, begin);
+            }
+            ++n;
+            u += tile1 - tile0;
+            pos = seg_end;
+            if (pos >= end) break;
+            if (u == sh[s].units) {
+                u = 0;
+                do {
+                    if (++s == num_seqs) { s = 0; ++kvh; }
+                } while (prefix[s + 1] == prefix[s]);
+            }
+        }
+    }
+    return n;
+}
+
+// What the combine pass derives for item (kv_head, seq, row_tile): the slots it merges.
+// Returns the number of slots written (0: the item was not cut), -1 if the item is empty.
+int hook_combine_slots(const int* ctx, const int* q_len, const int* new_len, int num_seqs, int h_kv, int group,
+                       int rows_per_tile, int n_wg, int kvh, int s, int rt, int* slots, int cap) {
+    using namespace dfx;
+    int before = 0, all = 0;
+    SeqShape mine{};
+    for (int i = 0; i < num_seqs; ++i) {
+        const SeqShape sh = make_seq_shape(ctx[i], q_len[i], new_len[i], group, rows_per_tile);
+        if (i < s) before += sh.units;
+        if (i == s) mine = sh;
+        all += sh.units;
+    }
+    if (rt >= mine.n_row_tiles || mine.n_tiles == 0) return -1;
+    const int64_t total = static_cast<int64_t>(all) * h_kv;
+    const int64_t item_begin = static_cast<int64_t>(kvh) * all + before + static_cast<int64_t>(rt) * mine.n_tiles;
+    const int64_t item_end = item_begin + mine.n_tiles;
+    const int wa = wg_of_unit(item_begin, total, n_wg), wb = wg_of_unit(item_end - 1, total, n_wg);
+    if (wa == wb) return 0;
+    int n = 0;
+    for (int w = wa; w <= wb; ++w) {
+        const int64_t ws = wg_first_unit(w, total, n_wg), we = wg_first_unit(w + 1, total, n_wg);
+        if (ws >= we) continue;
+        const int64_t pb = ws > item_begin ? ws : item_begin;
+        if (n < cap) slots[n] = partial_slot(w, pb, ws);
+        ++n;
+    }
+    return n;
+}
+}

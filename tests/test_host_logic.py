@@ -1,0 +1,144 @@
+"""CPU tests of the library's host-side logic: exported symbols, argument checking, the
+host/device helper code (FP8 quantiser, bf16 rounding) and the work partition."""
+import ctypes as C
+import re
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from diffulex_amd import _lib
+from oracle import fp8_e4m3
+import hosthooks
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_library_exports_every_declared_symbol():
+    header = open(os.path.join(ROOT, "include", "diffulex_amd.h")).read()
+    declared = set(re.findall(r"\b(dfx_[a-z0-9_]+)\s*\(", header))
+    assert declared == set(_lib.EXPORTS)
+    lib = _lib.load()
+    for name in declared:
+        assert getattr(lib, name) is not None
+    assert lib.dfx_abi_version() == _lib.DFX_ABI_VERSION
+    assert lib.dfx_status_string(0) == b"ok"
+    assert lib.dfx_status_string(-2) == b"unsupported shape"
+
+
+def test_struct_layout_matches_header():
+    # 14 pointers/int64 + 13 int64 + 11 int32 + 1 float, no padding surprises
+    assert C.sizeof(_lib.AttnParams) == 8 * 27 + 4 * 12
+
+
+def test_argument_errors_do_not_launch():
+    lib = _lib.load()
+    # null pointers with non-zero sizes
+    assert lib.dfx_kv_store_unified(None, None, 512, 512, None, None, None, 0, 4, 16, 4, 128, 0, None, None, None) == -1
+    # zero tokens is a no-op
+    assert lib.dfx_kv_store_unified(None, None, 512, 512, None, None, None, 0, 0, 16, 4, 128, 0, None, None, None) == 0
+    # bad index type / dtype
+    assert lib.dfx_kv_store_unified(16, 16, 512, 512, 16, 16, 16, 7, 4, 16, 4, 128, 0, None, None, None) == -1
+    assert lib.dfx_kv_store_unified(16, 16, 512, 512, 16, 16, 16, 0, 4, 16, 4, 128, 1, None, None, None) == -1
+    p = _lib.AttnParams()
+    p.num_seqs, p.num_q_heads, p.num_kv_heads, p.head_dim = 2, 28, 4, 96
+    assert lib.dfx_paged_attn_workspace_bytes(C.byref(p)) == -2       # head_dim 96 unsupported
+    p.head_dim, p.num_q_heads = 128, 30
+    assert lib.dfx_paged_attn_workspace_bytes(C.byref(p)) == -1       # 30 % 4 != 0
+    p.num_q_heads, p.max_workgroups, p.max_seqlen_q = 28, 8, 32
+    need = lib.dfx_paged_attn_workspace_bytes(C.byref(p))
+    assert need == 2 * 8 * 256 * (2 * 4 * 4 * 4 + 4) * 4               # NB = 2 (224 rows), hd 128
+    assert lib.dfx_paged_attn(C.byref(p), None) == -1                  # null tensors
+
+
+def test_device_quantiser_source_matches_oracle_on_host():
+    hooks = hosthooks.load()
+    bits = (np.arange(65536, dtype=np.uint32) << 16)
+    x = bits.view(np.float32)
+    x = np.ascontiguousarray(x[np.isfinite(x)])
+    out = np.zeros(x.shape, dtype=np.uint8)
+    for scale in (1.0, 0.0123, 3.7, 2.0 ** -20, 11.0, 0.0078125):
+        hooks.hook_quantise_e4m3(x.ctypes.data, C.c_float(scale), out.ctypes.data, x.size)
+        want = fp8_e4m3.quantize_per_head(x.reshape(-1, 1, 1), np.array([scale], np.float32)).reshape(-1)
+        assert np.array_equal(out, want), scale
+    codes = np.arange(256, dtype=np.uint8)
+    f = np.zeros(256, dtype=np.float32)
+    hooks.hook_e4m3_to_f32(codes.ctypes.data, f.ctypes.data, 256)
+    want = fp8_e4m3.decode_e4m3fn(codes)
+    ok = ~np.isnan(want)
+    assert np.array_equal(f[ok].view(np.uint32), want[ok].view(np.uint32)) and np.all(np.isnan(f[~ok]))
+
+
+def test_bf16_rounding_helper_matches_torch():
+    hooks = hosthooks.load()
+    rng = np.random.default_rng(1)
+    x = np.concatenate([rng.standard_normal(100000).astype(np.float32),
+                        np.array([0.0, -0.0, 1.0, 1.00390625, 1.01171875, 3.3895314e38, np.inf, -np.inf], np.float32)])
+    out = np.zeros(x.shape, dtype=np.uint16)
+    hooks.hook_bf16_round(x.ctypes.data, out.ctypes.data, x.size)
+    want = torch.from_numpy(x).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+    assert np.array_equal(out, want)
+
+
+def _walk(hooks, ctx, q_len, new_len, h_kv, group, rows_per_tile, n_wg):
+    ctx, q_len, new_len = (np.ascontiguousarray(a, dtype=np.int32) for a in (ctx, q_len, new_len))
+    cap = 200000
+    rec = np.zeros((cap, 8), dtype=np.int64)
+    n = hooks.hook_walk_segments(ctx.ctypes.data, q_len.ctypes.data, new_len.ctypes.data, len(ctx), h_kv, group,
+                                 rows_per_tile, n_wg, rec.ctypes.data, cap)
+    assert n <= cap
+    return rec[:n]
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_partition_covers_every_tile_once_and_combine_finds_the_pieces(seed):
+    hooks = hosthooks.load()
+    rng = np.random.default_rng(seed)
+    b = int(rng.integers(1, 40))
+    h_kv = int(rng.integers(1, 5))
+    group = int(rng.choice([1, 2, 4, 7, 8]))
+    rows_per_tile = int(rng.choice([128, 256]))
+    n_wg = int(rng.choice([1, 2, 3, 7, 64, 256, 1000]))
+    ctx = rng.integers(0, 700, b)
+    q_len = rng.choice([0, 32, 64, 96, 200], b)
+    new_len = np.where(q_len > 0, q_len, 0)
+    if seed % 3 == 0:
+        ctx[rng.integers(0, b)] = 0
+    rec = _walk(hooks, ctx, q_len, new_len, h_kv, group, rows_per_tile, n_wg)
+    ctx32, q32, new32 = (np.ascontiguousarray(a, dtype=np.int32) for a in (ctx, q_len, new_len))
+    # expected tiles per item
+    seen = {}
+    slots_by_item = {}
+    slot_owner = {}
+    for w, kvh, s, rt, t0, t1, complete, slot in rec.tolist():
+        n_tiles = -(-int(ctx[s]) // 64) + -(-int(new_len[s]) // 64)
+        assert 0 <= t0 < t1 <= n_tiles
+        assert bool(complete) == (t0 == 0 and t1 == n_tiles)
+        cover = seen.setdefault((kvh, s, rt), [])
+        cover.append((t0, t1))
+        if not complete:
+            assert slot in (2 * w, 2 * w + 1)
+            assert slot not in slot_owner, "a partial slot is written twice"
+            slot_owner[slot] = (kvh, s, rt)
+            slots_by_item.setdefault((kvh, s, rt), []).append(slot)
+    for kvh in range(h_kv):
+        for s in range(b):
+            n_tiles = -(-int(ctx[s]) // 64) + -(-int(new_len[s]) // 64)
+            n_rt = -(-group * int(q_len[s]) // rows_per_tile)
+            for rt in range(n_rt):
+                if n_tiles == 0:
+                    continue
+                pieces = sorted(seen[(kvh, s, rt)])
+                assert pieces[0][0] == 0 and pieces[-1][1] == n_tiles
+                for a, bb in zip(pieces, pieces[1:]):
+                    assert a[1] == bb[0]
+                # combine pass derives the same slots
+                out = np.zeros(4096, dtype=np.int32)
+                n = hooks.hook_combine_slots(ctx32.ctypes.data, q32.ctypes.data, new32.ctypes.data, b, h_kv, group,
+                                             rows_per_tile, n_wg, kvh, s, rt, out.ctypes.data, 4096)
+                want = sorted(slots_by_item.get((kvh, s, rt), []))
+                assert sorted(out[:n].tolist()) == want
+    assert len(seen) == sum(1 for kvh in range(h_kv) for s in range(b)
+                            for rt in range(-(-group * int(q_len[s]) // rows_per_tile))
+                            if -(-int(ctx[s]) // 64) + -(-int(new_len[s]) // 64) > 0)

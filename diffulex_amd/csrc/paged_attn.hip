@@ -570,8 +570,8 @@ __global__ void __launch_bounds__(kThreads) paged_attn_kernel(const KArgs a) {
 // merge its pieces and write the rows; otherwise the main kernel has already written them.
 template <int HD, int NB>
 __global__ void __launch_bounds__(kThreads) paged_attn_combine_kernel(const KArgs a) {
-    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-    Attn<HD, NB, false> at(a, smem);
+    __shared__ int scan_scratch[kWaves];
+    Attn<HD, NB, false> at(a, nullptr);  // no LDS stages here: only the register state and the epilogue
     using C = Cfg<HD, NB>;
     const int rt = blockIdx.x, s = blockIdx.y, kvh = blockIdx.z;
     // units before sequence s and per-head total, by a strided block reduction
@@ -582,8 +582,8 @@ __global__ void __launch_bounds__(kThreads) paged_attn_combine_kernel(const KArg
         if (sq < s) before += u;
     }
     int tot_all, tot_before;
-    block_inclusive_scan(all, at.misc, tot_all);
-    block_inclusive_scan(before, at.misc, tot_before);
+    block_inclusive_scan(all, scan_scratch, tot_all);
+    block_inclusive_scan(before, scan_scratch, tot_before);
     at.set_sequence(s, kvh);
     if (rt >= at.sh.n_row_tiles || at.sh.n_tiles == 0) return;
     const int64_t total = static_cast<int64_t>(tot_all) * a.h_kv;
@@ -681,7 +681,7 @@ int launch(const KArgs& ka, const Plan& plan, int rt_max, hipStream_t st) {
     hipLaunchKernelGGL(main_k, dim3(plan.n_wg), dim3(kThreads), lds, st, ka);
     if (hipGetLastError() != hipSuccess) return DFX_ERR_LAUNCH;
     if (plan.n_wg > 1 && rt_max > 0) {
-        hipLaunchKernelGGL(comb_k, dim3(rt_max, ka.num_seqs, ka.h_kv), dim3(kThreads), 64, st, ka);
+        hipLaunchKernelGGL(comb_k, dim3(rt_max, ka.num_seqs, ka.h_kv), dim3(kThreads), 0, st, ka);
         if (hipGetLastError() != hipSuccess) return DFX_ERR_LAUNCH;
     }
     return DFX_OK;

@@ -131,7 +131,10 @@ def load_kvcache(k_cache: torch.Tensor, v_cache: torch.Tensor, attn_metadata,
     v_output = torch.empty_like(k_output)
     bt = attn_metadata.block_tables
     assert bt.stride(1) == 1
-    rc = lib.dfx_kv_load(k_cache.data_ptr(), v_cache.data_ptr(), k_new.data_ptr(), v_new.data_ptr(),
+    # an empty tensor has a null data pointer; no fresh row is read then, any valid pointer serves
+    kn_ptr = k_new.data_ptr() if k_new.numel() else k_cache.data_ptr()
+    vn_ptr = v_new.data_ptr() if v_new.numel() else v_cache.data_ptr()
+    rc = lib.dfx_kv_load(k_cache.data_ptr(), v_cache.data_ptr(), kn_ptr, vn_ptr,
                          k_new.stride(0), v_new.stride(0), k_output.data_ptr(), v_output.data_ptr(),
                          bt.data_ptr(), bt.stride(0), ctxlens.data_ptr(), seqlens.data_ptr(),
                          cu_seqlens_q.data_ptr(), cu_seqlens_k.data_ptr(), NUM_SEQS, MAX_SEQ_BLOCKS,

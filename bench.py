@@ -1,0 +1,172 @@
+#!/usr/bin/env python3
+"""Headline benchmark: block-diffusion paged attention at the Dream-7B shape on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c4|c5] [--no-cpu]
+
+One step = one pass of the decode attention (``dfx_paged_attn``) over one synthetic batch
+(workload C3: 64 sequences, 28 query / 4 KV heads, head_dim 128, 256-token bf16 pages, prefix
+lengths uniform in [512, 2048], one 32-token diffusion block of queries per sequence).  Inputs
+are resident in HBM before the timed region; the KV cache is rotated over several independent
+copies so that consecutive steps cannot be served from the 256 MB Infinity Cache.
+
+Prints ONE JSON line: the metric (attention query tokens per second), the roofline position of
+the kernel (algorithmic bytes per launch / measured launch time against the 8 TB/s HBM peak)
+and the CPU baseline (the reference's PyTorch path, per-sequence gather + library SDPA in bf16,
+timed on this host's cores on a bounded slice of the same workload).
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
+MFMA_BF16_PEAK_TFLOPS = 2500.0
+# HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this command, scaled by
+# what the same counters read for a plain copy of known size (see profiles/); None until measured.
+MEASURED_TRAFFIC_BYTES = {}
+
+
+def algorithmic_bytes(wl) -> int:
+    kv_elt = wl.k_cache.element_size()
+    ctx = int(wl.context_lens.sum())
+    tq = int(wl.q.shape[0])
+    tn = int(wl.k_new.shape[0])
+    return (ctx * wl.num_kv_heads * wl.head_dim * 2 * kv_elt          # K + V prefix, once per KV head
+            + 2 * tq * wl.num_q_heads * wl.head_dim * 2                 # Q read, O written
+            + tn * wl.num_kv_heads * wl.head_dim * 2 * 2)               # fresh K, V
+
+
+def algorithmic_flops(wl) -> int:
+    from diffulex_amd.workloads import MASK_BLOCK_CAUSAL
+    ctx = wl.context_lens.tolist()
+    pairs = 0
+    for c in ctx:
+        ql = wl.q_len
+        if wl.mask_mode == MASK_BLOCK_CAUSAL:
+            vis = sum(min(ql, (i // wl.diffusion_block_size + 1) * wl.diffusion_block_size) for i in range(ql))
+        else:
+            vis = ql * ql
+        pairs += ql * c + vis
+    return 4 * wl.num_q_heads * wl.head_dim * pairs
+
+
+def cpu_baseline(name: str, budget_s: float = 15.0):
+    """The reference's PyTorch path on the host cores, on a bounded batch slice."""
+    from diffulex_amd.workloads import make_workload
+    from oracle import attention as oat
+    cores = os.cpu_count() or 1
+    cores = min(cores, 16)  # the GPU box gives 16 cores to a one-GPU job
+    torch.set_num_threads(cores)
+    from diffulex_amd.workloads import SPECS
+    n_seqs = min(SPECS[name]["num_seqs"], 16 if name == "c5" else 64)
+    wl = make_workload(name, num_seqs=n_seqs)
+
+    def run():
+        return oat.paged_attention_sdpa(wl.q, wl.k_new, wl.v_new, wl.k_cache, wl.v_cache, wl.block_tables,
+                                        wl.context_lens, wl.cu_seqlens_q, wl.cu_seqlens_q, wl.scale,
+                                        mask_mode=wl.mask_mode, dbs=wl.diffusion_block_size,
+                                        k_scale=wl.k_scale, v_scale=wl.v_scale)
+    run()  # warm-up
+    times = []
+    t_start = time.perf_counter()
+    while len(times) < 3 or (time.perf_counter() - t_start < budget_s and len(times) < 500):
+        t0 = time.perf_counter()
+        run()
+        times.append(time.perf_counter() - t0)
+    times.sort()
+    med = times[len(times) // 2]
+    return {
+        "value": wl.total_q_tokens / med, "unit": "query-tokens/s", "cores": cores, "kind": "port",
+        "sample": f"{n_seqs}-sequence slice of workload {name} (same shape, seeded), median of {len(times)} "
+                  f"runs of the per-sequence gather + torch SDPA (bf16) path; {med * 1e3:.1f} ms per run",
+        "gbs": algorithmic_bytes(wl) / med / 1e9,
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default="c3", choices=["c3", "c4", "c5", "c1"])
+    ap.add_argument("--copies", type=int, default=4, help="independent KV-cache copies rotated between steps")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: this path shards by KV head / sequence with no exchange step, "
+                 "and this build runs on a single MI355X (use --gpus 1)")
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU (the HIP kernels have no CPU fallback)")
+
+    import diffulex_amd as dfx
+    from diffulex_amd.workloads import make_workload
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    wl = make_workload(args.workload, device=dev)
+    caches = [(wl.k_cache, wl.v_cache)]
+    for _ in range(args.copies - 1):
+        caches.append((wl.k_cache.clone(), wl.v_cache.clone()))
+    kw = dict(block_tables=wl.block_tables, context_lens=wl.context_lens, cu_seqlens_q=wl.cu_seqlens_q,
+              cu_seqlens_new=wl.cu_seqlens_q, max_seqlen_q=wl.q_len, mask_mode=wl.mask_mode,
+              diffusion_block_size=wl.diffusion_block_size, k_scale=wl.k_scale, v_scale=wl.v_scale)
+    out = torch.empty_like(wl.q)
+
+    def step(i):
+        kc, vc = caches[i % len(caches)]
+        dfx.paged_attention(wl.q, wl.k_new, wl.v_new, kc, vc, wl.scale, out=out, **kw)
+
+    for i in range(args.warmup):
+        step(i)
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    start.record()
+    for i in range(args.steps):
+        step(i)
+    stop.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    ms = start.elapsed_time(stop) / args.steps
+
+    nbytes, nflops = algorithmic_bytes(wl), algorithmic_flops(wl)
+    gbs = nbytes / (ms * 1e-3) / 1e9
+    tflops = nflops / (ms * 1e-3) / 1e12
+    result = {
+        "metric": "attn query-tokens/sec + achieved HBM GB/s (% of peak), Dream-7B shape, 1 GPU",
+        "value": wl.total_q_tokens / (ms * 1e-3), "unit": "query-tokens/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16" if not wl.kv_fp8 else "bf16 (fp8-e4m3 KV)", "data": "synthetic",
+        "config": {
+            "workload": f"{args.workload}: block-diffusion paged attention, B={wl.num_seqs}, H_q={wl.num_q_heads}, "
+                        f"H_kv={wl.num_kv_heads}, head_dim={wl.head_dim}, page={wl.page_size}, "
+                        f"ctx in [{int(wl.context_lens.min())},{int(wl.context_lens.max())}] "
+                        f"(sum {int(wl.context_lens.sum())}), q_len={wl.q_len}, "
+                        f"mask={'block-causal' if wl.mask_mode else 'full'}, kv={'fp8-e4m3' if wl.kv_fp8 else 'bf16'}",
+            "kv_cache_copies_rotated": len(caches),
+            "host_wall_ms_per_step": wall_ms / args.steps,
+        },
+        "roofline": {
+            "bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS,
+            "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
+            "algorithmic_bytes": nbytes, "algorithmic_flops": nflops,
+            "mfma_tflops": tflops, "mfma_frac": tflops / MFMA_BF16_PEAK_TFLOPS,
+            "kernel": "paged_attn_kernel (+ combine pass), duration = timed region / steps",
+        },
+    }
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline(args.workload)
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

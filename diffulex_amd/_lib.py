@@ -15,6 +15,7 @@ DFX_OK = 0
 DFX_KV_BF16, DFX_KV_FP8_E4M3 = 0, 1
 DFX_MASK_FULL, DFX_MASK_BLOCK_CAUSAL = 0, 1
 DFX_INDEX_I32, DFX_INDEX_I64 = 0, 1
+DFX_ATTN_GENERIC_PATH = 1
 
 EXPORTS = (
     "dfx_abi_version", "dfx_status_string", "dfx_kv_store_unified", "dfx_kv_store_distinct",
@@ -40,7 +41,7 @@ class AttnParams(C.Structure):
         ("num_seqs", C.c_int32), ("num_q_heads", C.c_int32), ("num_kv_heads", C.c_int32), ("head_dim", C.c_int32),
         ("page_size", C.c_int32), ("max_pages_per_seq", C.c_int32), ("max_seqlen_q", C.c_int32),
         ("diffusion_block_size", C.c_int32), ("kv_dtype", C.c_int32), ("mask_mode", C.c_int32),
-        ("max_workgroups", C.c_int32), ("scale", C.c_float),
+        ("max_workgroups", C.c_int32), ("flags", C.c_int32), ("scale", C.c_float),
     ]
 
 

@@ -21,7 +21,7 @@ ARCH = "gfx950"
 
 # packed-fp32 instructions are kept out of the generated code on purpose
 HIP_FLAGS = [
-    f"--offload-arch={ARCH}", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function",
+    f"--offload-arch={ARCH}", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function", "-Wno-inline-asm",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
 ]
 SOURCES = ["capi.cpp", "kv_cache.hip", "paged_attn.hip"]

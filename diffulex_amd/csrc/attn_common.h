@@ -1,0 +1,346 @@
+// State and arithmetic shared by the paged-attention kernels: kernel arguments, the per-lane
+// attention state of one (sequence, KV head, row tile) item, the online softmax on S^T and
+// the epilogues (normalised rows, partial results, merge of partial results).
+//
+// MFMA 32x32x16 bf16 register layouts relied upon (lane l, h = l / 32):
+//   A: row l % 32, contraction elements 8h .. 8h+7        B: column l % 32, same elements
+//   C/D: column l % 32, rows 8*i + 4*h + j for accumulator index 4*i + j
+// S^T = K Q^T puts one query in one lane column, so the softmax row statistics are a
+// register reduction plus one cross-half shuffle, and the S^T accumulators, rounded to bf16,
+// are already the B operand of O^T += V^T P^T: elements 8*sl .. 8*sl+7 of block tb are
+// tokens 32*tb + 16*sl + {4h..4h+3, 8+4h..8+4h+3}.
+#pragma once
+
+#include "dfx_common.h"
+#include "partition.h"
+
+namespace dfx {
+
+constexpr int kThreads = 256;
+constexpr int kWaves = 4;
+constexpr int kMaxSeqs = 4095;
+constexpr float kLog2e = 1.4426950408889634f;
+
+struct KArgs {
+    const uint16_t* q;
+    const uint16_t* k_new;
+    const uint16_t* v_new;
+    const uint8_t* k_cache;
+    const uint8_t* v_cache;
+    uint16_t* out;
+    const int32_t* block_tables;
+    const int32_t* context_lens;
+    const int32_t* cu_q;
+    const int32_t* cu_new;
+    const float* k_scale;
+    const float* v_scale;
+    float* workspace;
+    int64_t q_st, q_sh, kn_st, kn_sh, vn_st, vn_sh, o_st, o_sh;
+    int64_t c_sp, c_st, c_sh;  // cache strides in elements: page, token, head
+    int64_t bt_stride, n_pages;
+    int num_seqs, h_kv, group, page_size, page_shift, max_pages, dbs, mask_mode, n_wg;
+    float c;  // scale * log2(e)
+};
+
+// Sizes that do not depend on how a kernel stages its tiles.
+template <int HD, int NB>
+struct Shape {
+    static constexpr int TN = kTileTokens;
+    static constexpr int RT = 32 * NB * kWaves;  // query rows per row tile
+    static constexpr int NSLAB = HD / 16;        // contraction slabs of Q K^T
+    static constexpr int NDB = HD / 32;          // 32-row blocks of O^T
+    static constexpr int PREFIX_BYTES = (kMaxSeqs + 1) * 4;
+    static constexpr int MISC_BYTES = 64;
+    static constexpr int O_VEC4 = NB * NDB * 4;  // float4 per lane in a partial result
+    static constexpr int SLOT_FLOATS = kThreads * (O_VEC4 * 4 + 2 * NB);
+};
+
+DFX_D float wave_xor32_max(float x) { return fmaxf(x, __shfl_xor(x, 32)); }
+
+DFX_D float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+DFX_D int block_inclusive_scan(int v, int* scratch, int& block_total) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    int x = v;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+        const int y = __shfl_up(x, d);
+        if (lane >= d) x += y;
+    }
+    if (lane == 63) scratch[wave] = x;
+    __syncthreads();
+    int off = 0, tot = 0;
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) {
+        const int t = scratch[w];
+        if (w < wave) off += t;
+        tot += t;
+    }
+    __syncthreads();
+    block_total = tot;
+    return x + off;
+}
+
+DFX_D SeqShape load_seq_shape(const KArgs& a, int s, int rows_per_tile) {
+    const int ctx = (a.context_lens != nullptr && a.k_cache != nullptr) ? a.context_lens[s] : 0;
+    const int q_len = a.cu_q[s + 1] - a.cu_q[s];
+    const int new_len = a.cu_new[s + 1] - a.cu_new[s];
+    return make_seq_shape(ctx, q_len, new_len, a.group, rows_per_tile);
+}
+
+// What the softmax needs to know about one KV tile.
+struct TileInfo {
+    int base;      // index of the tile's first token within its kind (context or fresh)
+    int limit;     // number of valid tokens of that kind
+    bool is_ctx;
+    float c_tile;  // logit -> log2 domain factor (scale * log2 e, times k_scale for FP8 context)
+    float v_mul;   // factor applied to P before the PV product (v_scale for FP8 context, else 1)
+};
+
+template <int HD, int NB>
+struct AttnState {
+    using S = Shape<HD, NB>;
+
+    const KArgs& a;
+    const int tid, lane, wave, col, half;
+
+    SeqShape sh;
+    int s, kvh, q0, n0;
+    bf16x8 qf[NB][S::NSLAB];
+    f32x16 o[S::NDB][NB];
+    float m_run[NB], l_run[NB];
+    int vis_limit[NB];
+
+    DFX_D explicit AttnState(const KArgs& args)
+        : a(args), tid(threadIdx.x), lane(threadIdx.x & 63), wave(threadIdx.x >> 6), col(threadIdx.x & 31),
+          half((threadIdx.x >> 5) & 1) {}
+
+    DFX_D void set_sequence(int seq, int kv_head) {
+        s = seq;
+        kvh = kv_head;
+        sh = load_seq_shape(a, s, S::RT);
+        q0 = a.cu_q[s];
+        n0 = a.cu_new[s];
+    }
+
+    DFX_D TileInfo tile_info(const SeqShape& shp, int kv_head, int tile, bool fp8) const {
+        TileInfo t;
+        t.is_ctx = tile < shp.n_ctx_tiles;
+        t.base = (t.is_ctx ? tile : tile - shp.n_ctx_tiles) * S::TN;
+        t.limit = t.is_ctx ? shp.ctx : shp.new_len;
+        t.c_tile = a.c;
+        t.v_mul = 1.0f;
+        if (fp8 && t.is_ctx) {
+            t.c_tile = fmaxf(a.c * a.k_scale[kv_head], 1e-30f);
+            t.v_mul = a.v_scale[kv_head];
+        }
+        return t;
+    }
+
+    DFX_D int row_of(int rt, int qb) const { return rt * S::RT + wave * (32 * NB) + qb * 32 + col; }
+
+    DFX_D void reset_accumulators() {
+#pragma unroll
+        for (int qb = 0; qb < NB; ++qb) {
+            m_run[qb] = -INFINITY;
+            l_run[qb] = 0.0f;
+#pragma unroll
+            for (int db = 0; db < S::NDB; ++db)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) o[db][qb][e] = 0.0f;
+        }
+    }
+
+    // Q rows of row tile rt into B-operand registers (zeros for rows past G * q_len).
+    DFX_D void load_queries(int rt) {
+#pragma unroll
+        for (int qb = 0; qb < NB; ++qb) {
+            const int r = row_of(rt, qb);
+            const bool valid = r < a.group * sh.q_len;
+            const int g = valid ? r / sh.q_len : 0;
+            const int i = valid ? r - g * sh.q_len : 0;
+            vis_limit[qb] = (i / a.dbs + 1) * a.dbs;
+            const uint16_t* qp = a.q + (q0 + i) * a.q_st + (kvh * a.group + g) * a.q_sh + half * 8;
+#pragma unroll
+            for (int slab = 0; slab < S::NSLAB; ++slab) {
+                u32x4 v = {0, 0, 0, 0};
+                if (valid) v = *reinterpret_cast<const u32x4*>(qp + slab * 16);
+                qf[qb][slab] = __builtin_bit_cast(bf16x8, v);
+            }
+        }
+        reset_accumulators();
+    }
+
+    // Mask, online softmax and bf16 rounding of one tile's S^T; updates m_run, l_run and
+    // rescales o when a row maximum grows.  pb[qb][tb][sl] is the B operand of the PV product.
+    template <bool SCALE_P>
+    DFX_D void softmax_tile(f32x16 (&sc)[2][NB], const TileInfo& t, bf16x8 (&pb)[NB][2][2]) {
+        const bool mask_valid = t.base + S::TN > t.limit;
+        const bool mask_bc = !t.is_ctx && a.mask_mode == DFX_MASK_BLOCK_CAUSAL;
+        if (mask_valid || mask_bc) {
+#pragma unroll
+            for (int qb = 0; qb < NB; ++qb) {
+                int lim = t.limit;
+                if (mask_bc) lim = min(lim, vis_limit[qb]);
+#pragma unroll
+                for (int tb = 0; tb < 2; ++tb)
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) {
+                        const int tok = t.base + tb * 32 + (e >> 2) * 8 + half * 4 + (e & 3);
+                        if (tok >= lim) sc[tb][qb][e] = -INFINITY;
+                    }
+            }
+        }
+#pragma unroll
+        for (int qb = 0; qb < NB; ++qb) {
+            float mx = -INFINITY;
+#pragma unroll
+            for (int tb = 0; tb < 2; ++tb)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) mx = fmaxf(mx, sc[tb][qb][e]);
+            mx = wave_xor32_max(mx);
+            const float m_new = fmaxf(m_run[qb], mx * t.c_tile);
+            if (__any(m_new > m_run[qb])) {
+                const float alpha = (m_new == -INFINITY) ? 1.0f : fast_exp2(m_run[qb] - m_new);
+                l_run[qb] *= alpha;
+#pragma unroll
+                for (int db = 0; db < S::NDB; ++db)
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) o[db][qb][e] *= alpha;
+                m_run[qb] = m_new;
+            }
+            const float m_safe = (m_run[qb] == -INFINITY) ? 0.0f : m_run[qb];
+            float lsum = 0.0f;
+#pragma unroll
+            for (int tb = 0; tb < 2; ++tb) {
+                float p[16];
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    p[e] = fast_exp2(__builtin_fmaf(sc[tb][qb][e], t.c_tile, -m_safe));
+                    lsum += p[e];
+                    if (SCALE_P) p[e] *= t.v_mul;
+                }
+#pragma unroll
+                for (int sl = 0; sl < 2; ++sl) {
+                    bf16x8 v;
+#pragma unroll
+                    for (int e = 0; e < 8; e += 2) {
+                        const bf16x2 r = __builtin_convertvector(f32x2{p[sl * 8 + e], p[sl * 8 + e + 1]}, bf16x2);
+                        v[e] = r.x;
+                        v[e + 1] = r.y;
+                    }
+                    pb[qb][tb][sl] = v;
+                }
+            }
+            l_run[qb] += lsum;
+        }
+    }
+
+    DFX_D void row_sums(float (&l_tot)[NB]) const {
+#pragma unroll
+        for (int qb = 0; qb < NB; ++qb) l_tot[qb] = l_run[qb] + __shfl_xor(l_run[qb], 32);
+    }
+
+    // Normalised rows: accumulator 4*i + j of block db is element d = 32*db + 8*i + 4*half + j.
+    DFX_D void store_output(int rt, const float (&l_tot)[NB]) const {
+#pragma unroll
+        for (int qb = 0; qb < NB; ++qb) {
+            const int r = row_of(rt, qb);
+            if (r >= a.group * sh.q_len) continue;
+            const int g = r / sh.q_len;
+            const int i = r - g * sh.q_len;
+            const float inv = 1.0f / l_tot[qb];
+            uint16_t* op = a.out + (q0 + i) * a.o_st + (kvh * a.group + g) * a.o_sh + half * 4;
+#pragma unroll
+            for (int db = 0; db < S::NDB; ++db)
+#pragma unroll
+                for (int ii = 0; ii < 4; ++ii) {
+                    const bf16x2 lo = __builtin_convertvector(
+                        f32x2{o[db][qb][ii * 4 + 0] * inv, o[db][qb][ii * 4 + 1] * inv}, bf16x2);
+                    const bf16x2 hi = __builtin_convertvector(
+                        f32x2{o[db][qb][ii * 4 + 2] * inv, o[db][qb][ii * 4 + 3] * inv}, bf16x2);
+                    u32x2 w;
+                    w.x = __builtin_bit_cast(uint32_t, lo);
+                    w.y = __builtin_bit_cast(uint32_t, hi);
+                    *reinterpret_cast<u32x2*>(op + db * 32 + ii * 8) = w;
+                }
+        }
+    }
+
+    DFX_D float* slot_ptr(int slot) const { return a.workspace + static_cast<int64_t>(slot) * S::SLOT_FLOATS; }
+
+    // Unnormalised accumulators, running maxima and row sums of a piece of an item.
+    DFX_D void store_partial(int slot, const float (&l_tot)[NB]) const {
+        float* sp = slot_ptr(slot);
+        f32x4* ov = reinterpret_cast<f32x4*>(sp);
+#pragma unroll
+        for (int qb = 0; qb < NB; ++qb)
+#pragma unroll
+            for (int db = 0; db < S::NDB; ++db)
+#pragma unroll
+                for (int ii = 0; ii < 4; ++ii)
+                    ov[((qb * S::NDB + db) * 4 + ii) * kThreads + tid] =
+                        f32x4{o[db][qb][ii * 4 + 0], o[db][qb][ii * 4 + 1], o[db][qb][ii * 4 + 2],
+                              o[db][qb][ii * 4 + 3]};
+        float* ml = sp + S::O_VEC4 * 4 * kThreads;
+#pragma unroll
+        for (int qb = 0; qb < NB; ++qb) {
+            ml[qb * kThreads + tid] = m_run[qb];
+            ml[(NB + qb) * kThreads + tid] = l_tot[qb];
+        }
+    }
+
+    // Merge one stored partial into the running state (l_run holds whole-row sums here).
+    DFX_D void merge_partial(int slot) {
+        const float* sp = slot_ptr(slot);
+        const f32x4* ov = reinterpret_cast<const f32x4*>(sp);
+        const float* ml = sp + S::O_VEC4 * 4 * kThreads;
+#pragma unroll
+        for (int qb = 0; qb < NB; ++qb) {
+            const float mp = ml[qb * kThreads + tid];
+            const float lp = ml[(NB + qb) * kThreads + tid];
+            const float mn = fmaxf(m_run[qb], mp);
+            const float wa = (m_run[qb] == -INFINITY) ? 0.0f : fast_exp2(m_run[qb] - mn);
+            const float wb = (mp == -INFINITY) ? 0.0f : fast_exp2(mp - mn);
+            l_run[qb] = l_run[qb] * wa + lp * wb;
+            m_run[qb] = mn;
+#pragma unroll
+            for (int db = 0; db < S::NDB; ++db)
+#pragma unroll
+                for (int ii = 0; ii < 4; ++ii) {
+                    const f32x4 v = ov[((qb * S::NDB + db) * 4 + ii) * kThreads + tid];
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) o[db][qb][ii * 4 + j] = o[db][qb][ii * 4 + j] * wa + v[j] * wb;
+                }
+        }
+    }
+};
+
+// Exclusive prefix of units(s) into prefix[0..num_seqs]; returns the per-head total.
+template <int RT>
+DFX_D int build_unit_prefix(const KArgs& a, int* prefix, int* scratch) {
+    int carry = 0;
+    for (int base = 0; base < a.num_seqs; base += kThreads) {
+        const int sq = base + threadIdx.x;
+        const int u = sq < a.num_seqs ? load_seq_shape(a, sq, RT).units : 0;
+        int tot;
+        const int incl = block_inclusive_scan(u, scratch, tot);
+        if (sq < a.num_seqs) prefix[sq + 1] = carry + incl;
+        carry += tot;
+    }
+    if (threadIdx.x == 0) prefix[0] = 0;
+    __syncthreads();
+    return carry;
+}
+
+// The sequence whose unit range contains rem (0 <= rem < per-head total).
+DFX_D int locate_sequence(const KArgs& a, const int* prefix, int* scratch, int rem) {
+    for (int sq = threadIdx.x; sq < a.num_seqs; sq += kThreads)
+        if (prefix[sq] <= rem && rem < prefix[sq + 1]) scratch[8] = sq;
+    __syncthreads();
+    const int r = scratch[8];
+    __syncthreads();
+    return r;
+}
+
+}  // namespace dfx

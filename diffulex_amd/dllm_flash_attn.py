@@ -29,7 +29,7 @@ def _workspace(device: torch.device, stream: int, nbytes: int) -> torch.Tensor:
 
 def paged_attention(q, k, v, k_cache, v_cache, scale, *, block_tables, context_lens, cu_seqlens_q,
                     cu_seqlens_new, max_seqlen_q, mask_mode=_lib.DFX_MASK_FULL, diffusion_block_size=32,
-                    k_scale=None, v_scale=None, max_workgroups=0, out=None) -> torch.Tensor:
+                    k_scale=None, v_scale=None, max_workgroups=0, out=None, flags=0) -> torch.Tensor:
     """Marshal tensors into ``dfx_attn_params`` and launch ``dfx_paged_attn`` on the
     current stream.  q: [T, H_q, hd]; k, v: [T_new, H_kv, hd]; caches
     [pages, page, H_kv, hd] or None."""
@@ -78,6 +78,7 @@ def paged_attention(q, k, v, k_cache, v_cache, scale, *, block_tables, context_l
     p.diffusion_block_size = int(diffusion_block_size)
     p.mask_mode = int(mask_mode)
     p.max_workgroups = int(max_workgroups)
+    p.flags = int(flags)
     p.scale = float(scale)
     need = lib.dfx_paged_attn_workspace_bytes(C.byref(p))
     if need < 0:

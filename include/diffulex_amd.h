@@ -43,6 +43,9 @@ typedef enum dfx_mask_mode {
 
 typedef enum dfx_index_type { DFX_INDEX_I32 = 0, DFX_INDEX_I64 = 1 } dfx_index_type;
 
+/* dfx_attn_params.flags */
+#define DFX_ATTN_GENERIC_PATH 1 /* use the generic tile path even where the streaming path applies */
+
 /* ABI version of the loaded library (== DFX_ABI_VERSION it was built with). */
 int dfx_abi_version(void);
 
@@ -159,7 +162,8 @@ typedef struct dfx_attn_params {
     int32_t diffusion_block_size;
     int32_t kv_dtype;            /* dfx_kv_dtype of the caches (k_new/v_new are always bf16) */
     int32_t mask_mode;           /* dfx_mask_mode */
-    int32_t max_workgroups;      /* 0: one per compute unit; >0 caps the persistent grid */
+    int32_t max_workgroups;      /* 0: one per compute unit; >0: exactly this many persistent workgroups */
+    int32_t flags;               /* DFX_ATTN_* bits, 0 by default */
     float scale;
 } dfx_attn_params;
 

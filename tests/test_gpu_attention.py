@@ -16,6 +16,10 @@ pytestmark = pytest.mark.gpu
 HERE = os.path.dirname(os.path.abspath(__file__))
 
 
+GENERIC = _lib.DFX_ATTN_GENERIC_PATH   # force the generic tile path where the streaming path would apply
+PATHS = [0, GENERIC]
+
+
 def _run(wl, max_workgroups=0, **kw):
     args = dict(block_tables=wl.block_tables, context_lens=wl.context_lens, cu_seqlens_q=wl.cu_seqlens_q,
                 cu_seqlens_new=wl.cu_seqlens_q, max_seqlen_q=wl.q_len, mask_mode=wl.mask_mode,
@@ -27,11 +31,12 @@ def _run(wl, max_workgroups=0, **kw):
     return out
 
 
+@pytest.mark.parametrize("flags", PATHS)
 @pytest.mark.parametrize("max_wg", [1, 3, 0])
-def test_c1_against_oracle_and_golden(dev, max_wg):
+def test_c1_against_oracle_and_golden(dev, max_wg, flags):
     wl = make_workload("c1")
     want = oracle_fp32(wl)
-    got = _run(wl.to(dev), max_wg)
+    got = _run(wl.to(dev), max_wg, flags=flags)
     assert max_abs_err(got, want) <= ATOL_BF16
     fx = np.load(os.path.join(HERE, "golden", "c1_attention.npz"))
     assert np.array_equal(fx["q_bits"], wl.q.view(torch.int16).numpy()), "seeded inputs differ from the fixture"
@@ -49,12 +54,13 @@ REF_CASES = [
 ]
 
 
+@pytest.mark.parametrize("flags", PATHS)
 @pytest.mark.parametrize("case", REF_CASES)
 @pytest.mark.parametrize("max_wg", [2, 0])
-def test_reference_test_shapes(dev, case, max_wg):
+def test_reference_test_shapes(dev, case, max_wg, flags):
     wl = make_workload("c1", seed=17, **case)
     want = oracle_fp32(wl)
-    got = _run(wl.to(dev), max_wg)
+    got = _run(wl.to(dev), max_wg, flags=flags)
     assert max_abs_err(got, want) <= ATOL_BF16
 
 
@@ -70,13 +76,14 @@ EDGE_CASES = [
 ]
 
 
+@pytest.mark.parametrize("flags", PATHS)
 @pytest.mark.parametrize("case", EDGE_CASES)
 @pytest.mark.parametrize("mask", [MASK_FULL, MASK_BLOCK_CAUSAL])
 @pytest.mark.parametrize("max_wg", [1, 5, 0])
-def test_edge_cases(dev, case, mask, max_wg):
+def test_edge_cases(dev, case, mask, max_wg, flags):
     wl = make_workload("c1", seed=23, mask=mask, **case)
     want = oracle_fp32(wl)
-    got = _run(wl.to(dev), max_wg)
+    got = _run(wl.to(dev), max_wg, flags=flags)
     assert max_abs_err(got, want) <= ATOL_BF16
 
 
@@ -89,9 +96,10 @@ def test_ragged_query_lengths_and_empty_sequences(dev):
     wl.cu_seqlens_q = cu
     want = oracle_fp32(wl)
     g = wl.to(dev)
-    for max_wg in (1, 7, 0):
-        got = _run(g, max_wg, max_seqlen_q=96)
-        assert max_abs_err(got, want) <= ATOL_BF16
+    for flags in PATHS:
+        for max_wg in (1, 7, 0):
+            got = _run(g, max_wg, max_seqlen_q=96, flags=flags)
+            assert max_abs_err(got, want) <= ATOL_BF16
 
 
 @pytest.mark.parametrize("over", [
@@ -106,10 +114,11 @@ def test_fp8_kv_against_oracle(dev, over):
         assert max_abs_err(got, want) <= ATOL_FP8
 
 
-def test_d2f_block_causal_small_c4(dev):
+@pytest.mark.parametrize("flags", PATHS)
+def test_d2f_block_causal_small_c4(dev, flags):
     wl = make_workload("c4", num_seqs=3, ctx=(100, 700))
     want = oracle_fp32(wl)
-    got = _run(wl.to(dev))
+    got = _run(wl.to(dev), flags=flags)
     assert max_abs_err(got, want) <= ATOL_BF16
     # with every fresh token visible (the reference's current D2F behaviour) the result differs
     full = _run(wl.to(dev), mask_mode=MASK_FULL)
@@ -193,9 +202,11 @@ def test_invariants_at_full_c3_size(dev):
         wl.q, wl.k_new, wl.v_new, kc2, vc2, wl.scale, block_tables=bt2, context_lens=wl.context_lens,
         cu_seqlens_q=wl.cu_seqlens_q, cu_seqlens_new=wl.cu_seqlens_q, max_seqlen_q=wl.q_len)
     assert torch.equal(out2, out)
-    # the partition does not change the result beyond rounding
+    # neither the partition nor the tile path changes the result beyond rounding
     out3 = _run(wl, max_workgroups=97)
     assert max_abs_err(out3, out) <= 1e-2
+    out4 = _run(wl, flags=GENERIC)
+    assert max_abs_err(out4, out) <= 1e-2
 
 
 def test_full_size_c4_and_c5_on_sampled_sequences(dev):

@@ -20,6 +20,10 @@ constexpr int kThreads = 256;
 constexpr int kWaves = 4;
 constexpr int kMaxSeqs = 4095;
 constexpr float kLog2e = 1.4426950408889634f;
+// The running row maximum is only raised (and the accumulators rescaled) when a tile exceeds it
+// by more than this many powers of two; until then probabilities up to 2^8 are accumulated
+// against the stale maximum, which fp32 accumulators and bf16 probabilities hold without loss.
+constexpr float kRescaleThreshold = 8.0f;
 
 struct KArgs {
     const uint16_t* q;
@@ -173,8 +177,11 @@ struct AttnState {
 
     // Mask, online softmax and bf16 rounding of one tile's S^T; updates m_run, l_run and
     // rescales o when a row maximum grows.  pb[qb][tb][sl] is the B operand of the PV product.
-    template <bool SCALE_P>
-    DFX_D void softmax_tile(f32x16 (&sc)[2][NB], const TileInfo& t, bf16x8 (&pb)[NB][2][2]) {
+    // before_rescale() runs ahead of any vector-ALU access to o (kernels that issue their matrix
+    // instructions behind the compiler's back insert the required wait states there).
+    template <bool SCALE_P, typename BeforeRescale>
+    DFX_D void softmax_tile(f32x16 (&sc)[2][NB], const TileInfo& t, bf16x8 (&pb)[NB][2][2],
+                            BeforeRescale&& before_rescale) {
         const bool mask_valid = t.base + S::TN > t.limit;
         const bool mask_bc = !t.is_ctx && a.mask_mode == DFX_MASK_BLOCK_CAUSAL;
         if (mask_valid || mask_bc) {
@@ -199,8 +206,10 @@ struct AttnState {
 #pragma unroll
                 for (int e = 0; e < 16; ++e) mx = fmaxf(mx, sc[tb][qb][e]);
             mx = wave_xor32_max(mx);
-            const float m_new = fmaxf(m_run[qb], mx * t.c_tile);
-            if (__any(m_new > m_run[qb])) {
+            const float m_tile = mx * t.c_tile;
+            if (__any(m_tile > m_run[qb] + kRescaleThreshold)) {
+                before_rescale();
+                const float m_new = fmaxf(m_run[qb], m_tile);
                 const float alpha = (m_new == -INFINITY) ? 1.0f : fast_exp2(m_run[qb] - m_new);
                 l_run[qb] *= alpha;
 #pragma unroll

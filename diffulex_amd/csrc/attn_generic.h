@@ -208,7 +208,7 @@ struct GenericAttn : AttnState<HD, NB> {
         }
 
         bf16x8 pb[NB][2][2];
-        this->template softmax_tile<FP8>(sc, t, pb);
+        this->template softmax_tile<FP8>(sc, t, pb, [] {});
 
         const uint8_t* vrow = vs + col * C::VSTRIDE + half * 16;
 #pragma unroll

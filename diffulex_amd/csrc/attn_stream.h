@@ -6,6 +6,12 @@
 // range: tiles of the next (sequence, head) item are already on their way while the current
 // item is finished.
 //
+// Everything data dependent about a unit (which sequence / head / tile it is, where its rows
+// start in memory, whether it opens or closes an item) is worked out ahead of time by all 256
+// lanes in parallel and kept in a small LDS table, kPlanUnits units at a time.  The tile loop
+// itself reads that table and issues nothing to memory but the asynchronous tile loads, so
+// their in-order completion counter can be waited on exactly.
+//
 // LDS tile layout: row-major [token][head_dim] as in the cache, with the 16-byte chunks of a
 // row XOR-swizzled by the row index.  A direct-to-LDS load writes lane i's 16 bytes at
 // wave_base + 16*i, so the swizzle is applied on the global side: lane i fetches the chunk
@@ -27,6 +33,21 @@
 
 namespace dfx {
 
+// One unit of the plan: wave-uniform facts (UnitDesc) and the start of each wave's 16-row
+// band of the tile in memory (BandDesc).
+struct UnitDesc {
+    int32_t s, kvh, rt, q0;
+    int32_t q_len, base, limit, flags;
+    int32_t slot, run, pad1, pad2;  // run: units from this one to the end of this workgroup's piece of the item
+};
+static_assert(sizeof(UnitDesc) == 48, "UnitDesc is read as three 16-byte LDS words");
+struct BandDesc {
+    int64_t off;   // byte offset of the band's first row from the K (== from the V) base pointer
+    int32_t last;  // last valid row of the band; later rows re-read it
+    int32_t is_ctx;
+};
+enum : int32_t { kUnitCtx = 1, kUnitFirst = 2, kUnitLast = 4, kUnitComplete = 8 };
+
 template <int HD, int NB>
 struct StreamCfg : Shape<HD, NB> {
     using S = Shape<HD, NB>;
@@ -39,21 +60,27 @@ struct StreamCfg : Shape<HD, NB> {
     static constexpr int IPW = MAT_BYTES / 1024 / kWaves;  // loads per wave per matrix per tile
     static constexpr int LOADS_PER_UNIT = 2 * IPW;
     static constexpr int ROWS_PER_WAVE = IPW * RPI;        // 16
-    static constexpr int LDS_BYTES = S::PREFIX_BYTES + S::MISC_BYTES + kStages * STAGE_BYTES;
+    static constexpr int kPlanUnits = 128;                 // units planned (and then streamed) at a time
+    static constexpr int UNIT_TABLE_BYTES = kPlanUnits * static_cast<int>(sizeof(UnitDesc));
+    static constexpr int BAND_TABLE_BYTES = kPlanUnits * kWaves * static_cast<int>(sizeof(BandDesc));
+    static constexpr int UNIT_TABLE_OFF = S::PREFIX_BYTES + S::MISC_BYTES;
+    static constexpr int BAND_TABLE_OFF = UNIT_TABLE_OFF + UNIT_TABLE_BYTES;
+    static constexpr int STAGES_OFF = BAND_TABLE_OFF + BAND_TABLE_BYTES;
+    static constexpr int LDS_BYTES = STAGES_OFF + kStages * STAGE_BYTES;
     static_assert(ROWS_PER_WAVE == 16, "a wave loads a 16-row band of each tile");
+    static_assert(LDS_BYTES <= 160 * 1024, "LDS budget of a gfx950 compute unit");
 
     // chunk position = chunk index ^ swizzle(row); 16 consecutive rows of one chunk column hit
     // 16 different 16-byte bank groups (the LDS has 64 banks)
     DFX_HD static int swizzle(int row) { return HD == 128 ? (row & 15) : ((row >> 1) & 7); }
 };
 
-DFX_D uint32_t lds_offset(const void* p) { return static_cast<uint32_t>(reinterpret_cast<uintptr_t>(p)); }
-
-// One wave-wide 16-byte-per-lane direct-to-LDS load; lane i's data lands at lds_wave_base + 16*i.
-DFX_D void async_load16(const void* gptr, uint32_t lds_wave_base) {
-    asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off nt"
+// One wave-wide 16-byte-per-lane direct-to-LDS load from base + voff; lane i's data lands at
+// lds_wave_base + 16*i.  base and lds_wave_base must be wave-uniform.
+DFX_D void async_load16(const void* base, uint32_t voff, uint32_t lds_wave_base) {
+    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1 nt"
                  :
-                 : "v"(gptr), "s"(__builtin_amdgcn_readfirstlane(lds_wave_base))
+                 : "v"(voff), "s"(base), "s"(__builtin_amdgcn_readfirstlane(lds_wave_base))
                  : "memory", "m0");
 }
 
@@ -62,13 +89,35 @@ DFX_D void wait_async_loads() {
     asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
 }
 
-// Position in the workgroup's unit range, with the shape of the sequence it is in.
-struct UnitCursor {
-    int64_t pos;
-    int kvh, s, u;
-    SeqShape sh;
-    int n0;
-};
+DFX_D int uniform(int v) { return __builtin_amdgcn_readfirstlane(v); }
+
+// The matrix instructions of the tile loop are issued from inline assembly so that the register
+// file split is fixed by their operand constraints: the O^T accumulators live in the accumulation
+// registers, which only matrix instructions touch in the loop, and the score accumulators in
+// ordinary vector registers, where the softmax works on them in place.  Being volatile they keep
+// their program order: an accumulator is reused every 4th (scores) or 8th (output) instruction,
+// far beyond the result latency.  What the compiler can no longer do for them is insert the wait
+// states the ISA requires around matrix instructions: each one is therefore preceded by two wait
+// states (a vector-ALU result may feed it), and mfma_results_ready() / mfma_outputs_ready() put
+// 18 wait states, the longest the ISA asks for, between a matrix result and a vector-ALU reader.
+DFX_D void mfma_scores_first(f32x16& sc, bf16x8 k, bf16x8 q) {
+    asm volatile("s_nop 1\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(sc) : "v"(k), "v"(q));
+}
+DFX_D void mfma_scores(f32x16& sc, bf16x8 k, bf16x8 q) {
+    asm volatile("s_nop 1\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(sc) : "v"(k), "v"(q));
+}
+DFX_D void mfma_output(f32x16& acc, bf16x8 v, bf16x8 p) {
+    asm volatile("s_nop 1\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(acc) : "v"(v), "v"(p));
+}
+DFX_D void mfma_results_ready(f32x16& x0, f32x16& x1, f32x16& x2, f32x16& x3) {
+    asm volatile("s_nop 15\n\ts_nop 1" : "+v"(x0), "+v"(x1), "+v"(x2), "+v"(x3));
+}
+DFX_D void mfma_results_ready(f32x16& x0, f32x16& x1) {
+    asm volatile("s_nop 15\n\ts_nop 1" : "+v"(x0), "+v"(x1));
+}
+DFX_D void mfma_outputs_ready(f32x16& x0, f32x16& x1, f32x16& x2, f32x16& x3) {
+    asm volatile("s_nop 15\n\ts_nop 1" : "+a"(x0), "+a"(x1), "+a"(x2), "+a"(x3));
+}
 
 template <int HD, int NB>
 struct StreamAttn : AttnState<HD, NB> {
@@ -80,89 +129,123 @@ struct StreamAttn : AttnState<HD, NB> {
     using Base::lane;
     using Base::o;
     using Base::qf;
+    using Base::tid;
     using Base::wave;
 
     uint8_t* lds;
     int* prefix;
     int* misc;
-    uint32_t stage0;  // LDS byte offset of stage 0
+    UnitDesc* units;
+    BandDesc* bands;
+    uint32_t stages_lds;  // LDS byte address of stage 0
+    int64_t begin, end;
+    int per_head;
 
     DFX_D StreamAttn(const KArgs& args, uint8_t* smem)
         : Base(args), lds(smem), prefix(reinterpret_cast<int*>(smem)),
           misc(reinterpret_cast<int*>(smem + C::PREFIX_BYTES)),
-          stage0(lds_offset(smem) + C::PREFIX_BYTES + C::MISC_BYTES) {}
+          units(reinterpret_cast<UnitDesc*>(smem + C::UNIT_TABLE_OFF)),
+          bands(reinterpret_cast<BandDesc*>(smem + C::BAND_TABLE_OFF)),
+          stages_lds(static_cast<uint32_t>(reinterpret_cast<uintptr_t>(smem)) + C::STAGES_OFF) {}
 
-    DFX_D void cursor_enter(UnitCursor& c) const {
-        c.sh = load_seq_shape(a, c.s, C::RT);
-        c.n0 = a.cu_new[c.s];
-    }
-
-    DFX_D void cursor_advance(UnitCursor& c, int64_t end) const {
-        ++c.pos;
-        ++c.u;
-        if (c.pos >= end) return;
-        if (c.u == c.sh.units) {
-            c.u = 0;
-            do {
-                if (++c.s == a.num_seqs) {
-                    c.s = 0;
-                    ++c.kvh;
-                }
-            } while (prefix[c.s + 1] == prefix[c.s]);
-            cursor_enter(c);
+    // ---- planning --------------------------------------------------------------------------
+    // Describe units [first, first + count) in the plan table (entry i is unit first + i); one
+    // lane per (unit, wave).
+    DFX_D void plan_units(int64_t first, int count) const {
+        for (int idx = tid; idx < count * kWaves; idx += kThreads) {
+            const int64_t pos = first + (idx >> 2);
+            const int w = idx & 3;
+            const int slot_in_ring = idx >> 2;
+            const int kv_head = static_cast<int>(pos / per_head);
+            const int rem = static_cast<int>(pos - static_cast<int64_t>(kv_head) * per_head);
+            int lo = 0, hi = a.num_seqs;  // the sequence with prefix[s] <= rem < prefix[s + 1]
+            while (lo < hi) {
+                const int mid = (lo + hi) >> 1;
+                if (prefix[mid + 1] <= rem) lo = mid + 1;
+                else hi = mid;
+            }
+            const int sq = lo;
+            const SeqShape shp = load_seq_shape(a, sq, C::RT);
+            const int u = rem - prefix[sq];
+            const int rt = u / shp.n_tiles;
+            const int tile = u - rt * shp.n_tiles;
+            const bool is_ctx = tile < shp.n_ctx_tiles;
+            const int base = (is_ctx ? tile : tile - shp.n_ctx_tiles) * C::TN;
+            const int limit = is_ctx ? shp.ctx : shp.new_len;
+            // the piece of the item this workgroup owns
+            const int64_t before = pos - begin, after = end - pos;
+            const int tile0 = before >= tile ? 0 : tile - static_cast<int>(before);
+            const int tile1 = after >= shp.n_tiles - tile ? shp.n_tiles : tile + static_cast<int>(after);
+            if (w == 0) {
+                UnitDesc d;
+                d.s = sq;
+                d.kvh = kv_head;
+                d.rt = rt;
+                d.q0 = a.cu_q[sq];
+                d.q_len = shp.q_len;
+                d.base = base;
+                d.limit = limit;
+                d.flags = (is_ctx ? kUnitCtx : 0) | (tile == tile0 ? kUnitFirst : 0) |
+                          (tile == tile1 - 1 ? kUnitLast : 0) |
+                          (tile0 == 0 && tile1 == shp.n_tiles ? kUnitComplete : 0);
+                d.slot = partial_slot(static_cast<int>(blockIdx.x), pos - (tile - tile0), begin);
+                d.run = tile1 - tile;
+                d.pad1 = d.pad2 = 0;
+                units[slot_in_ring] = d;
+            }
+            // Rows past the end re-read the last valid rows (finite data; their scores are masked).
+            int band = base + w * C::ROWS_PER_WAVE;
+            if (band >= limit) band = ((limit - 1) / C::ROWS_PER_WAVE) * C::ROWS_PER_WAVE;
+            BandDesc b;
+            if (is_ctx) {
+                const int p = a.page_shift >= 0 ? (band >> a.page_shift) : (band / a.page_size);
+                int64_t page = p < a.max_pages ? a.block_tables[static_cast<int64_t>(sq) * a.bt_stride + p] : 0;
+                page = page < 0 ? 0 : (page >= a.n_pages ? a.n_pages - 1 : page);
+                b.off = (page * a.c_sp + static_cast<int64_t>(band - p * a.page_size) * a.c_st + kv_head * a.c_sh) * 2;
+            } else {
+                b.off = ((static_cast<int64_t>(a.cu_new[sq]) + band) * a.kn_st + kv_head * a.kn_sh) * 2;
+            }
+            b.last = limit - 1 - band;
+            b.is_ctx = is_ctx ? 1 : 0;
+            bands[slot_in_ring * kWaves + w] = b;
         }
     }
 
-    // Start the loads of the unit at c into ring stage `stage` (this wave's 16-row band of K and V).
-    DFX_D void issue_unit(const UnitCursor& c, int stage) const {
-        const int tile = c.u % c.sh.n_tiles;
-        const bool is_ctx = tile < c.sh.n_ctx_tiles;
-        const int base = (is_ctx ? tile : tile - c.sh.n_ctx_tiles) * C::TN;
-        const int limit = is_ctx ? c.sh.ctx : c.sh.new_len;
-        // Rows past the end re-read the last valid rows (finite data; their scores are masked).
-        int band = base + wave * C::ROWS_PER_WAVE;
-        if (band >= limit) band = ((limit - 1) / C::ROWS_PER_WAVE) * C::ROWS_PER_WAVE;
-        const uint8_t* kbase;
-        const uint8_t* vbase;
-        int64_t row_stride;  // bytes
-        if (is_ctx) {
-            const int p = a.page_shift >= 0 ? (band >> a.page_shift) : (band / a.page_size);
-            int64_t page = a.block_tables[static_cast<int64_t>(c.s) * a.bt_stride + p];
-            page = page < 0 ? 0 : (page >= a.n_pages ? a.n_pages - 1 : page);
-            const int64_t off = (page * a.c_sp + static_cast<int64_t>(band - p * a.page_size) * a.c_st + c.kvh * a.c_sh) * 2;
-            kbase = a.k_cache + off;
-            vbase = a.v_cache + off;
-            row_stride = a.c_st * 2;
-        } else {
-            const int64_t t = c.n0 + band;
-            kbase = reinterpret_cast<const uint8_t*>(a.k_new + t * a.kn_st + c.kvh * a.kn_sh);
-            vbase = reinterpret_cast<const uint8_t*>(a.v_new + t * a.vn_st + c.kvh * a.vn_sh);
-            row_stride = a.kn_st * 2;
-        }
-        const int64_t v_row_stride = is_ctx ? row_stride : a.vn_st * 2;
-        const int last = limit - 1 - band;  // last valid row of the band (>= 0)
-        const uint32_t dst = stage0 + stage * C::STAGE_BYTES + wave * (C::IPW * 1024);
+    // ---- loads -----------------------------------------------------------------------------
+    // Start the loads of planned unit `rel` (this wave's 16-row band of K and V) into its ring stage.
+    DFX_D void issue_unit(int rel) const {
+        const BandDesc b = bands[rel * kWaves + wave];
+        const int last = uniform(b.last);
+        const bool is_ctx = uniform(b.is_ctx) != 0;
+        const int64_t off = (static_cast<int64_t>(uniform(static_cast<int>(b.off >> 32))) << 32) |
+                            static_cast<uint32_t>(uniform(static_cast<int>(b.off)));
+        const uint8_t* kbase = (is_ctx ? a.k_cache : reinterpret_cast<const uint8_t*>(a.k_new)) + off;
+        const uint8_t* vbase = (is_ctx ? a.v_cache : reinterpret_cast<const uint8_t*>(a.v_new)) + off;
+        const uint32_t row_stride = static_cast<uint32_t>(is_ctx ? a.c_st : a.kn_st) * 2u;
+        const uint32_t dst = stages_lds + (rel % C::kStages) * C::STAGE_BYTES + wave * (C::IPW * 1024);
 #pragma unroll
         for (int j = 0; j < C::IPW; ++j) {
-            int r = j * C::RPI + lane / C::CPR;          // row inside the band
+            const int r = j * C::RPI + lane / C::CPR;  // row inside the band
             const int lds_row = wave * C::ROWS_PER_WAVE + r;
             const int chunk = (lane % C::CPR) ^ C::swizzle(lds_row);
-            r = min(r, last);
-            async_load16(kbase + r * row_stride + chunk * 16, dst + j * 1024);
-            async_load16(vbase + r * v_row_stride + chunk * 16, dst + C::MAT_BYTES + j * 1024);
+            const uint32_t voff = static_cast<uint32_t>(min(r, last)) * row_stride + chunk * 16;
+            async_load16(kbase, voff, dst + j * 1024);
+            async_load16(vbase, voff, dst + C::MAT_BYTES + j * 1024);
         }
     }
 
-    DFX_D bf16x8 read_k(uint32_t k_lds, int tb, int slab) const {
+    // ---- tile arithmetic -------------------------------------------------------------------
+    DFX_D bf16x8 read_k(const uint8_t* k_tile, int tb, int slab) const {
         const int row = tb * 32 + col;
         const int pos = (2 * slab + half) ^ C::swizzle(row);
-        return *reinterpret_cast<const bf16x8*>(lds + (k_lds - lds_offset(lds)) + row * C::ROWB + pos * 16);
+        return *reinterpret_cast<const bf16x8*>(k_tile + row * C::ROWB + pos * 16);
     }
 
     // V^T operand for token slab (tb, sl) and d block db.
-    DFX_D bf16x8 read_vt(uint32_t v_lds, int tb, int sl, int db) const {
+    DFX_D bf16x8 read_vt(const uint8_t* v_tile, int tb, int sl, int db) const {
         typedef short short4v __attribute__((ext_vector_type(4)));
         typedef short short8v __attribute__((ext_vector_type(8)));
+        typedef __attribute__((address_space(3))) short4v lds_short4v;
         const int g16 = lane >> 4, sl16 = lane & 15;
         short4v r[2];
 #pragma unroll
@@ -170,51 +253,69 @@ struct StreamAttn : AttnState<HD, NB> {
             const int row = tb * 32 + sl * 16 + ii * 8 + (g16 >> 1) * 4 + (sl16 >> 2);
             const int chunk = db * 4 + (g16 & 1) * 2 + ((sl16 & 3) >> 1);
             const int pos = chunk ^ C::swizzle(row);
-            const uint8_t* p = lds + (v_lds - lds_offset(lds)) + row * C::ROWB + pos * 16 + (sl16 & 1) * 8;
-            r[ii] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                reinterpret_cast<short4v __attribute__((address_space(3)))*>(
-                    reinterpret_cast<uintptr_t>(p)));
+            const uint8_t* p = v_tile + row * C::ROWB + pos * 16 + (sl16 & 1) * 8;
+            r[ii] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4v*)(p));
         }
         const short8v v = __builtin_shufflevector(r[0], r[1], 0, 1, 2, 3, 4, 5, 6, 7);
         return __builtin_bit_cast(bf16x8, v);
     }
 
-    DFX_D void compute(int stage, const TileInfo& t) {
-        const uint32_t k_lds = stage0 + stage * C::STAGE_BYTES;
-        const uint32_t v_lds = k_lds + C::MAT_BYTES;
-        f32x16 sc[2][NB];
-#pragma unroll
-        for (int tb = 0; tb < 2; ++tb)
-#pragma unroll
-            for (int qb = 0; qb < NB; ++qb)
-#pragma unroll
-                for (int e = 0; e < 16; ++e) sc[tb][qb][e] = 0.0f;
+    DFX_D void scores(const uint8_t* k_tile, f32x16 (&sc)[2][NB]) const {
 #pragma unroll
         for (int slab = 0; slab < C::NSLAB; ++slab) {
             bf16x8 ka[2];
 #pragma unroll
-            for (int tb = 0; tb < 2; ++tb) ka[tb] = read_k(k_lds, tb, slab);
+            for (int tb = 0; tb < 2; ++tb) ka[tb] = read_k(k_tile, tb, slab);
 #pragma unroll
             for (int tb = 0; tb < 2; ++tb)
 #pragma unroll
-                for (int qb = 0; qb < NB; ++qb)
-                    sc[tb][qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[tb], qf[qb][slab], sc[tb][qb], 0, 0, 0);
-            __builtin_amdgcn_sched_barrier(0);
+                for (int qb = 0; qb < NB; ++qb) {
+                    if (slab == 0) mfma_scores_first(sc[tb][qb], ka[tb], qf[qb][slab]);
+                    else mfma_scores(sc[tb][qb], ka[tb], qf[qb][slab]);
+                }
         }
-        bf16x8 pb[NB][2][2];
-        this->template softmax_tile<false>(sc, t, pb);
+        if constexpr (NB == 2) mfma_results_ready(sc[0][0], sc[0][1], sc[1][0], sc[1][1]);
+        else mfma_results_ready(sc[0][0], sc[1][0]);
+    }
+
+    // Wait states before vector instructions read the O^T accumulators (rescale, epilogue).
+    DFX_D void outputs_ready() {
+#pragma unroll
+        for (int qb = 0; qb < NB; ++qb) {
+            if constexpr (C::NDB == 4) mfma_outputs_ready(o[0][qb], o[1][qb], o[2][qb], o[3][qb]);
+            else mfma_outputs_ready(o[0][qb], o[1][qb], o[0][qb], o[1][qb]);
+        }
+    }
+
+    DFX_D void accumulate(const uint8_t* v_tile, const bf16x8 (&pb)[NB][2][2]) {
 #pragma unroll
         for (int tb = 0; tb < 2; ++tb)
 #pragma unroll
             for (int sl = 0; sl < 2; ++sl)
 #pragma unroll
                 for (int db = 0; db < C::NDB; ++db) {
-                    const bf16x8 va = read_vt(v_lds, tb, sl, db);
+                    const bf16x8 va = read_vt(v_tile, tb, sl, db);
 #pragma unroll
-                    for (int qb = 0; qb < NB; ++qb)
-                        o[db][qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, pb[qb][tb][sl], o[db][qb], 0, 0, 0);
-                    __builtin_amdgcn_sched_barrier(0);
+                    for (int qb = 0; qb < NB; ++qb) mfma_output(o[db][qb], va, pb[qb][tb][sl]);
                 }
+    }
+
+    // Make the compiler wait for the query loads here (before more asynchronous loads are queued
+    // behind them, which its own wait would otherwise have to drain as well).
+    DFX_D void touch_queries() const {
+#pragma unroll
+        for (int qb = 0; qb < NB; ++qb)
+#pragma unroll
+            for (int slab = 0; slab < C::NSLAB; ++slab) asm volatile("" : : "v"(qf[qb][slab]));
+    }
+
+    // Adopt the item of unit d as the current one and fetch its query rows.
+    DFX_D void begin_item(const UnitDesc& d) {
+        this->s = uniform(d.s);
+        this->kvh = uniform(d.kvh);
+        this->q0 = uniform(d.q0);
+        this->sh.q_len = uniform(d.q_len);
+        this->load_queries(uniform(d.rt));
     }
 };
 
@@ -223,67 +324,69 @@ __global__ void __launch_bounds__(kThreads) paged_attn_stream_kernel(const KArgs
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     using C = StreamCfg<HD, NB>;
     StreamAttn<HD, NB> at(a, smem);
-    const int per_head = build_unit_prefix<C::RT>(a, at.prefix, at.misc);
-    const int64_t total = static_cast<int64_t>(per_head) * a.h_kv;
+    at.per_head = build_unit_prefix<C::RT>(a, at.prefix, at.misc);
+    const int64_t total = static_cast<int64_t>(at.per_head) * a.h_kv;
     if (total == 0) return;
     const int w = blockIdx.x;
-    const int64_t begin = wg_first_unit(w, total, a.n_wg);
-    const int64_t end = wg_first_unit(w + 1, total, a.n_wg);
-    if (begin >= end) return;
+    at.begin = wg_first_unit(w, total, a.n_wg);
+    at.end = wg_first_unit(w + 1, total, a.n_wg);
+    if (at.begin >= at.end) return;
+    const int64_t begin = at.begin, end = at.end;
 
-    UnitCursor ld;
-    ld.pos = begin;
-    ld.kvh = static_cast<int>(begin / per_head);
-    const int rem = static_cast<int>(begin - static_cast<int64_t>(ld.kvh) * per_head);
-    ld.s = locate_sequence(a, at.prefix, at.misc, rem);
-    ld.u = rem - at.prefix[ld.s];
-    at.cursor_enter(ld);
-    UnitCursor cp = ld;
+    for (int64_t chunk = begin; chunk < end; chunk += C::kPlanUnits) {
+        const int n_units = static_cast<int>(min(static_cast<int64_t>(C::kPlanUnits), end - chunk));
+        __syncthreads();  // every wave is done with the previous plan and its stages
+        at.plan_units(chunk, n_units);
+        __syncthreads();
 
-    // fill the ring: kStages - 1 units in flight
-    int64_t issued = begin;
-    for (int i = 0; i < C::kStages - 1 && ld.pos < end; ++i) {
-        at.issue_unit(ld, static_cast<int>((issued - begin) % C::kStages));
-        at.cursor_advance(ld, end);
-        ++issued;
-    }
+        int issued = 0;  // ring fill: kStages - 1 units in flight
+        for (; issued < C::kStages - 1 && issued < n_units; ++issued) at.issue_unit(issued);
 
-    while (cp.pos < end) {
-        // one segment: units of the same (sequence, head, row tile)
-        at.s = cp.s;
-        at.kvh = cp.kvh;
-        at.sh = cp.sh;
-        at.q0 = a.cu_q[cp.s];
-        at.n0 = cp.n0;
-        const int n_tiles = cp.sh.n_tiles;
-        const int rt = cp.u / n_tiles;
-        const int tile0 = cp.u - rt * n_tiles;
-        const int64_t seg_begin = cp.pos;
-        const int64_t seg_end = min(cp.pos + (n_tiles - tile0), end);
-        const int tile1 = tile0 + static_cast<int>(seg_end - cp.pos);
-        at.load_queries(rt);
-        for (int tile = tile0; tile < tile1; ++tile) {
-            // the unit at cp.pos must have landed: allow only the younger ones to be outstanding
-            const int younger = static_cast<int>(issued - cp.pos) - 1;
-            if (younger >= 2) wait_async_loads<2 * C::LOADS_PER_UNIT>();
-            else if (younger == 1) wait_async_loads<C::LOADS_PER_UNIT>();
-            else wait_async_loads<0>();
-            __builtin_amdgcn_s_barrier();
-            // every wave has finished the previous unit: its stage may be overwritten
-            if (ld.pos < end) {
-                at.issue_unit(ld, static_cast<int>((issued - begin) % C::kStages));
-                at.cursor_advance(ld, end);
-                ++issued;
+        int rel = 0;
+        while (rel < n_units) {
+            // a run of units of one item: all of this workgroup's piece of it, or up to the end of the plan
+            const UnitDesc d = at.units[rel];
+            const int flags = uniform(d.flags);
+            const int run_end = min(rel + uniform(d.run), n_units);
+            if (flags & kUnitFirst) at.begin_item(d);
+            bool queries_pending = (flags & kUnitFirst) != 0;
+            for (; rel < run_end; ++rel) {
+                // the unit must have landed: only younger units may still be outstanding
+                const int younger = issued - rel - 1;
+                if (younger >= 2) wait_async_loads<2 * C::LOADS_PER_UNIT>();
+                else if (younger == 1) wait_async_loads<C::LOADS_PER_UNIT>();
+                else wait_async_loads<0>();
+                __builtin_amdgcn_s_barrier();
+                // every wave has finished the previous unit: its stage may be overwritten
+                if (queries_pending) {
+                    at.touch_queries();
+                    queries_pending = false;
+                }
+                if (issued < n_units) at.issue_unit(issued++);
+
+                const UnitDesc u = at.units[rel];
+                TileInfo t;
+                t.base = uniform(u.base);
+                t.limit = uniform(u.limit);
+                t.is_ctx = (uniform(u.flags) & kUnitCtx) != 0;
+                t.c_tile = a.c;
+                t.v_mul = 1.0f;
+                const uint8_t* k_tile = smem + C::STAGES_OFF + (rel % C::kStages) * C::STAGE_BYTES;
+                f32x16 sc[2][NB];
+                at.scores(k_tile, sc);
+                bf16x8 pb[NB][2][2];
+                at.template softmax_tile<false>(sc, t, pb, [&] { at.outputs_ready(); });
+                at.accumulate(k_tile + C::MAT_BYTES, pb);
             }
-            const TileInfo t = at.tile_info(cp.sh, cp.kvh, tile, false);
-            at.compute(static_cast<int>((cp.pos - begin) % C::kStages), t);
-            at.cursor_advance(cp, end);
+            const UnitDesc e = at.units[rel - 1];
+            if (uniform(e.flags) & kUnitLast) {
+                at.outputs_ready();
+                float l_tot[NB];
+                at.row_sums(l_tot);
+                if (uniform(e.flags) & kUnitComplete) at.store_output(uniform(e.rt), l_tot);
+                else at.store_partial(uniform(e.slot), l_tot);
+            }
         }
-        float l_tot[NB];
-        at.row_sums(l_tot);
-        const bool complete = tile0 == 0 && tile1 == n_tiles;
-        if (complete) at.store_output(rt, l_tot);
-        else at.store_partial(partial_slot(w, seg_begin, begin), l_tot);
     }
 }
 

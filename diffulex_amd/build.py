@@ -35,7 +35,7 @@ def _hipcc() -> str:
 
 
 def _compile(src: Path, obj: Path) -> None:
-    cmd = [_hipcc(), *HIP_FLAGS, "-x", "hip", "-c", str(src), "-o", str(obj)]
+    cmd = [_hipcc(), *HIP_FLAGS, *os.environ.get("DFX_EXTRA_FLAGS", "").split(), "-x", "hip", "-c", str(src), "-o", str(obj)]
     res = subprocess.run(cmd, capture_output=True, text=True)
     # the host pass does not know the packed-fp32 feature name; that warning is expected
     err = "\n".join(l for l in res.stderr.splitlines() if "packed-fp32-ops" not in l)

@@ -16,8 +16,9 @@
 
 namespace dfx {
 
-constexpr int kThreads = 256;
+constexpr int kThreads = 256;  // workgroup size of the 4-wave kernels
 constexpr int kWaves = 4;
+constexpr int kMaxWaves = 8;
 constexpr int kMaxSeqs = 4095;
 constexpr float kLog2e = 1.4426950408889634f;
 // The running row maximum is only raised (and the accumulators rescaled) when a tile exceeds it
@@ -47,16 +48,22 @@ struct KArgs {
 };
 
 // Sizes that do not depend on how a kernel stages its tiles.
-template <int HD, int NB>
+// HD: head_dim; NB: 32-row query blocks per wave; NW: waves per workgroup.
+template <int HD, int NB, int NW = kWaves>
 struct Shape {
     static constexpr int TN = kTileTokens;
-    static constexpr int RT = 32 * NB * kWaves;  // query rows per row tile
+    static constexpr int THREADS = 64 * NW;
+    static constexpr int RT = 32 * NB * NW;      // query rows per row tile
     static constexpr int NSLAB = HD / 16;        // contraction slabs of Q K^T
     static constexpr int NDB = HD / 32;          // 32-row blocks of O^T
     static constexpr int PREFIX_BYTES = (kMaxSeqs + 1) * 4;
     static constexpr int MISC_BYTES = 64;
-    static constexpr int O_VEC4 = NB * NDB * 4;  // float4 per lane in a partial result
-    static constexpr int SLOT_FLOATS = kThreads * (O_VEC4 * 4 + 2 * NB);
+    // A partial result is stored per 32-row query block b = wave * NB + qb, whatever the shape of
+    // the workgroup that wrote it: NDB * 4 float4 per lane of O^T, then the running maximum and
+    // the row sum of the lane's query.
+    static constexpr int BLOCKS = NB * NW;
+    static constexpr int BLOCK_FLOATS = 64 * (NDB * 16 + 2);
+    static constexpr int SLOT_FLOATS = BLOCKS * BLOCK_FLOATS;
 };
 
 DFX_D float wave_xor32_max(float x) { return fmaxf(x, __shfl_xor(x, 32)); }
@@ -74,11 +81,14 @@ DFX_D int block_inclusive_scan(int v, int* scratch, int& block_total) {
     if (lane == 63) scratch[wave] = x;
     __syncthreads();
     int off = 0, tot = 0;
+    const int n_waves = blockDim.x >> 6;
 #pragma unroll
-    for (int w = 0; w < kWaves; ++w) {
-        const int t = scratch[w];
-        if (w < wave) off += t;
-        tot += t;
+    for (int w = 0; w < kMaxWaves; ++w) {
+        if (w < n_waves) {
+            const int t = scratch[w];
+            if (w < wave) off += t;
+            tot += t;
+        }
     }
     __syncthreads();
     block_total = tot;
@@ -101,9 +111,9 @@ struct TileInfo {
     float v_mul;   // factor applied to P before the PV product (v_scale for FP8 context, else 1)
 };
 
-template <int HD, int NB>
+template <int HD, int NB, int NW = kWaves>
 struct AttnState {
-    using S = Shape<HD, NB>;
+    using S = Shape<HD, NB, NW>;
 
     const KArgs& a;
     const int tid, lane, wave, col, half;
@@ -141,7 +151,7 @@ struct AttnState {
         return t;
     }
 
-    DFX_D int row_of(int rt, int qb) const { return rt * S::RT + wave * (32 * NB) + qb * 32 + col; }
+    DFX_D int row_of(int rt, int qb) const { return rt * S::RT + (wave * NB + qb) * 32 + col; }
 
     DFX_D void reset_accumulators() {
 #pragma unroll
@@ -280,34 +290,31 @@ struct AttnState {
 
     // Unnormalised accumulators, running maxima and row sums of a piece of an item.
     DFX_D void store_partial(int slot, const float (&l_tot)[NB]) const {
-        float* sp = slot_ptr(slot);
-        f32x4* ov = reinterpret_cast<f32x4*>(sp);
 #pragma unroll
-        for (int qb = 0; qb < NB; ++qb)
+        for (int qb = 0; qb < NB; ++qb) {
+            float* bp = slot_ptr(slot) + (wave * NB + qb) * S::BLOCK_FLOATS;
+            f32x4* ov = reinterpret_cast<f32x4*>(bp);
 #pragma unroll
             for (int db = 0; db < S::NDB; ++db)
 #pragma unroll
                 for (int ii = 0; ii < 4; ++ii)
-                    ov[((qb * S::NDB + db) * 4 + ii) * kThreads + tid] =
-                        f32x4{o[db][qb][ii * 4 + 0], o[db][qb][ii * 4 + 1], o[db][qb][ii * 4 + 2],
-                              o[db][qb][ii * 4 + 3]};
-        float* ml = sp + S::O_VEC4 * 4 * kThreads;
-#pragma unroll
-        for (int qb = 0; qb < NB; ++qb) {
-            ml[qb * kThreads + tid] = m_run[qb];
-            ml[(NB + qb) * kThreads + tid] = l_tot[qb];
+                    ov[(db * 4 + ii) * 64 + lane] = f32x4{o[db][qb][ii * 4 + 0], o[db][qb][ii * 4 + 1],
+                                                          o[db][qb][ii * 4 + 2], o[db][qb][ii * 4 + 3]};
+            float* ml = bp + S::NDB * 16 * 64;
+            ml[lane] = m_run[qb];
+            ml[64 + lane] = l_tot[qb];
         }
     }
 
     // Merge one stored partial into the running state (l_run holds whole-row sums here).
     DFX_D void merge_partial(int slot) {
-        const float* sp = slot_ptr(slot);
-        const f32x4* ov = reinterpret_cast<const f32x4*>(sp);
-        const float* ml = sp + S::O_VEC4 * 4 * kThreads;
 #pragma unroll
         for (int qb = 0; qb < NB; ++qb) {
-            const float mp = ml[qb * kThreads + tid];
-            const float lp = ml[(NB + qb) * kThreads + tid];
+            const float* bp = slot_ptr(slot) + (wave * NB + qb) * S::BLOCK_FLOATS;
+            const f32x4* ov = reinterpret_cast<const f32x4*>(bp);
+            const float* ml = bp + S::NDB * 16 * 64;
+            const float mp = ml[lane];
+            const float lp = ml[64 + lane];
             const float mn = fmaxf(m_run[qb], mp);
             const float wa = (m_run[qb] == -INFINITY) ? 0.0f : fast_exp2(m_run[qb] - mn);
             const float wb = (mp == -INFINITY) ? 0.0f : fast_exp2(mp - mn);
@@ -317,7 +324,7 @@ struct AttnState {
             for (int db = 0; db < S::NDB; ++db)
 #pragma unroll
                 for (int ii = 0; ii < 4; ++ii) {
-                    const f32x4 v = ov[((qb * S::NDB + db) * 4 + ii) * kThreads + tid];
+                    const f32x4 v = ov[(db * 4 + ii) * 64 + lane];
 #pragma unroll
                     for (int j = 0; j < 4; ++j) o[db][qb][ii * 4 + j] = o[db][qb][ii * 4 + j] * wa + v[j] * wb;
                 }
@@ -329,7 +336,8 @@ struct AttnState {
 template <int RT>
 DFX_D int build_unit_prefix(const KArgs& a, int* prefix, int* scratch) {
     int carry = 0;
-    for (int base = 0; base < a.num_seqs; base += kThreads) {
+    const int n_threads = blockDim.x;
+    for (int base = 0; base < a.num_seqs; base += n_threads) {
         const int sq = base + threadIdx.x;
         const int u = sq < a.num_seqs ? load_seq_shape(a, sq, RT).units : 0;
         int tot;
@@ -344,10 +352,10 @@ DFX_D int build_unit_prefix(const KArgs& a, int* prefix, int* scratch) {
 
 // The sequence whose unit range contains rem (0 <= rem < per-head total).
 DFX_D int locate_sequence(const KArgs& a, const int* prefix, int* scratch, int rem) {
-    for (int sq = threadIdx.x; sq < a.num_seqs; sq += kThreads)
-        if (prefix[sq] <= rem && rem < prefix[sq + 1]) scratch[8] = sq;
+    for (int sq = threadIdx.x; sq < a.num_seqs; sq += blockDim.x)
+        if (prefix[sq] <= rem && rem < prefix[sq + 1]) scratch[kMaxWaves] = sq;
     __syncthreads();
-    const int r = scratch[8];
+    const int r = scratch[kMaxWaves];
     __syncthreads();
     return r;
 }

@@ -48,26 +48,26 @@ struct BandDesc {
 };
 enum : int32_t { kUnitCtx = 1, kUnitFirst = 2, kUnitLast = 4, kUnitComplete = 8 };
 
-template <int HD, int NB>
-struct StreamCfg : Shape<HD, NB> {
-    using S = Shape<HD, NB>;
+template <int HD, int NB, int NW>
+struct StreamCfg : Shape<HD, NB, NW> {
+    using S = Shape<HD, NB, NW>;
     static constexpr int ROWB = HD * 2;               // bytes per token row
     static constexpr int CPR = ROWB / 16;             // 16-byte chunks per row
     static constexpr int RPI = 1024 / ROWB;           // rows one wave-wide load covers
     static constexpr int MAT_BYTES = S::TN * ROWB;    // K (or V) tile
     static constexpr int STAGE_BYTES = 2 * MAT_BYTES;
     static constexpr int kStages = 4;
-    static constexpr int IPW = MAT_BYTES / 1024 / kWaves;  // loads per wave per matrix per tile
+    static constexpr int IPW = MAT_BYTES / 1024 / NW;  // loads per wave per matrix per tile
     static constexpr int LOADS_PER_UNIT = 2 * IPW;
-    static constexpr int ROWS_PER_WAVE = IPW * RPI;        // 16
-    static constexpr int kPlanUnits = 128;                 // units planned (and then streamed) at a time
+    static constexpr int ROWS_PER_WAVE = IPW * RPI;        // 16 (4 waves) or 8 (8 waves)
+    static constexpr int kPlanUnits = 512 / NW;            // units planned (and then streamed) at a time
     static constexpr int UNIT_TABLE_BYTES = kPlanUnits * static_cast<int>(sizeof(UnitDesc));
-    static constexpr int BAND_TABLE_BYTES = kPlanUnits * kWaves * static_cast<int>(sizeof(BandDesc));
+    static constexpr int BAND_TABLE_BYTES = kPlanUnits * NW * static_cast<int>(sizeof(BandDesc));
     static constexpr int UNIT_TABLE_OFF = S::PREFIX_BYTES + S::MISC_BYTES;
     static constexpr int BAND_TABLE_OFF = UNIT_TABLE_OFF + UNIT_TABLE_BYTES;
     static constexpr int STAGES_OFF = BAND_TABLE_OFF + BAND_TABLE_BYTES;
     static constexpr int LDS_BYTES = STAGES_OFF + kStages * STAGE_BYTES;
-    static_assert(ROWS_PER_WAVE == 16, "a wave loads a 16-row band of each tile");
+    static_assert(ROWS_PER_WAVE * NW == S::TN && IPW >= 1, "the waves' row bands tile the 64 rows");
     static_assert(LDS_BYTES <= 160 * 1024, "LDS budget of a gfx950 compute unit");
 
     // chunk position = chunk index ^ swizzle(row); 16 consecutive rows of one chunk column hit
@@ -119,10 +119,10 @@ DFX_D void mfma_outputs_ready(f32x16& x0, f32x16& x1, f32x16& x2, f32x16& x3) {
     asm volatile("s_nop 15\n\ts_nop 1" : "+a"(x0), "+a"(x1), "+a"(x2), "+a"(x3));
 }
 
-template <int HD, int NB>
-struct StreamAttn : AttnState<HD, NB> {
-    using Base = AttnState<HD, NB>;
-    using C = StreamCfg<HD, NB>;
+template <int HD, int NB, int NW>
+struct StreamAttn : AttnState<HD, NB, NW> {
+    using Base = AttnState<HD, NB, NW>;
+    using C = StreamCfg<HD, NB, NW>;
     using Base::a;
     using Base::col;
     using Base::half;
@@ -152,10 +152,10 @@ struct StreamAttn : AttnState<HD, NB> {
     // Describe units [first, first + count) in the plan table (entry i is unit first + i); one
     // lane per (unit, wave).
     DFX_D void plan_units(int64_t first, int count) const {
-        for (int idx = tid; idx < count * kWaves; idx += kThreads) {
-            const int64_t pos = first + (idx >> 2);
-            const int w = idx & 3;
-            const int slot_in_ring = idx >> 2;
+        for (int idx = tid; idx < count * NW; idx += C::THREADS) {
+            const int64_t pos = first + idx / NW;
+            const int w = idx % NW;
+            const int slot_in_ring = idx / NW;
             const int kv_head = static_cast<int>(pos / per_head);
             const int rem = static_cast<int>(pos - static_cast<int64_t>(kv_head) * per_head);
             int lo = 0, hi = a.num_seqs;  // the sequence with prefix[s] <= rem < prefix[s + 1]
@@ -207,14 +207,14 @@ struct StreamAttn : AttnState<HD, NB> {
             }
             b.last = limit - 1 - band;
             b.is_ctx = is_ctx ? 1 : 0;
-            bands[slot_in_ring * kWaves + w] = b;
+            bands[slot_in_ring * NW + w] = b;
         }
     }
 
     // ---- loads -----------------------------------------------------------------------------
     // Start the loads of planned unit `rel` (this wave's 16-row band of K and V) into its ring stage.
     DFX_D void issue_unit(int rel) const {
-        const BandDesc b = bands[rel * kWaves + wave];
+        const BandDesc b = bands[rel * NW + wave];
         const int last = uniform(b.last);
         const bool is_ctx = uniform(b.is_ctx) != 0;
         const int64_t off = (static_cast<int64_t>(uniform(static_cast<int>(b.off >> 32))) << 32) |
@@ -260,18 +260,25 @@ struct StreamAttn : AttnState<HD, NB> {
         return __builtin_bit_cast(bf16x8, v);
     }
 
+    // The LDS operands of the next step are requested before the matrix instructions of the
+    // current one: being volatile assembly those pin the order, so the LDS latency is hidden
+    // only by what the source puts in between.
     DFX_D void scores(const uint8_t* k_tile, f32x16 (&sc)[2][NB]) const {
+        bf16x8 ka[2][2];
+#pragma unroll
+        for (int tb = 0; tb < 2; ++tb) ka[0][tb] = read_k(k_tile, tb, 0);
 #pragma unroll
         for (int slab = 0; slab < C::NSLAB; ++slab) {
-            bf16x8 ka[2];
+            if (slab + 1 < C::NSLAB) {
 #pragma unroll
-            for (int tb = 0; tb < 2; ++tb) ka[tb] = read_k(k_tile, tb, slab);
+                for (int tb = 0; tb < 2; ++tb) ka[(slab + 1) & 1][tb] = read_k(k_tile, tb, slab + 1);
+            }
 #pragma unroll
             for (int tb = 0; tb < 2; ++tb)
 #pragma unroll
                 for (int qb = 0; qb < NB; ++qb) {
-                    if (slab == 0) mfma_scores_first(sc[tb][qb], ka[tb], qf[qb][slab]);
-                    else mfma_scores(sc[tb][qb], ka[tb], qf[qb][slab]);
+                    if (slab == 0) mfma_scores_first(sc[tb][qb], ka[slab & 1][tb], qf[qb][slab]);
+                    else mfma_scores(sc[tb][qb], ka[slab & 1][tb], qf[qb][slab]);
                 }
         }
         if constexpr (NB == 2) mfma_results_ready(sc[0][0], sc[0][1], sc[1][0], sc[1][1]);
@@ -288,16 +295,20 @@ struct StreamAttn : AttnState<HD, NB> {
     }
 
     DFX_D void accumulate(const uint8_t* v_tile, const bf16x8 (&pb)[NB][2][2]) {
+        constexpr int kSteps = 4 * C::NDB;  // (tb, sl, db)
+        bf16x8 va[3];
+        va[0] = read_vt(v_tile, 0, 0, 0);
+        va[1] = read_vt(v_tile, 0, 0, 1);
 #pragma unroll
-        for (int tb = 0; tb < 2; ++tb)
+        for (int st = 0; st < kSteps; ++st) {
+            const int tb = st / (2 * C::NDB), sl = (st / C::NDB) & 1, db = st % C::NDB;
+            if (st + 2 < kSteps) {
+                const int n = st + 2;
+                va[n % 3] = read_vt(v_tile, n / (2 * C::NDB), (n / C::NDB) & 1, n % C::NDB);
+            }
 #pragma unroll
-            for (int sl = 0; sl < 2; ++sl)
-#pragma unroll
-                for (int db = 0; db < C::NDB; ++db) {
-                    const bf16x8 va = read_vt(v_tile, tb, sl, db);
-#pragma unroll
-                    for (int qb = 0; qb < NB; ++qb) mfma_output(o[db][qb], va, pb[qb][tb][sl]);
-                }
+            for (int qb = 0; qb < NB; ++qb) mfma_output(o[db][qb], va[st % 3], pb[qb][tb][sl]);
+        }
     }
 
     // Make the compiler wait for the query loads here (before more asynchronous loads are queued
@@ -319,11 +330,11 @@ struct StreamAttn : AttnState<HD, NB> {
     }
 };
 
-template <int HD, int NB>
-__global__ void __launch_bounds__(kThreads) paged_attn_stream_kernel(const KArgs a) {
+template <int HD, int NB, int NW>
+__global__ void __launch_bounds__(64 * NW) paged_attn_stream_kernel(const KArgs a) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-    using C = StreamCfg<HD, NB>;
-    StreamAttn<HD, NB> at(a, smem);
+    using C = StreamCfg<HD, NB, NW>;
+    StreamAttn<HD, NB, NW> at(a, smem);
     at.per_head = build_unit_prefix<C::RT>(a, at.prefix, at.misc);
     const int64_t total = static_cast<int64_t>(at.per_head) * a.h_kv;
     if (total == 0) return;

@@ -108,10 +108,14 @@ int64_t plan_workspace_bytes(const Plan& plan) { return 2 * static_cast<int64_t>
 template <int HD, int NB, int PATH>
 int launch(const KArgs& ka, const Plan& plan, int rt_max, hipStream_t st) {
     void (*main_k)(const KArgs);
-    int lds;
+    int lds, threads = kThreads;
     if constexpr (PATH == 2) {
-        main_k = paged_attn_stream_kernel<HD, NB>;
-        lds = StreamCfg<HD, NB>::LDS_BYTES;
+        // the streaming path gives every wave one 32-row query block: 4 waves for up to 128 rows,
+        // 8 waves (two per SIMD, so one wave's softmax overlaps the other's matrix work) for 256
+        constexpr int NW = 4 * NB;
+        main_k = paged_attn_stream_kernel<HD, 1, NW>;
+        lds = StreamCfg<HD, 1, NW>::LDS_BYTES;
+        threads = 64 * NW;
     } else {
         main_k = paged_attn_generic_kernel<HD, NB, PATH == 1>;
         lds = GenericCfg<HD, NB>::LDS_BYTES;
@@ -124,7 +128,7 @@ int launch(const KArgs& ka, const Plan& plan, int rt_max, hipStream_t st) {
             return DFX_ERR_LAUNCH;
         configured = true;
     }
-    hipLaunchKernelGGL(main_k, dim3(plan.n_wg), dim3(kThreads), lds, st, ka);
+    hipLaunchKernelGGL(main_k, dim3(plan.n_wg), dim3(threads), lds, st, ka);
     if (hipGetLastError() != hipSuccess) return DFX_ERR_LAUNCH;
     if (plan.n_wg > 1 && rt_max > 0) {
         hipLaunchKernelGGL(comb_k, dim3(rt_max, ka.num_seqs, ka.h_kv), dim3(kThreads), 0, st, ka);

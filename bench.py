@@ -99,6 +99,9 @@ def main():
     ap.add_argument("--workload", default="c3", choices=["c3", "c4", "c5", "c1"])
     ap.add_argument("--copies", type=int, default=4, help="independent KV-cache copies rotated between steps")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="instead of the benchmark, run --steps plain device copies of 1 GiB (a kernel of known "
+                         "HBM traffic: 1 GiB read, 1 GiB written) to scale the FETCH_SIZE / WRITE_SIZE counters")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this path shards by KV head / sequence with no exchange step, "
@@ -111,6 +114,15 @@ def main():
 
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if args.calibrate_copy:
+        src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).random_(0, 255)
+        dst = torch.empty_like(src)
+        for _ in range(args.steps):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"calibration": "device copy", "bytes_read": 1 << 30, "bytes_written": 1 << 30,
+                          "launches": args.steps}))
+        return
     wl = make_workload(args.workload, device=dev)
     caches = [(wl.k_cache, wl.v_cache)]
     for _ in range(args.copies - 1):

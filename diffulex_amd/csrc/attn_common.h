@@ -39,7 +39,8 @@ struct KArgs {
     const int32_t* cu_new;
     const float* k_scale;
     const float* v_scale;
-    float* workspace;
+    float* workspace;  // partial-result slots
+    int* arrivals;     // one arrival counter per workgroup, zero between launches
     int64_t q_st, q_sh, kn_st, kn_sh, vn_st, vn_sh, o_st, o_sh;
     int64_t c_sp, c_st, c_sh;  // cache strides in elements: page, token, head
     int64_t bt_stride, n_pages;
@@ -288,21 +289,30 @@ struct AttnState {
 
     DFX_D float* slot_ptr(int slot) const { return a.workspace + static_cast<int64_t>(slot) * S::SLOT_FLOATS; }
 
-    // Unnormalised accumulators, running maxima and row sums of a piece of an item.
+    // Partial results travel between workgroups on different XCDs, whose L2 caches are not
+    // coherent with each other for ordinary accesses.  They are therefore written and read with
+    // device-scope (relaxed, atomic) accesses, which go through to memory, instead of bracketing
+    // ordinary accesses with device-scope fences: such a fence writes back and invalidates the
+    // whole L2 of the XCD, which costs far more than these few kilobytes.
+    DFX_D static void put(float* p, float v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+    DFX_D static float get(const float* p) {
+        return __hip_atomic_load(const_cast<float*>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+
+    // Unnormalised accumulators, running maxima and row sums of a piece of an item.  Layout of a
+    // 32-row block: accumulator e of d block db at float (db * 16 + e) * 64 + lane, then the
+    // maxima and the row sums.
     DFX_D void store_partial(int slot, const float (&l_tot)[NB]) const {
 #pragma unroll
         for (int qb = 0; qb < NB; ++qb) {
             float* bp = slot_ptr(slot) + (wave * NB + qb) * S::BLOCK_FLOATS;
-            f32x4* ov = reinterpret_cast<f32x4*>(bp);
 #pragma unroll
             for (int db = 0; db < S::NDB; ++db)
 #pragma unroll
-                for (int ii = 0; ii < 4; ++ii)
-                    ov[(db * 4 + ii) * 64 + lane] = f32x4{o[db][qb][ii * 4 + 0], o[db][qb][ii * 4 + 1],
-                                                          o[db][qb][ii * 4 + 2], o[db][qb][ii * 4 + 3]};
+                for (int e = 0; e < 16; ++e) put(bp + (db * 16 + e) * 64 + lane, o[db][qb][e]);
             float* ml = bp + S::NDB * 16 * 64;
-            ml[lane] = m_run[qb];
-            ml[64 + lane] = l_tot[qb];
+            put(ml + lane, m_run[qb]);
+            put(ml + 64 + lane, l_tot[qb]);
         }
     }
 
@@ -311,10 +321,9 @@ struct AttnState {
 #pragma unroll
         for (int qb = 0; qb < NB; ++qb) {
             const float* bp = slot_ptr(slot) + (wave * NB + qb) * S::BLOCK_FLOATS;
-            const f32x4* ov = reinterpret_cast<const f32x4*>(bp);
             const float* ml = bp + S::NDB * 16 * 64;
-            const float mp = ml[lane];
-            const float lp = ml[64 + lane];
+            const float mp = get(ml + lane);
+            const float lp = get(ml + 64 + lane);
             const float mn = fmaxf(m_run[qb], mp);
             const float wa = (m_run[qb] == -INFINITY) ? 0.0f : fast_exp2(m_run[qb] - mn);
             const float wb = (mp == -INFINITY) ? 0.0f : fast_exp2(mp - mn);
@@ -323,14 +332,68 @@ struct AttnState {
 #pragma unroll
             for (int db = 0; db < S::NDB; ++db)
 #pragma unroll
-                for (int ii = 0; ii < 4; ++ii) {
-                    const f32x4 v = ov[(db * 4 + ii) * 64 + lane];
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) o[db][qb][ii * 4 + j] = o[db][qb][ii * 4 + j] * wa + v[j] * wb;
-                }
+                for (int e = 0; e < 16; ++e)
+                    o[db][qb][e] = o[db][qb][e] * wa + get(bp + (db * 16 + e) * 64 + lane) * wb;
         }
     }
 };
+
+// Epilogue of a piece of an item that the partition cut into pieces owned by consecutive
+// workgroups.  Every piece but the last one to finish is stored as a partial result; the
+// workgroup that finishes last merges the stored ones into its own registers and writes the
+// rows.  Who is last is decided by an arrival counter per item (indexed by the workgroup that
+// owns the item's first unit; a workgroup owns at most one such cut item):
+//   - a workgroup that finds every other piece already arrived merges without storing its own;
+//   - otherwise it stores its piece, waits until the stores have completed, and increments the
+//     counter; if that increment was the last arrival after all, it merges the others.
+// Nobody waits for anybody.  The last arrival resets the counter for the next launch.  Must be
+// called by every thread of the workgroup; l_tot are whole-row sums; `flag` is one int of LDS.
+template <int HD, int NB, int NW>
+DFX_D void finish_cut_item(AttnState<HD, NB, NW>& at, int rt, int64_t item_begin, int n_tiles, const WgSplit& split,
+                           int my_slot, const float (&l_tot)[NB], int* flag) {
+    const KArgs& a = at.a;
+    const int me = static_cast<int>(blockIdx.x);
+    int wa, wb;
+    owners_of_units(split, me, item_begin, item_begin + n_tiles - 1, wa, wb);
+    int pieces = wb - wa + 1;
+    if (split.q == 0) {  // fewer units than workgroups: some ranges are empty
+        pieces = 0;
+        for (int w = wa; w <= wb; ++w)
+            if (split.first(w) < split.first(w + 1)) ++pieces;
+    }
+    int* counter = a.arrivals + wa;
+
+    if (threadIdx.x == 0) *flag = __hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    bool last = *flag == pieces - 1;
+    __syncthreads();
+    if (!last) {
+#ifndef DFX_DBG_NO_PSTORE
+        at.store_partial(my_slot, l_tot);
+#endif
+        __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this thread's write-through stores have completed
+        __syncthreads();
+        if (threadIdx.x == 0) *flag = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __syncthreads();
+        last = *flag == pieces - 1;
+        __syncthreads();
+        if (!last) return;
+    }
+#pragma unroll
+    for (int qb = 0; qb < NB; ++qb) at.l_run[qb] = l_tot[qb];
+    for (int w = wa; w <= wb; ++w) {
+        const int64_t ws = split.first(w);
+        if (w == me || ws >= split.first(w + 1)) continue;
+#ifndef DFX_DBG_NO_MERGE
+        at.merge_partial(partial_slot(w, ws > item_begin ? ws : item_begin, ws));
+#endif
+    }
+    float l_all[NB];
+#pragma unroll
+    for (int qb = 0; qb < NB; ++qb) l_all[qb] = at.l_run[qb];
+    at.store_output(rt, l_all);
+    if (threadIdx.x == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
 
 // Exclusive prefix of units(s) into prefix[0..num_seqs]; returns the per-head total.
 template <int RT>

@@ -225,7 +225,8 @@ struct GenericAttn : AttnState<HD, NB> {
                 }
     }
 
-    DFX_D void run_segment(int rt, int tile0, int tile1, bool complete, int slot) {
+    DFX_D void run_segment(int rt, int tile0, int tile1, int64_t item_begin, const WgSplit& split, int slot) {
+        const bool complete = tile0 == 0 && tile1 == this->sh.n_tiles;
         this->load_queries(rt);
         __syncthreads();  // the previous segment's last tile may still be read from LDS
         int buf = 0;
@@ -240,7 +241,7 @@ struct GenericAttn : AttnState<HD, NB> {
         float l_tot[NB];
         this->row_sums(l_tot);
         if (complete) this->store_output(rt, l_tot);
-        else this->store_partial(slot, l_tot);
+        else finish_cut_item(*this, rt, item_begin, this->sh.n_tiles, split, slot, l_tot, misc + kMaxWaves + 1);
     }
 };
 
@@ -252,8 +253,9 @@ __global__ void __launch_bounds__(kThreads) paged_attn_generic_kernel(const KArg
     const int64_t total = static_cast<int64_t>(per_head) * a.h_kv;
     if (total == 0) return;
     const int w = blockIdx.x;
-    const int64_t begin = wg_first_unit(w, total, a.n_wg);
-    const int64_t end = wg_first_unit(w + 1, total, a.n_wg);
+    const WgSplit split = make_wg_split(total, a.n_wg);
+    const int64_t begin = split.first(w);
+    const int64_t end = split.first(w + 1);
     if (begin >= end) return;
 
     int kvh = static_cast<int>(begin / per_head);
@@ -268,8 +270,7 @@ __global__ void __launch_bounds__(kThreads) paged_attn_generic_kernel(const KArg
         const int tile0 = u - rt * n_tiles;
         const int64_t seg_end = min(pos + (n_tiles - tile0), end);
         const int tile1 = tile0 + static_cast<int>(seg_end - pos);
-        const bool complete = tile0 == 0 && tile1 == n_tiles;
-        at.run_segment(rt, tile0, tile1, complete, partial_slot(w, pos, begin));
+        at.run_segment(rt, tile0, tile1, pos - tile0, split, partial_slot(w, pos, begin));
         u += tile1 - tile0;
         pos = seg_end;
         if (pos >= end) break;

@@ -38,7 +38,9 @@ namespace dfx {
 struct UnitDesc {
     int32_t s, kvh, rt, q0;
     int32_t q_len, base, limit, flags;
-    int32_t slot, run, pad1, pad2;  // run: units from this one to the end of this workgroup's piece of the item
+    int32_t slot, run;   // run: units from this one to the end of this workgroup's piece of the item
+    int32_t item_rel;    // first unit of the item, relative to the workgroup's first unit
+    int32_t n_tiles;     // KV tiles of the item
 };
 static_assert(sizeof(UnitDesc) == 48, "UnitDesc is read as three 16-byte LDS words");
 struct BandDesc {
@@ -190,7 +192,8 @@ struct StreamAttn : AttnState<HD, NB, NW> {
                           (tile0 == 0 && tile1 == shp.n_tiles ? kUnitComplete : 0);
                 d.slot = partial_slot(static_cast<int>(blockIdx.x), pos - (tile - tile0), begin);
                 d.run = tile1 - tile;
-                d.pad1 = d.pad2 = 0;
+                d.item_rel = static_cast<int>(pos - tile - begin);
+                d.n_tiles = shp.n_tiles;
                 units[slot_in_ring] = d;
             }
             // Rows past the end re-read the last valid rows (finite data; their scores are masked).
@@ -311,8 +314,9 @@ struct StreamAttn : AttnState<HD, NB, NW> {
         }
     }
 
-    // Make the compiler wait for the query loads here (before more asynchronous loads are queued
-    // behind them, which its own wait would otherwise have to drain as well).
+    // Make the compiler wait for the query loads here, once per item.  Left to itself it puts the
+    // wait before their first use inside the tile loop, where it also drains the asynchronous tile
+    // loads issued since, in every iteration.
     DFX_D void touch_queries() const {
 #pragma unroll
         for (int qb = 0; qb < NB; ++qb)
@@ -327,6 +331,7 @@ struct StreamAttn : AttnState<HD, NB, NW> {
         this->q0 = uniform(d.q0);
         this->sh.q_len = uniform(d.q_len);
         this->load_queries(uniform(d.rt));
+        touch_queries();
     }
 };
 
@@ -339,8 +344,9 @@ __global__ void __launch_bounds__(64 * NW) paged_attn_stream_kernel(const KArgs 
     const int64_t total = static_cast<int64_t>(at.per_head) * a.h_kv;
     if (total == 0) return;
     const int w = blockIdx.x;
-    at.begin = wg_first_unit(w, total, a.n_wg);
-    at.end = wg_first_unit(w + 1, total, a.n_wg);
+    const WgSplit split = make_wg_split(total, a.n_wg);
+    at.begin = split.first(w);
+    at.end = split.first(w + 1);
     if (at.begin >= at.end) return;
     const int64_t begin = at.begin, end = at.end;
 
@@ -360,7 +366,6 @@ __global__ void __launch_bounds__(64 * NW) paged_attn_stream_kernel(const KArgs 
             const int flags = uniform(d.flags);
             const int run_end = min(rel + uniform(d.run), n_units);
             if (flags & kUnitFirst) at.begin_item(d);
-            bool queries_pending = (flags & kUnitFirst) != 0;
             for (; rel < run_end; ++rel) {
                 // the unit must have landed: only younger units may still be outstanding
                 const int younger = issued - rel - 1;
@@ -369,10 +374,6 @@ __global__ void __launch_bounds__(64 * NW) paged_attn_stream_kernel(const KArgs 
                 else wait_async_loads<0>();
                 __builtin_amdgcn_s_barrier();
                 // every wave has finished the previous unit: its stage may be overwritten
-                if (queries_pending) {
-                    at.touch_queries();
-                    queries_pending = false;
-                }
                 if (issued < n_units) at.issue_unit(issued++);
 
                 const UnitDesc u = at.units[rel];
@@ -395,7 +396,8 @@ __global__ void __launch_bounds__(64 * NW) paged_attn_stream_kernel(const KArgs 
                 float l_tot[NB];
                 at.row_sums(l_tot);
                 if (uniform(e.flags) & kUnitComplete) at.store_output(uniform(e.rt), l_tot);
-                else at.store_partial(uniform(e.slot), l_tot);
+                else finish_cut_item(at, uniform(e.rt), begin + uniform(e.item_rel), uniform(e.n_tiles), split,
+                                     uniform(e.slot), l_tot, at.misc + kMaxWaves + 1);
             }
         }
     }

@@ -1,4 +1,4 @@
-// Block-diffusion paged attention for gfx950 (MI355X): kernels, combine pass and C entry points.
+// Block-diffusion paged attention for gfx950 (MI355X): kernel dispatch and C entry points.
 //
 // One persistent workgroup (4 wavefronts) per compute unit walks an equal share of the linear
 // work list described in partition.h.  For one (sequence, KV head, row tile) item the
@@ -14,47 +14,6 @@
 
 namespace dfx {
 namespace {
-
-// One workgroup per (row tile, sequence, KV head): if the item was cut by the partition,
-// merge its pieces and write the rows; otherwise the main kernel has already written them.
-template <int HD, int NB>
-__global__ void __launch_bounds__(kThreads) paged_attn_combine_kernel(const KArgs a) {
-    __shared__ int scan_scratch[kWaves];
-    AttnState<HD, NB> at(a);
-    using S = Shape<HD, NB>;
-    const int rt = blockIdx.x, s = blockIdx.y, kvh = blockIdx.z;
-    // units before sequence s and per-head total, by a strided block reduction
-    int before = 0, all = 0;
-    for (int sq = threadIdx.x; sq < a.num_seqs; sq += kThreads) {
-        const int u = load_seq_shape(a, sq, S::RT).units;
-        all += u;
-        if (sq < s) before += u;
-    }
-    int tot_all, tot_before;
-    block_inclusive_scan(all, scan_scratch, tot_all);
-    block_inclusive_scan(before, scan_scratch, tot_before);
-    at.set_sequence(s, kvh);
-    if (rt >= at.sh.n_row_tiles || at.sh.n_tiles == 0) return;
-    const int64_t total = static_cast<int64_t>(tot_all) * a.h_kv;
-    const int64_t item_begin =
-        static_cast<int64_t>(kvh) * tot_all + tot_before + static_cast<int64_t>(rt) * at.sh.n_tiles;
-    const int64_t item_end = item_begin + at.sh.n_tiles;
-    const int wa = wg_of_unit(item_begin, total, a.n_wg);
-    const int wb = wg_of_unit(item_end - 1, total, a.n_wg);
-    if (wa == wb) return;
-    at.reset_accumulators();
-    for (int w = wa; w <= wb; ++w) {
-        const int64_t ws = wg_first_unit(w, total, a.n_wg);
-        const int64_t we = wg_first_unit(w + 1, total, a.n_wg);
-        if (ws >= we) continue;
-        const int64_t pb = ws > item_begin ? ws : item_begin;
-        at.merge_partial(partial_slot(w, pb, ws));
-    }
-    float l_tot[NB];
-#pragma unroll
-    for (int qb = 0; qb < NB; ++qb) l_tot[qb] = at.l_run[qb];
-    at.store_output(rt, l_tot);
-}
 
 struct Plan {
     int hd, nb, n_wg;
@@ -102,11 +61,16 @@ int make_plan(const dfx_attn_params* p, Plan& plan) {
     return DFX_OK;
 }
 
-int64_t plan_workspace_bytes(const Plan& plan) { return 2 * static_cast<int64_t>(plan.n_wg) * plan.slot_floats * 4; }
+// Workspace layout: arrival counters (one int per workgroup, rounded up to 256 bytes), then two
+// partial-result slots per workgroup.
+int64_t counter_bytes(const Plan& plan) { return (static_cast<int64_t>(plan.n_wg) * 4 + 255) / 256 * 256; }
+int64_t plan_workspace_bytes(const Plan& plan) {
+    return counter_bytes(plan) + 2 * static_cast<int64_t>(plan.n_wg) * plan.slot_floats * 4;
+}
 
 // PATH: 0 generic bf16, 1 generic FP8, 2 streaming bf16
 template <int HD, int NB, int PATH>
-int launch(const KArgs& ka, const Plan& plan, int rt_max, hipStream_t st) {
+int launch(const KArgs& ka, const Plan& plan, hipStream_t st) {
     void (*main_k)(const KArgs);
     int lds, threads = kThreads;
     if constexpr (PATH == 2) {
@@ -120,7 +84,6 @@ int launch(const KArgs& ka, const Plan& plan, int rt_max, hipStream_t st) {
         main_k = paged_attn_generic_kernel<HD, NB, PATH == 1>;
         lds = GenericCfg<HD, NB>::LDS_BYTES;
     }
-    auto comb_k = paged_attn_combine_kernel<HD, NB>;
     static bool configured = false;  // raising the dynamic LDS limit is idempotent
     if (!configured) {
         if (hipFuncSetAttribute(reinterpret_cast<const void*>(main_k), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -130,10 +93,6 @@ int launch(const KArgs& ka, const Plan& plan, int rt_max, hipStream_t st) {
     }
     hipLaunchKernelGGL(main_k, dim3(plan.n_wg), dim3(threads), lds, st, ka);
     if (hipGetLastError() != hipSuccess) return DFX_ERR_LAUNCH;
-    if (plan.n_wg > 1 && rt_max > 0) {
-        hipLaunchKernelGGL(comb_k, dim3(rt_max, ka.num_seqs, ka.h_kv), dim3(kThreads), 0, st, ka);
-        if (hipGetLastError() != hipSuccess) return DFX_ERR_LAUNCH;
-    }
     return DFX_OK;
 }
 
@@ -193,7 +152,8 @@ extern "C" int dfx_paged_attn(const dfx_attn_params* p, dfx_stream_t stream) {
     ka.cu_new = p->cu_seqlens_new;
     ka.k_scale = p->k_scale;
     ka.v_scale = p->v_scale;
-    ka.workspace = static_cast<float*>(p->workspace);
+    ka.arrivals = static_cast<int*>(p->workspace);
+    ka.workspace = reinterpret_cast<float*>(static_cast<uint8_t*>(p->workspace) + counter_bytes(plan));
     ka.q_st = p->q_stride_token;
     ka.q_sh = p->q_stride_head;
     ka.kn_st = p->kn_stride_token;
@@ -222,17 +182,12 @@ extern "C" int dfx_paged_attn(const dfx_attn_params* p, dfx_stream_t stream) {
     ka.n_wg = plan.n_wg;
     ka.c = p->scale * kLog2e;
 
-    const int rows_per_tile = 32 * plan.nb * kWaves;
-    const int64_t rows = static_cast<int64_t>(ka.group) * p->max_seqlen_q;
-    const int64_t rt_max = (rows + rows_per_tile - 1) / rows_per_tile;
-    if (rt_max > 65535) return DFX_ERR_UNSUPPORTED;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    const int rtm = static_cast<int>(rt_max);
 #define DFX_ATTN_CASE(HD_, NB_)                                               \
     if (plan.hd == HD_ && plan.nb == NB_) {                                   \
-        if (plan.stream) return launch<HD_, NB_, 2>(ka, plan, rtm, st);       \
-        if (plan.fp8) return launch<HD_, NB_, 1>(ka, plan, rtm, st);          \
-        return launch<HD_, NB_, 0>(ka, plan, rtm, st);                        \
+        if (plan.stream) return launch<HD_, NB_, 2>(ka, plan, st);       \
+        if (plan.fp8) return launch<HD_, NB_, 1>(ka, plan, st);          \
+        return launch<HD_, NB_, 0>(ka, plan, st);                        \
     }
     DFX_ATTN_CASE(64, 1)
     DFX_ATTN_CASE(64, 2)

@@ -52,6 +52,34 @@ DFX_HD int wg_of_unit(int64_t u, int64_t total, int n_wg) {
     return static_cast<int>(((u + 1) * n_wg - 1) / total);
 }
 
+// The same cut points without a 64-bit division at every use: with total = q * n_wg + r,
+// floor(w * total / n_wg) = w * q + floor(w * r / n_wg), and w * r fits 32 bits (n_wg < 65536).
+struct WgSplit {
+    int64_t q;
+    uint32_t r;
+    int n_wg;
+    DFX_HD int64_t first(int w) const {
+        return static_cast<int64_t>(w) * q + (static_cast<uint32_t>(w) * r) / static_cast<uint32_t>(n_wg);
+    }
+};
+
+DFX_HD WgSplit make_wg_split(int64_t total, int n_wg) {
+    WgSplit sp;
+    sp.q = total / n_wg;
+    sp.r = static_cast<uint32_t>(total - sp.q * n_wg);
+    sp.n_wg = n_wg;
+    return sp;
+}
+
+// The workgroups wa..wb whose ranges meet units [first_unit, last_unit] (wa = wg_of_unit(first_unit),
+// wb = wg_of_unit(last_unit)), found by walking from a workgroup `me` that owns one of those units.
+DFX_HD void owners_of_units(const WgSplit& sp, int me, int64_t first_unit, int64_t last_unit, int& wa, int& wb) {
+    wa = me;
+    while (sp.first(wa) > first_unit) --wa;
+    wb = me;
+    while (wb + 1 < sp.n_wg && sp.first(wb + 1) <= last_unit) ++wb;
+}
+
 // A workgroup writes at most two partial results: slot 2w for a piece that starts at the
 // first unit of its range, slot 2w+1 for a piece that starts later (it then necessarily
 // runs to the end of the range).

@@ -22,7 +22,8 @@ def _workspace(device: torch.device, stream: int, nbytes: int) -> torch.Tensor:
     key = (device.index, stream)
     ws = _workspaces.get(key)
     if ws is None or ws.numel() < nbytes:
-        ws = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=device)
+        # zero-filled once: the arrival counters at its start must be 0 before the first launch
+        ws = torch.zeros(max(nbytes, 1), dtype=torch.uint8, device=device)
         _workspaces[key] = ws
     return ws
 

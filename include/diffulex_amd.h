@@ -147,7 +147,8 @@ typedef struct dfx_attn_params {
     const int32_t* cu_seqlens_new; /* [num_seqs + 1] offsets of the fresh K/V rows */
     const float* k_scale;        /* fp32 [num_kv_heads], DFX_KV_FP8_E4M3 only */
     const float* v_scale;
-    void* workspace;             /* >= dfx_paged_attn_workspace_bytes(), 256-byte aligned */
+    void* workspace;             /* >= dfx_paged_attn_workspace_bytes(), 256-byte aligned, zero-filled
+                                    once before its first use (every call leaves it ready for the next) */
     int64_t workspace_bytes;
     int64_t q_stride_token, q_stride_head;
     int64_t kn_stride_token, kn_stride_head; /* k_new */
@@ -168,7 +169,11 @@ typedef struct dfx_attn_params {
 } dfx_attn_params;
 
 /* Bytes of scratch dfx_paged_attn needs for these shapes (depends on the sizes
- * and max_workgroups only, never on device data). Negative: dfx_status. */
+ * and max_workgroups only, never on device data). Negative: dfx_status.
+ * The workspace starts with one arrival counter per workgroup, which the kernel
+ * expects to be zero and resets before it ends: zero-fill a new workspace once
+ * (hipMemsetAsync, or a fill kernel under graph capture).  Calls that share a
+ * workspace must not overlap in time. */
 int64_t dfx_paged_attn_workspace_bytes(const dfx_attn_params* params);
 
 int dfx_paged_attn(const dfx_attn_params* params, dfx_stream_t stream);

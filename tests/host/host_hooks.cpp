@@ -38,6 +38,8 @@ int64_t hook_walk_segments(const int* ctx, const int* q_len, const int* new_len,
     if (total == 0) return 0;
     for (int w = 0; w < n_wg; ++w) {
         const int64_t begin = wg_first_unit(w, total, n_wg), end = wg_first_unit(w + 1, total, n_wg);
+        const WgSplit split = make_wg_split(total, n_wg);
+        if (split.first(w) != begin || split.first(w + 1) != end) return -1;  // the two forms of the cut agree
         if (begin >= end) continue;
         int kvh = static_cast<int>(begin / per_head);
         const int rem = static_cast<int>(begin - static_cast<int64_t>(kvh) * per_head);
@@ -71,8 +73,9 @@ int64_t hook_walk_segments(const int* ctx, const int* q_len, const int* new_len,
     return n;
 }
 
-// What the combine pass derives for item (kv_head, seq, row_tile): the slots it merges.
-// Returns the number of slots written (0: the item was not cut), -1 if the item is empty.
+// What the workgroups that own pieces of item (kv_head, seq, row_tile) derive when they finish
+// their piece: the slots of all pieces.  Returns the number of slots written (0: the item was
+// not cut), -1 if the item is empty, -2 if the walk from some owner disagrees with wg_of_unit.
 int hook_combine_slots(const int* ctx, const int* q_len, const int* new_len, int num_seqs, int h_kv, int group,
                        int rows_per_tile, int n_wg, int kvh, int s, int rt, int* slots, int cap) {
     using namespace dfx;
@@ -89,6 +92,13 @@ int hook_combine_slots(const int* ctx, const int* q_len, const int* new_len, int
     const int64_t item_begin = static_cast<int64_t>(kvh) * all + before + static_cast<int64_t>(rt) * mine.n_tiles;
     const int64_t item_end = item_begin + mine.n_tiles;
     const int wa = wg_of_unit(item_begin, total, n_wg), wb = wg_of_unit(item_end - 1, total, n_wg);
+    const WgSplit split = make_wg_split(total, n_wg);
+    for (int me = wa; me <= wb; ++me) {
+        if (split.first(me) >= split.first(me + 1)) continue;  // owns nothing
+        int xa, xb;
+        owners_of_units(split, me, item_begin, item_end - 1, xa, xb);
+        if (xa != wa || xb != wb) return -2;
+    }
     if (wa == wb) return 0;
     int n = 0;
     for (int w = wa; w <= wb; ++w) {

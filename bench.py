@@ -30,8 +30,8 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this command, scaled by
-# what the same counters read for a plain copy of known size (see profiles/); None until measured.
-MEASURED_TRAFFIC_BYTES = {}
+# what the same counters read for a plain copy of known size (profiles/paged_attn_stream_kernel_c3.md).
+MEASURED_TRAFFIC_BYTES = {"c3": 283.4e6}
 
 
 def algorithmic_bytes(wl) -> int:
@@ -91,12 +91,68 @@ def cpu_baseline(name: str, budget_s: float = 15.0):
     }
 
 
+def bench_kv_cache(args, dev):
+    """Workload C2: paged KV-cache store of one fresh block per sequence, then the gather of every
+    context (plus the fresh rows) into packed buffers -- both through the C ABI, outputs preallocated."""
+    import ctypes as C
+    from diffulex_amd import _lib
+    from diffulex_amd.workloads import make_workload
+    lib = _lib.load()
+    wl = make_workload("c2", device=dev)
+    st = torch.cuda.current_stream().cuda_stream
+    n_new, h, hd = wl.k_new.shape
+    total = int(wl.cu_seqlens_k[-1])
+    max_total = int((wl.context_lens + wl.seq_lens_new).max())
+    k_out = torch.empty((total, h, hd), device=dev, dtype=wl.k_cache.dtype)
+    v_out = torch.empty_like(k_out)
+    n_slots = wl.k_cache.shape[0] * wl.k_cache.shape[1]
+    bt = wl.block_tables
+
+    def step(_):
+        rc = lib.dfx_kv_store_unified(wl.k_new.data_ptr(), wl.v_new.data_ptr(), wl.k_new.stride(0), wl.v_new.stride(0),
+                                      wl.k_cache.data_ptr(), wl.v_cache.data_ptr(), wl.slot_mapping.data_ptr(),
+                                      _lib.DFX_INDEX_I32, n_new, n_slots, h, hd, _lib.DFX_KV_BF16, None, None, st)
+        _lib.check(rc, "dfx_kv_store_unified")
+        rc = lib.dfx_kv_load(wl.k_cache.data_ptr(), wl.v_cache.data_ptr(), wl.k_new.data_ptr(), wl.v_new.data_ptr(),
+                             wl.k_new.stride(0), wl.v_new.stride(0), k_out.data_ptr(), v_out.data_ptr(),
+                             bt.data_ptr(), bt.stride(0), wl.context_lens.data_ptr(), wl.seq_lens_new.data_ptr(),
+                             wl.cu_seqlens_q.data_ptr(), wl.cu_seqlens_k.data_ptr(), wl.num_seqs, bt.shape[1],
+                             wl.k_cache.shape[0], wl.page_size, h, hd, max_total, _lib.DFX_KV_BF16, None, None, st)
+        _lib.check(rc, "dfx_kv_load")
+
+    for i in range(args.warmup):
+        step(i)
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for i in range(args.steps):
+        step(i)
+    stop.record()
+    torch.cuda.synchronize()
+    ms = start.elapsed_time(stop) / args.steps
+    row = h * hd * wl.k_cache.element_size()
+    nbytes = 2 * 2 * n_new * row + 2 * 2 * total * row  # K and V: store reads+writes the block, load reads+writes every row
+    gbs = nbytes / (ms * 1e-3) / 1e9
+    tokens = n_new + total
+    print(json.dumps({
+        "metric": "paged KV-cache store + load, tokens moved per second and achieved HBM GB/s, 1 GPU",
+        "value": tokens / (ms * 1e-3), "unit": "kv-tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "u16 (bit copy)",
+        "data": "synthetic",
+        "config": {"workload": f"c2: store {n_new} fresh tokens (B={wl.num_seqs} x 32) by slot_mapping, then gather "
+                               f"{total} context+fresh tokens by block_table; H_kv={h}, head_dim={hd}, page={wl.page_size}"},
+        "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS,
+                     "traffic": None, "algorithmic_bytes": nbytes,
+                     "kernel": "kv_store_unified + kv_load, duration = timed region / steps (two launches)"},
+    }))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="c3", choices=["c3", "c4", "c5", "c1"])
+    ap.add_argument("--workload", default="c3", choices=["c3", "c4", "c5", "c1", "c2"])
     ap.add_argument("--copies", type=int, default=4, help="independent KV-cache copies rotated between steps")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -122,6 +178,9 @@ def main():
         torch.cuda.synchronize()
         print(json.dumps({"calibration": "device copy", "bytes_read": 1 << 30, "bytes_written": 1 << 30,
                           "launches": args.steps}))
+        return
+    if args.workload == "c2":
+        bench_kv_cache(args, dev)
         return
     wl = make_workload(args.workload, device=dev)
     caches = [(wl.k_cache, wl.v_cache)]
@@ -172,7 +231,8 @@ def main():
             "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
             "algorithmic_bytes": nbytes, "algorithmic_flops": nflops,
             "mfma_tflops": tflops, "mfma_frac": tflops / MFMA_BF16_PEAK_TFLOPS,
-            "kernel": "paged_attn_kernel (+ combine pass), duration = timed region / steps",
+            "kernel": "paged_attn_stream_kernel / paged_attn_generic_kernel (one launch per step), "
+                      "duration = timed region / steps",
         },
     }
     if not args.no_cpu:

@@ -291,28 +291,40 @@ struct AttnState {
 
     // Partial results travel between workgroups on different XCDs, whose L2 caches are not
     // coherent with each other for ordinary accesses.  They are therefore written and read with
-    // device-scope (relaxed, atomic) accesses, which go through to memory, instead of bracketing
-    // ordinary accesses with device-scope fences: such a fence writes back and invalidates the
-    // whole L2 of the XCD, which costs far more than these few kilobytes.
-    DFX_D static void put(float* p, float v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
-    DFX_D static float get(const float* p) {
-        return __hip_atomic_load(const_cast<float*>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    // device-scope accesses (the sc1 cache-policy bit of the buffer instructions), which go
+    // through to memory, instead of bracketing ordinary accesses with device-scope fences: such a
+    // fence writes back and invalidates the whole L2 of the XCD, which costs far more than these
+    // few kilobytes.  16 bytes per lane: one such instruction keeps the address unit busy as
+    // long as a 4-byte one.
+    typedef uint32_t u32x4v __attribute__((ext_vector_type(4)));
+    static constexpr int kDeviceScope = 16;  // cache policy: sc1
+
+    DFX_D __amdgpu_buffer_rsrc_t block_resource(int slot, int qb) const {
+        float* bp = slot_ptr(slot) + (wave * NB + qb) * S::BLOCK_FLOATS;
+        return __builtin_amdgcn_make_buffer_rsrc(bp, 0, S::BLOCK_FLOATS * 4, 0x00020000);
     }
 
     // Unnormalised accumulators, running maxima and row sums of a piece of an item.  Layout of a
-    // 32-row block: accumulator e of d block db at float (db * 16 + e) * 64 + lane, then the
-    // maxima and the row sums.
+    // 32-row block: accumulators 4*ii .. 4*ii+3 of d block db as 16 bytes at ((db * 4 + ii) * 64
+    // + lane) * 16, then the maxima and the row sums (one float per lane each).
     DFX_D void store_partial(int slot, const float (&l_tot)[NB]) const {
 #pragma unroll
         for (int qb = 0; qb < NB; ++qb) {
-            float* bp = slot_ptr(slot) + (wave * NB + qb) * S::BLOCK_FLOATS;
+            const __amdgpu_buffer_rsrc_t rs = block_resource(slot, qb);
 #pragma unroll
             for (int db = 0; db < S::NDB; ++db)
 #pragma unroll
-                for (int e = 0; e < 16; ++e) put(bp + (db * 16 + e) * 64 + lane, o[db][qb][e]);
-            float* ml = bp + S::NDB * 16 * 64;
-            put(ml + lane, m_run[qb]);
-            put(ml + 64 + lane, l_tot[qb]);
+                for (int ii = 0; ii < 4; ++ii) {
+                    const f32x4 v = {o[db][qb][ii * 4 + 0], o[db][qb][ii * 4 + 1], o[db][qb][ii * 4 + 2],
+                                     o[db][qb][ii * 4 + 3]};
+                    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4v, v), rs,
+                                                           ((db * 4 + ii) * 64 + lane) * 16, 0, kDeviceScope);
+                }
+            const int ml = S::NDB * 16 * 64 * 4;
+            __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, m_run[qb]), rs, ml + lane * 4, 0,
+                                                  kDeviceScope);
+            __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, l_tot[qb]), rs, ml + 256 + lane * 4, 0,
+                                                  kDeviceScope);
         }
     }
 
@@ -320,20 +332,28 @@ struct AttnState {
     DFX_D void merge_partial(int slot) {
 #pragma unroll
         for (int qb = 0; qb < NB; ++qb) {
-            const float* bp = slot_ptr(slot) + (wave * NB + qb) * S::BLOCK_FLOATS;
-            const float* ml = bp + S::NDB * 16 * 64;
-            const float mp = get(ml + lane);
-            const float lp = get(ml + 64 + lane);
+            const __amdgpu_buffer_rsrc_t rs = block_resource(slot, qb);
+            const int ml = S::NDB * 16 * 64 * 4;
+            const float mp = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rs, ml + lane * 4, 0, kDeviceScope));
+            const float lp =
+                __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rs, ml + 256 + lane * 4, 0, kDeviceScope));
             const float mn = fmaxf(m_run[qb], mp);
             const float wa = (m_run[qb] == -INFINITY) ? 0.0f : fast_exp2(m_run[qb] - mn);
             const float wb = (mp == -INFINITY) ? 0.0f : fast_exp2(mp - mn);
-            l_run[qb] = l_run[qb] * wa + lp * wb;
+            // products and sum are rounded separately: merging a into b then gives the same bits as
+            // b into a, so it does not matter which of two pieces does the merging
+            l_run[qb] = __fadd_rn(__fmul_rn(l_run[qb], wa), __fmul_rn(lp, wb));
             m_run[qb] = mn;
 #pragma unroll
             for (int db = 0; db < S::NDB; ++db)
 #pragma unroll
-                for (int e = 0; e < 16; ++e)
-                    o[db][qb][e] = o[db][qb][e] * wa + get(bp + (db * 16 + e) * 64 + lane) * wb;
+                for (int ii = 0; ii < 4; ++ii) {
+                    const f32x4 v = __builtin_bit_cast(
+                        f32x4, __builtin_amdgcn_raw_buffer_load_b128(rs, ((db * 4 + ii) * 64 + lane) * 16, 0, kDeviceScope));
+#pragma unroll
+                    for (int j = 0; j < 4; ++j)
+                        o[db][qb][ii * 4 + j] = __fadd_rn(__fmul_rn(o[db][qb][ii * 4 + j], wa), __fmul_rn(v[j], wb));
+                }
         }
     }
 };
@@ -341,7 +361,7 @@ struct AttnState {
 // Epilogue of a piece of an item that the partition cut into pieces owned by consecutive
 // workgroups.  Every piece but the last one to finish is stored as a partial result; the
 // workgroup that finishes last merges the stored ones into its own registers and writes the
-// rows.  Who is last is decided by an arrival counter per item (indexed by the workgroup that
+// rows (bit-identical whichever piece that is).  Who is last is decided by an arrival counter per item (indexed by the workgroup that
 // owns the item's first unit; a workgroup owns at most one such cut item):
 //   - a workgroup that finds every other piece already arrived merges without storing its own;
 //   - otherwise it stores its piece, waits until the stores have completed, and increments the
@@ -367,11 +387,13 @@ DFX_D void finish_cut_item(AttnState<HD, NB, NW>& at, int rt, int64_t item_begin
     __syncthreads();
     bool last = *flag == pieces - 1;
     __syncthreads();
-    if (!last) {
-#ifndef DFX_DBG_NO_PSTORE
+    bool stored = false;
+    if (!last || pieces > 2) {
         at.store_partial(my_slot, l_tot);
-#endif
         __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this thread's write-through stores have completed
+        stored = true;
+    }
+    if (!last) {
         __syncthreads();
         if (threadIdx.x == 0) *flag = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __syncthreads();
@@ -379,15 +401,23 @@ DFX_D void finish_cut_item(AttnState<HD, NB, NW>& at, int rt, int64_t item_begin
         __syncthreads();
         if (!last) return;
     }
+    // The result must not depend on which piece arrives last.  Two pieces: the merge is
+    // commutative bit for bit (see merge_partial).  More (rare): every piece, this one included,
+    // is merged from memory in workgroup order, starting from the empty state.
+    const bool from_memory = pieces > 2;
+    if (from_memory) {
+        __syncthreads();  // every thread's stores of this piece have completed
+        at.reset_accumulators();
+    } else {
 #pragma unroll
-    for (int qb = 0; qb < NB; ++qb) at.l_run[qb] = l_tot[qb];
+        for (int qb = 0; qb < NB; ++qb) at.l_run[qb] = l_tot[qb];
+    }
     for (int w = wa; w <= wb; ++w) {
         const int64_t ws = split.first(w);
-        if (w == me || ws >= split.first(w + 1)) continue;
-#ifndef DFX_DBG_NO_MERGE
+        if ((w == me && !from_memory) || ws >= split.first(w + 1)) continue;
         at.merge_partial(partial_slot(w, ws > item_begin ? ws : item_begin, ws));
-#endif
     }
+    (void)stored;
     float l_all[NB];
 #pragma unroll
     for (int qb = 0; qb < NB; ++qb) l_all[qb] = at.l_run[qb];

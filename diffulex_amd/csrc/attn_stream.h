@@ -50,7 +50,13 @@ struct BandDesc {
 };
 enum : int32_t { kUnitCtx = 1, kUnitFirst = 2, kUnitLast = 4, kUnitComplete = 8 };
 
-template <int HD, int NB, int NW>
+// COMPACT: a configuration small enough (2 stages, short plan, at most kCompactMaxSeqs sequences)
+// for two workgroups to share a compute unit.  Items with at most 128 rows run with four waves,
+// one per SIMD, which then does nothing while its wave waits for LDS, for the issue of a load or
+// at the barrier; a second, independent workgroup on the same SIMDs fills those gaps.
+constexpr int kCompactMaxSeqs = 1023;
+
+template <int HD, int NB, int NW, bool COMPACT = false>
 struct StreamCfg : Shape<HD, NB, NW> {
     using S = Shape<HD, NB, NW>;
     static constexpr int ROWB = HD * 2;               // bytes per token row
@@ -58,19 +64,20 @@ struct StreamCfg : Shape<HD, NB, NW> {
     static constexpr int RPI = 1024 / ROWB;           // rows one wave-wide load covers
     static constexpr int MAT_BYTES = S::TN * ROWB;    // K (or V) tile
     static constexpr int STAGE_BYTES = 2 * MAT_BYTES;
-    static constexpr int kStages = 4;
+    static constexpr int kStages = COMPACT ? 2 : 4;
     static constexpr int IPW = MAT_BYTES / 1024 / NW;  // loads per wave per matrix per tile
     static constexpr int LOADS_PER_UNIT = 2 * IPW;
     static constexpr int ROWS_PER_WAVE = IPW * RPI;        // 16 (4 waves) or 8 (8 waves)
-    static constexpr int kPlanUnits = 512 / NW;            // units planned (and then streamed) at a time
+    static constexpr int kPlanUnits = COMPACT ? 32 : 512 / NW;  // units planned (and then streamed) at a time
+    static constexpr int PREFIX_BYTES = COMPACT ? (kCompactMaxSeqs + 1) * 4 : S::PREFIX_BYTES;
     static constexpr int UNIT_TABLE_BYTES = kPlanUnits * static_cast<int>(sizeof(UnitDesc));
     static constexpr int BAND_TABLE_BYTES = kPlanUnits * NW * static_cast<int>(sizeof(BandDesc));
-    static constexpr int UNIT_TABLE_OFF = S::PREFIX_BYTES + S::MISC_BYTES;
+    static constexpr int UNIT_TABLE_OFF = PREFIX_BYTES + S::MISC_BYTES;
     static constexpr int BAND_TABLE_OFF = UNIT_TABLE_OFF + UNIT_TABLE_BYTES;
     static constexpr int STAGES_OFF = BAND_TABLE_OFF + BAND_TABLE_BYTES;
     static constexpr int LDS_BYTES = STAGES_OFF + kStages * STAGE_BYTES;
     static_assert(ROWS_PER_WAVE * NW == S::TN && IPW >= 1, "the waves' row bands tile the 64 rows");
-    static_assert(LDS_BYTES <= 160 * 1024, "LDS budget of a gfx950 compute unit");
+    static_assert(LDS_BYTES <= (COMPACT ? 80 : 160) * 1024, "LDS budget of a gfx950 compute unit");
 
     // chunk position = chunk index ^ swizzle(row); 16 consecutive rows of one chunk column hit
     // 16 different 16-byte bank groups (the LDS has 64 banks)
@@ -121,10 +128,10 @@ DFX_D void mfma_outputs_ready(f32x16& x0, f32x16& x1, f32x16& x2, f32x16& x3) {
     asm volatile("s_nop 15\n\ts_nop 1" : "+a"(x0), "+a"(x1), "+a"(x2), "+a"(x3));
 }
 
-template <int HD, int NB, int NW>
+template <int HD, int NB, int NW, bool COMPACT = false>
 struct StreamAttn : AttnState<HD, NB, NW> {
     using Base = AttnState<HD, NB, NW>;
-    using C = StreamCfg<HD, NB, NW>;
+    using C = StreamCfg<HD, NB, NW, COMPACT>;
     using Base::a;
     using Base::col;
     using Base::half;
@@ -335,11 +342,11 @@ struct StreamAttn : AttnState<HD, NB, NW> {
     }
 };
 
-template <int HD, int NB, int NW>
-__global__ void __launch_bounds__(64 * NW) paged_attn_stream_kernel(const KArgs a) {
+template <int HD, int NB, int NW, bool COMPACT>
+__global__ void __launch_bounds__(64 * NW, COMPACT ? 2 : 1) paged_attn_stream_kernel(const KArgs a) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-    using C = StreamCfg<HD, NB, NW>;
-    StreamAttn<HD, NB, NW> at(a, smem);
+    using C = StreamCfg<HD, NB, NW, COMPACT>;
+    StreamAttn<HD, NB, NW, COMPACT> at(a, smem);
     at.per_head = build_unit_prefix<C::RT>(a, at.prefix, at.misc);
     const int64_t total = static_cast<int64_t>(at.per_head) * a.h_kv;
     if (total == 0) return;

@@ -15,10 +15,13 @@
 namespace dfx {
 namespace {
 
+constexpr int kMaxWorkgroups = 65535;
+
 struct Plan {
     int hd, nb, n_wg;
     bool fp8;
-    bool stream;  // streaming tile path (else generic)
+    bool stream;   // streaming tile path (else generic)
+    bool compact;  // streaming path, two workgroups per compute unit
     int64_t slot_floats;
 };
 
@@ -49,21 +52,25 @@ int make_plan(const dfx_attn_params* p, Plan& plan) {
     plan.fp8 = p->kv_dtype == DFX_KV_FP8_E4M3 && p->k_cache != nullptr;
     plan.stream = !plan.fp8 && !(p->flags & DFX_ATTN_GENERIC_PATH) &&
                   (p->k_cache == nullptr || (p->page_size > 0 && p->page_size % 16 == 0));
+    plan.compact = plan.stream && plan.nb == 1 && p->num_seqs <= kCompactMaxSeqs;
     if (p->max_workgroups > 0) {
         plan.n_wg = p->max_workgroups;
     } else {
         plan.n_wg = device_cu_count();
         if (plan.n_wg <= 0) return DFX_ERR_LAUNCH;
+        if (plan.compact) plan.n_wg *= 2;
     }
-    if (plan.n_wg > 65535) return DFX_ERR_INVALID_ARG;
+    if (plan.n_wg > kMaxWorkgroups) return DFX_ERR_INVALID_ARG;
     if (plan.hd == 64) plan.slot_floats = plan.nb == 1 ? Shape<64, 1>::SLOT_FLOATS : Shape<64, 2>::SLOT_FLOATS;
     else plan.slot_floats = plan.nb == 1 ? Shape<128, 1>::SLOT_FLOATS : Shape<128, 2>::SLOT_FLOATS;
     return DFX_OK;
 }
 
-// Workspace layout: arrival counters (one int per workgroup, rounded up to 256 bytes), then two
-// partial-result slots per workgroup.
-int64_t counter_bytes(const Plan& plan) { return (static_cast<int64_t>(plan.n_wg) * 4 + 255) / 256 * 256; }
+// Workspace layout: arrival counters (one int per workgroup), then two partial-result slots per
+// workgroup.  The counter area has the same size whatever the launch (room for the largest
+// grid): calls with different workgroup counts may share a workspace, and the counters must
+// never land where an earlier call left partial results.
+int64_t counter_bytes(const Plan&) { return (static_cast<int64_t>(kMaxWorkgroups) + 1) * 4; }
 int64_t plan_workspace_bytes(const Plan& plan) {
     return counter_bytes(plan) + 2 * static_cast<int64_t>(plan.n_wg) * plan.slot_floats * 4;
 }
@@ -77,19 +84,25 @@ int launch(const KArgs& ka, const Plan& plan, hipStream_t st) {
         // the streaming path gives every wave one 32-row query block: 4 waves for up to 128 rows,
         // 8 waves (two per SIMD, so one wave's softmax overlaps the other's matrix work) for 256
         constexpr int NW = 4 * NB;
-        main_k = paged_attn_stream_kernel<HD, 1, NW>;
-        lds = StreamCfg<HD, 1, NW>::LDS_BYTES;
+        if (NB == 1 && plan.compact) {
+            main_k = paged_attn_stream_kernel<HD, 1, 4, true>;
+            lds = StreamCfg<HD, 1, 4, true>::LDS_BYTES;
+        } else {
+            main_k = paged_attn_stream_kernel<HD, 1, NW, false>;
+            lds = StreamCfg<HD, 1, NW, false>::LDS_BYTES;
+        }
         threads = 64 * NW;
     } else {
         main_k = paged_attn_generic_kernel<HD, NB, PATH == 1>;
         lds = GenericCfg<HD, NB>::LDS_BYTES;
     }
-    static bool configured = false;  // raising the dynamic LDS limit is idempotent
-    if (!configured) {
+    static bool configured[2] = {false, false};  // raising the dynamic LDS limit is idempotent
+    bool& done = configured[plan.compact ? 1 : 0];
+    if (!done) {
         if (hipFuncSetAttribute(reinterpret_cast<const void*>(main_k), hipFuncAttributeMaxDynamicSharedMemorySize,
                                 lds) != hipSuccess)
             return DFX_ERR_LAUNCH;
-        configured = true;
+        done = true;
     }
     hipLaunchKernelGGL(main_k, dim3(plan.n_wg), dim3(threads), lds, st, ka);
     if (hipGetLastError() != hipSuccess) return DFX_ERR_LAUNCH;

@@ -31,7 +31,7 @@ HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this command, scaled by
 # what the same counters read for a plain copy of known size (profiles/paged_attn_stream_kernel_c3.md).
-MEASURED_TRAFFIC_BYTES = {"c3": 283.4e6}
+MEASURED_TRAFFIC_BYTES = {"c3": 291.5e6}
 
 
 def algorithmic_bytes(wl) -> int:

@@ -1,25 +1,26 @@
 // Generic tile path of the paged-attention kernel: any page size, bf16 or FP8-E4M3 cache.
 //
-// A 64-token tile goes global --16-byte loads--> registers --> LDS, K as [token][d] rows with
-// a 16-byte skew, V transposed to [d][token] (2-byte LDS stores) with the token order the PV
-// product wants.  FP8 codes are widened to bf16 on the way into LDS (the widening is exact),
-// so the MFMA loop is the same for both cache types; the per-head scales are folded into the
-// softmax constants.  One tile is staged in registers while the previous one is computed.
+// A 64-token tile goes global --16-byte loads--> registers --> LDS, K and V in the swizzled
+// row-major layout of attn_tile.h, so the matrix and softmax arithmetic is the one the streaming
+// path uses.  FP8 codes are widened to bf16 on the way into LDS (the widening is exact), so the
+// arithmetic is the same for both cache types; the per-head scales are folded into the softmax
+// constants.  One tile is staged in registers while the previous one is computed.
 #pragma once
 
-#include "attn_common.h"
+#include "attn_tile.h"
 
 namespace dfx {
 
 template <int HD, int NB>
 struct GenericCfg : Shape<HD, NB> {
     using S = Shape<HD, NB>;
-    static constexpr int KSTRIDE = HD * 2 + 16;     // bytes per K row in LDS
-    static constexpr int VSTRIDE = S::TN * 2 + 16;  // bytes per V^T row in LDS
-    static constexpr int K_BYTES = S::TN * KSTRIDE;
-    static constexpr int V_BYTES = HD * VSTRIDE;
-    static constexpr int STAGE_BYTES = K_BYTES + V_BYTES;
-    static constexpr int LDS_BYTES = S::PREFIX_BYTES + S::MISC_BYTES + 2 * STAGE_BYTES;
+    static constexpr int K_BYTES = TileLayout<HD>::MAT_BYTES;
+    static constexpr int STAGE_BYTES = 2 * K_BYTES;  // K tile, V tile
+    // the block-table entries of the piece of an item being processed, so that the tile loop
+    // does not chase a table entry in global memory before every row it loads
+    static constexpr int kTableEntries = 4096;
+    static constexpr int TABLE_OFF = S::PREFIX_BYTES + S::MISC_BYTES + 2 * STAGE_BYTES;
+    static constexpr int LDS_BYTES = TABLE_OFF + kTableEntries * 4;
     static constexpr int CH16 = S::TN * HD * 2 / 16 / kThreads;  // 16-byte chunks per lane, bf16 tile
     static constexpr int CH8 = S::TN * HD / 16 / kThreads;       // 16-byte chunks per lane, fp8 tile
 };
@@ -32,14 +33,10 @@ DFX_D uint32_t fp8x2_to_bf16x2(uint32_t w) {
     return (__float_as_uint(f.x) >> 16) | (__float_as_uint(f.y) & 0xffff0000u);
 }
 
-// Position of token row r inside a V^T row: within every 16 tokens the 4-token groups
-// (0,1,2,3) are stored in the order (0,2,1,3), so that the eight contraction elements a
-// lane of half h needs for one MFMA, tokens {4h..4h+3} and {8+4h..8+4h+3}, are contiguous.
-DFX_D int vt_pos(int r) { return (r & ~12) | ((r & 4) << 1) | ((r & 8) >> 1); }
-
 template <int HD, int NB, bool FP8>
-struct GenericAttn : AttnState<HD, NB> {
-    using Base = AttnState<HD, NB>;
+struct GenericAttn : TileMath<HD, NB, kWaves> {
+    using Base = TileMath<HD, NB, kWaves>;
+    using L = TileLayout<HD>;
     using C = GenericCfg<HD, NB>;
     using Base::a;
     using Base::col;
@@ -55,12 +52,33 @@ struct GenericAttn : AttnState<HD, NB> {
     uint8_t* lds;
     int* prefix;
     int* misc;
+    int* table;        // block-table entries [table_p0, table_p0 + table_n) of sequence s, if table_n > 0
+    int table_p0, table_n;
     u32x4 kst[C::CH16], vst[C::CH16];
     bool staged_fp8;
 
     DFX_D GenericAttn(const KArgs& args, uint8_t* smem)
         : Base(args), lds(smem), prefix(reinterpret_cast<int*>(smem)),
-          misc(reinterpret_cast<int*>(smem + C::PREFIX_BYTES)) {}
+          misc(reinterpret_cast<int*>(smem + C::PREFIX_BYTES)), table(reinterpret_cast<int*>(smem + C::TABLE_OFF)),
+          table_p0(0), table_n(0) {}
+
+    // Copy the block-table entries that tiles [tile0, tile1) of the current sequence need into LDS
+    // (skipped, and looked up in global memory instead, if they do not fit).  The caller's
+    // barrier makes them visible.
+    DFX_D void cache_block_table(int tile0, int tile1) {
+        table_n = 0;
+        const int tok0 = tile0 * C::TN;
+        const int tok1 = min(tile1 * C::TN, sh.ctx);
+        if (tok1 <= tok0) return;
+        const int p0 = tok0 / a.page_size, p1 = (tok1 - 1) / a.page_size;
+        if (p1 - p0 + 1 > C::kTableEntries) return;
+        table_p0 = p0;
+        table_n = p1 - p0 + 1;
+        for (int i = tid; i < table_n; i += kThreads) {
+            const int p = p0 + i;
+            table[i] = p < a.max_pages ? a.block_tables[static_cast<int64_t>(s) * a.bt_stride + p] : -1;
+        }
+    }
 
     DFX_D uint8_t* k_stage(int b) const { return lds + C::PREFIX_BYTES + C::MISC_BYTES + b * C::STAGE_BYTES; }
     DFX_D uint8_t* v_stage(int b) const { return k_stage(b) + C::K_BYTES; }
@@ -69,7 +87,8 @@ struct GenericAttn : AttnState<HD, NB> {
         const int p = a.page_shift >= 0 ? (tok >> a.page_shift) : (tok / a.page_size);
         const int off = tok - p * a.page_size;
         int64_t page = -1;
-        if (p < a.max_pages) page = a.block_tables[static_cast<int64_t>(s) * a.bt_stride + p];
+        if (table_n > 0) page = table[p - table_p0];
+        else if (p < a.max_pages) page = a.block_tables[static_cast<int64_t>(s) * a.bt_stride + p];
         ok = ok && page >= 0 && page < a.n_pages;
         return page * a.c_sp + off * a.c_st + kvh * a.c_sh;
     }
@@ -128,19 +147,6 @@ struct GenericAttn : AttnState<HD, NB> {
         }
     }
 
-    DFX_D void put_v8(uint8_t* vs, int d0, int row, u32x4 v) const {
-        uint16_t* base = reinterpret_cast<uint16_t*>(vs + d0 * C::VSTRIDE) + vt_pos(row);
-        constexpr int RS = C::VSTRIDE / 2;
-        base[0 * RS] = static_cast<uint16_t>(v.x);
-        base[1 * RS] = static_cast<uint16_t>(v.x >> 16);
-        base[2 * RS] = static_cast<uint16_t>(v.y);
-        base[3 * RS] = static_cast<uint16_t>(v.y >> 16);
-        base[4 * RS] = static_cast<uint16_t>(v.z);
-        base[5 * RS] = static_cast<uint16_t>(v.z >> 16);
-        base[6 * RS] = static_cast<uint16_t>(v.w);
-        base[7 * RS] = static_cast<uint16_t>(v.w >> 16);
-    }
-
     DFX_D static void widen16(u32x4 codes, u32x4& lo, u32x4& hi) {
         lo = u32x4{fp8x2_to_bf16x2<false>(codes.x), fp8x2_to_bf16x2<true>(codes.x),
                    fp8x2_to_bf16x2<false>(codes.y), fp8x2_to_bf16x2<true>(codes.y)};
@@ -153,19 +159,18 @@ struct GenericAttn : AttnState<HD, NB> {
         uint8_t* ks = k_stage(buf);
         uint8_t* vs = v_stage(buf);
         if (FP8 && staged_fp8) {
-            constexpr int CPR = HD / 16;
+            constexpr int CPR = HD / 16;  // 16-code chunks per row, each widening to two bf16 chunks
 #pragma unroll
             for (int i = 0; i < C::CH8; ++i) {
                 const int c = tid + kThreads * i;
                 const int row = c / CPR, cc = c % CPR;
                 u32x4 lo, hi;
                 widen16(kst[i], lo, hi);
-                u32x4* kd = reinterpret_cast<u32x4*>(ks + row * C::KSTRIDE + cc * 32);
-                kd[0] = lo;
-                kd[1] = hi;
+                *reinterpret_cast<u32x4*>(ks + L::chunk_offset(row, 2 * cc)) = lo;
+                *reinterpret_cast<u32x4*>(ks + L::chunk_offset(row, 2 * cc + 1)) = hi;
                 widen16(vst[i], lo, hi);
-                put_v8(vs, cc * 16, row, lo);
-                put_v8(vs, cc * 16 + 8, row, hi);
+                *reinterpret_cast<u32x4*>(vs + L::chunk_offset(row, 2 * cc)) = lo;
+                *reinterpret_cast<u32x4*>(vs + L::chunk_offset(row, 2 * cc + 1)) = hi;
             }
         } else {
             constexpr int CPR = HD / 8;
@@ -173,8 +178,8 @@ struct GenericAttn : AttnState<HD, NB> {
             for (int i = 0; i < C::CH16; ++i) {
                 const int c = tid + kThreads * i;
                 const int row = c / CPR, cc = c % CPR;
-                *reinterpret_cast<u32x4*>(ks + row * C::KSTRIDE + cc * 16) = kst[i];
-                put_v8(vs, cc * 8, row, vst[i]);
+                *reinterpret_cast<u32x4*>(ks + L::chunk_offset(row, cc)) = kst[i];
+                *reinterpret_cast<u32x4*>(vs + L::chunk_offset(row, cc)) = vst[i];
             }
         }
     }
@@ -182,53 +187,19 @@ struct GenericAttn : AttnState<HD, NB> {
     // one tile of attention from LDS
     DFX_D void compute(int buf, int tile) {
         const TileInfo t = this->tile_info(sh, kvh, tile, FP8);
-        const uint8_t* ks = k_stage(buf);
-        const uint8_t* vs = v_stage(buf);
-
         f32x16 sc[2][NB];
-#pragma unroll
-        for (int tb = 0; tb < 2; ++tb)
-#pragma unroll
-            for (int qb = 0; qb < NB; ++qb)
-#pragma unroll
-                for (int e = 0; e < 16; ++e) sc[tb][qb][e] = 0.0f;
-
-        const uint8_t* krow = ks + col * C::KSTRIDE + half * 16;
-#pragma unroll
-        for (int slab = 0; slab < C::NSLAB; ++slab) {
-            bf16x8 ka[2];
-#pragma unroll
-            for (int tb = 0; tb < 2; ++tb)
-                ka[tb] = *reinterpret_cast<const bf16x8*>(krow + tb * 32 * C::KSTRIDE + slab * 32);
-#pragma unroll
-            for (int tb = 0; tb < 2; ++tb)
-#pragma unroll
-                for (int qb = 0; qb < NB; ++qb)
-                    sc[tb][qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[tb], qf[qb][slab], sc[tb][qb], 0, 0, 0);
-        }
-
+        this->scores(k_stage(buf), sc);
         bf16x8 pb[NB][2][2];
-        this->template softmax_tile<FP8>(sc, t, pb, [] {});
-
-        const uint8_t* vrow = vs + col * C::VSTRIDE + half * 16;
-#pragma unroll
-        for (int tb = 0; tb < 2; ++tb)
-#pragma unroll
-            for (int sl = 0; sl < 2; ++sl)
-#pragma unroll
-                for (int db = 0; db < C::NDB; ++db) {
-                    const bf16x8 va =
-                        *reinterpret_cast<const bf16x8*>(vrow + db * 32 * C::VSTRIDE + (tb * 32 + sl * 16) * 2);
-#pragma unroll
-                    for (int qb = 0; qb < NB; ++qb)
-                        o[db][qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, pb[qb][tb][sl], o[db][qb], 0, 0, 0);
-                }
+        this->template softmax_tile<FP8>(sc, t, pb, [&] { this->outputs_ready(); });
+        this->accumulate(v_stage(buf), pb);
     }
 
     DFX_D void run_segment(int rt, int tile0, int tile1, int64_t item_begin, const WgSplit& split, int slot) {
         const bool complete = tile0 == 0 && tile1 == this->sh.n_tiles;
         this->load_queries(rt);
-        __syncthreads();  // the previous segment's last tile may still be read from LDS
+        __syncthreads();  // the previous segment's last tile and block-table entries may still be read from LDS
+        cache_block_table(tile0, tile1);
+        __syncthreads();
         int buf = 0;
         issue(tile0);
         for (int t = tile0; t < tile1; ++t) {
@@ -238,6 +209,7 @@ struct GenericAttn : AttnState<HD, NB> {
             compute(buf, t);
             buf ^= 1;
         }
+        this->outputs_ready();
         float l_tot[NB];
         this->row_sums(l_tot);
         if (complete) this->store_output(rt, l_tot);

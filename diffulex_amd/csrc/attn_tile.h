@@ -1,0 +1,158 @@
+// Tile arithmetic shared by the paged-attention kernels: the LDS layout of a K or V tile, the
+// matrix-instruction helpers, and S^T = K Q^T / O^T += V^T P^T on tiles in that layout.
+//
+// LDS tile layout: row-major [token][head_dim] as in the cache, with the 16-byte chunks of a
+// row XOR-swizzled by the row index.
+//   K operand (A of S^T = K Q^T): ds_read_b128 of chunk (2*slab + h) of row (lane % 32).
+//   V operand (A of O^T += V^T P^T): needs 8 tokens of one d per lane, i.e. a column of the
+//     tile.  ds_read_b64_tr_b16 transposes inside groups of 16 lanes: lane i of a group
+//     receives element (i % 4) of what lanes {i/4, 4 + i/4, 8 + i/4, 12 + i/4} of the group
+//     addressed.  Source lane s therefore points at token row (s / 4), elements 4*(s % 4)..+3
+//     of a 16-wide d range, and lane i ends up with 4 consecutive tokens of d = i.
+#pragma once
+
+#include "attn_common.h"
+
+namespace dfx {
+
+DFX_D int uniform(int v) { return __builtin_amdgcn_readfirstlane(v); }
+
+template <int HD>
+struct TileLayout {
+    static constexpr int ROWB = HD * 2;                   // bytes per token row
+    static constexpr int CPR = ROWB / 16;                 // 16-byte chunks per row
+    static constexpr int MAT_BYTES = kTileTokens * ROWB;  // one K (or V) tile
+    // chunk position = chunk index ^ swizzle(row); 16 consecutive rows of one chunk column hit
+    // 16 different 16-byte bank groups (the LDS has 64 banks)
+    DFX_HD static int swizzle(int row) { return HD == 128 ? (row & 15) : ((row >> 1) & 7); }
+    // byte offset of 16-byte chunk c of token row r inside a tile
+    DFX_HD static int chunk_offset(int r, int c) { return r * ROWB + ((c ^ swizzle(r)) * 16); }
+};
+
+// The matrix instructions of the tile loop are issued from inline assembly so that the register
+// file split is fixed by their operand constraints: the O^T accumulators live in the accumulation
+// registers, which only matrix instructions touch in the loop, and the score accumulators in
+// ordinary vector registers, where the softmax works on them in place.  Being volatile they keep
+// their program order: an accumulator is reused every 4th (scores) or 8th (output) instruction,
+// far beyond the result latency.  What the compiler can no longer do for them is insert the wait
+// states the ISA requires around matrix instructions: each one is therefore preceded by two wait
+// states (a vector-ALU result may feed it), and mfma_results_ready() / mfma_outputs_ready() put
+// 18 wait states, the longest the ISA asks for, between a matrix result and a vector-ALU reader.
+DFX_D void mfma_scores_first(f32x16& sc, bf16x8 k, bf16x8 q) {
+    asm volatile("s_nop 1\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(sc) : "v"(k), "v"(q));
+}
+DFX_D void mfma_scores(f32x16& sc, bf16x8 k, bf16x8 q) {
+    asm volatile("s_nop 1\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(sc) : "v"(k), "v"(q));
+}
+DFX_D void mfma_output(f32x16& acc, bf16x8 v, bf16x8 p) {
+    asm volatile("s_nop 1\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(acc) : "v"(v), "v"(p));
+}
+DFX_D void mfma_results_ready(f32x16& x0, f32x16& x1, f32x16& x2, f32x16& x3) {
+    asm volatile("s_nop 15\n\ts_nop 1" : "+v"(x0), "+v"(x1), "+v"(x2), "+v"(x3));
+}
+DFX_D void mfma_results_ready(f32x16& x0, f32x16& x1) {
+    asm volatile("s_nop 15\n\ts_nop 1" : "+v"(x0), "+v"(x1));
+}
+DFX_D void mfma_outputs_ready(f32x16& x0, f32x16& x1, f32x16& x2, f32x16& x3) {
+    asm volatile("s_nop 15\n\ts_nop 1" : "+a"(x0), "+a"(x1), "+a"(x2), "+a"(x3));
+}
+DFX_D void mfma_outputs_ready(f32x16& x0, f32x16& x1) {
+    asm volatile("s_nop 15\n\ts_nop 1" : "+a"(x0), "+a"(x1));
+}
+
+template <int HD, int NB, int NW>
+struct TileMath : AttnState<HD, NB, NW> {
+    using Base = AttnState<HD, NB, NW>;
+    using S = Shape<HD, NB, NW>;
+    using L = TileLayout<HD>;
+    using Base::col;
+    using Base::half;
+    using Base::lane;
+    using Base::o;
+    using Base::qf;
+
+    DFX_D explicit TileMath(const KArgs& args) : Base(args) {}
+
+    // ---- tile arithmetic -------------------------------------------------------------------
+    DFX_D bf16x8 read_k(const uint8_t* k_tile, int tb, int slab) const {
+        const int row = tb * 32 + col;
+        const int pos = (2 * slab + half) ^ L::swizzle(row);
+        return *reinterpret_cast<const bf16x8*>(k_tile + row * L::ROWB + pos * 16);
+    }
+
+    // V^T operand for token slab (tb, sl) and d block db.
+    DFX_D bf16x8 read_vt(const uint8_t* v_tile, int tb, int sl, int db) const {
+        typedef short short4v __attribute__((ext_vector_type(4)));
+        typedef short short8v __attribute__((ext_vector_type(8)));
+        typedef __attribute__((address_space(3))) short4v lds_short4v;
+        const int g16 = lane >> 4, sl16 = lane & 15;
+        short4v r[2];
+#pragma unroll
+        for (int ii = 0; ii < 2; ++ii) {
+            const int row = tb * 32 + sl * 16 + ii * 8 + (g16 >> 1) * 4 + (sl16 >> 2);
+            const int chunk = db * 4 + (g16 & 1) * 2 + ((sl16 & 3) >> 1);
+            const int pos = chunk ^ L::swizzle(row);
+            const uint8_t* p = v_tile + row * L::ROWB + pos * 16 + (sl16 & 1) * 8;
+            r[ii] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4v*)(p));
+        }
+        const short8v v = __builtin_shufflevector(r[0], r[1], 0, 1, 2, 3, 4, 5, 6, 7);
+        return __builtin_bit_cast(bf16x8, v);
+    }
+
+    // The LDS operands of the next step are requested before the matrix instructions of the
+    // current one: being volatile assembly those pin the order, so the LDS latency is hidden
+    // only by what the source puts in between.
+    DFX_D void scores(const uint8_t* k_tile, f32x16 (&sc)[2][NB]) const {
+        bf16x8 ka[2][2];
+#pragma unroll
+        for (int tb = 0; tb < 2; ++tb) ka[0][tb] = read_k(k_tile, tb, 0);
+#pragma unroll
+        for (int slab = 0; slab < S::NSLAB; ++slab) {
+            if (slab + 1 < S::NSLAB) {
+#pragma unroll
+                for (int tb = 0; tb < 2; ++tb) ka[(slab + 1) & 1][tb] = read_k(k_tile, tb, slab + 1);
+            }
+#pragma unroll
+            for (int tb = 0; tb < 2; ++tb)
+#pragma unroll
+                for (int qb = 0; qb < NB; ++qb) {
+                    if (slab == 0) mfma_scores_first(sc[tb][qb], ka[slab & 1][tb], qf[qb][slab]);
+                    else mfma_scores(sc[tb][qb], ka[slab & 1][tb], qf[qb][slab]);
+                }
+        }
+        if constexpr (NB == 2) mfma_results_ready(sc[0][0], sc[0][1], sc[1][0], sc[1][1]);
+        else mfma_results_ready(sc[0][0], sc[1][0]);
+    }
+
+    // Wait states before vector instructions read the O^T accumulators (rescale, epilogue).
+    DFX_D void outputs_ready() {
+#pragma unroll
+        for (int qb = 0; qb < NB; ++qb) {
+            if constexpr (S::NDB == 4) mfma_outputs_ready(o[0][qb], o[1][qb], o[2][qb], o[3][qb]);
+            else mfma_outputs_ready(o[0][qb], o[1][qb]);  // (never one accumulator twice: the second would be a copy,
+                                                          //  made before the wait states)
+        }
+    }
+
+    DFX_D void accumulate(const uint8_t* v_tile, const bf16x8 (&pb)[NB][2][2]) {
+        constexpr int kSteps = 4 * S::NDB;  // (tb, sl, db)
+        bf16x8 va[3];
+        va[0] = read_vt(v_tile, 0, 0, 0);
+        va[1] = read_vt(v_tile, 0, 0, 1);
+#pragma unroll
+        for (int st = 0; st < kSteps; ++st) {
+            const int tb = st / (2 * S::NDB), sl = (st / S::NDB) & 1, db = st % S::NDB;
+            if (st + 2 < kSteps) {
+                const int n = st + 2;
+                va[n % 3] = read_vt(v_tile, n / (2 * S::NDB), (n / S::NDB) & 1, n % S::NDB);
+            }
+#pragma unroll
+            for (int qb = 0; qb < NB; ++qb) mfma_output(o[db][qb], va[st % 3], pb[qb][tb][sl]);
+        }
+        // the compiler may move the accumulators to other registers right behind this stream
+        outputs_ready();
+    }
+
+};
+
+}  // namespace dfx

@@ -25,14 +25,6 @@ struct GenericCfg : Shape<HD, NB> {
     static constexpr int CH8 = S::TN * HD / 16 / kThreads;       // 16-byte chunks per lane, fp8 tile
 };
 
-// Two e4m3 codes (bytes 0,1 or 2,3 of w) -> two bf16 packed in a dword.  An e4m3 value has 3
-// mantissa bits, so the upper half of its fp32 form is its bf16 form.
-template <bool HI>
-DFX_D uint32_t fp8x2_to_bf16x2(uint32_t w) {
-    const f32x2 f = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(w), HI);
-    return (__float_as_uint(f.x) >> 16) | (__float_as_uint(f.y) & 0xffff0000u);
-}
-
 template <int HD, int NB, bool FP8>
 struct GenericAttn : TileMath<HD, NB, kWaves> {
     using Base = TileMath<HD, NB, kWaves>;
@@ -145,13 +137,6 @@ struct GenericAttn : TileMath<HD, NB, kWaves> {
                 vst[i] = vv;
             }
         }
-    }
-
-    DFX_D static void widen16(u32x4 codes, u32x4& lo, u32x4& hi) {
-        lo = u32x4{fp8x2_to_bf16x2<false>(codes.x), fp8x2_to_bf16x2<true>(codes.x),
-                   fp8x2_to_bf16x2<false>(codes.y), fp8x2_to_bf16x2<true>(codes.y)};
-        hi = u32x4{fp8x2_to_bf16x2<false>(codes.z), fp8x2_to_bf16x2<true>(codes.z),
-                   fp8x2_to_bf16x2<false>(codes.w), fp8x2_to_bf16x2<true>(codes.w)};
     }
 
     // registers -> LDS

@@ -49,10 +49,14 @@ enum : int32_t { kUnitCtx = 1, kUnitFirst = 2, kUnitLast = 4, kUnitComplete = 8 
 // at the barrier; a second, independent workgroup on the same SIMDs fills those gaps.
 constexpr int kCompactMaxSeqs = 1023;
 
-template <int HD, int NB, int NW, bool COMPACT = false>
+//
+// KVB: bytes per cache element.  With FP8 codes (KVB == 1) a ring stage holds the tile as stored,
+// and each wave widens the rows it loaded itself into one of two bf16 tiles in the layout of
+// attn_tile.h one step before the matrix instructions read them (see the FP8 kernel below).
+template <int HD, int NB, int NW, bool COMPACT = false, int KVB = 2>
 struct StreamCfg : Shape<HD, NB, NW> {
     using S = Shape<HD, NB, NW>;
-    static constexpr int ROWB = HD * 2;               // bytes per token row
+    static constexpr int ROWB = HD * KVB;             // bytes per token row as loaded
     static constexpr int CPR = ROWB / 16;             // 16-byte chunks per row
     static constexpr int RPI = 1024 / ROWB;           // rows one wave-wide load covers
     static constexpr int MAT_BYTES = S::TN * ROWB;    // K (or V) tile
@@ -68,11 +72,15 @@ struct StreamCfg : Shape<HD, NB, NW> {
     static constexpr int UNIT_TABLE_OFF = PREFIX_BYTES + S::MISC_BYTES;
     static constexpr int BAND_TABLE_OFF = UNIT_TABLE_OFF + UNIT_TABLE_BYTES;
     static constexpr int STAGES_OFF = BAND_TABLE_OFF + BAND_TABLE_BYTES;
-    static constexpr int LDS_BYTES = STAGES_OFF + kStages * STAGE_BYTES;
+    static constexpr int WIDE_OFF = STAGES_OFF + kStages * STAGE_BYTES;
+    static constexpr int WIDE_BYTES = 2 * TileLayout<HD>::MAT_BYTES;  // widened K tile, widened V tile
+    static constexpr int LDS_BYTES = WIDE_OFF + (KVB == 1 ? 2 * WIDE_BYTES : 0);
+    static_assert(KVB == 2 || (KVB == 1 && !COMPACT), "bf16 or FP8 codes");
     static_assert(ROWS_PER_WAVE * NW == S::TN && IPW >= 1, "the waves' row bands tile the 64 rows");
     static_assert(LDS_BYTES <= (COMPACT ? 80 : 160) * 1024, "LDS budget of a gfx950 compute unit");
 
-    DFX_HD static int swizzle(int row) { return TileLayout<HD>::swizzle(row); }
+    // FP8 stages are read back by the lanes that loaded them, in load order: no swizzle needed
+    DFX_HD static int swizzle(int row) { return KVB == 2 ? TileLayout<HD>::swizzle(row) : 0; }
 };
 
 // One wave-wide 16-byte-per-lane direct-to-LDS load from base + voff; lane i's data lands at
@@ -89,10 +97,11 @@ DFX_D void wait_async_loads() {
     asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
 }
 
-template <int HD, int NB, int NW, bool COMPACT = false>
+template <int HD, int NB, int NW, bool COMPACT = false, int KVB = 2>
 struct StreamAttn : TileMath<HD, NB, NW> {
     using Base = TileMath<HD, NB, NW>;
-    using C = StreamCfg<HD, NB, NW, COMPACT>;
+    using C = StreamCfg<HD, NB, NW, COMPACT, KVB>;
+    using L = TileLayout<HD>;
     using Base::a;
     using Base::col;
     using Base::half;
@@ -110,6 +119,7 @@ struct StreamAttn : TileMath<HD, NB, NW> {
     uint32_t stages_lds;  // LDS byte address of stage 0
     int64_t begin, end;
     int per_head;
+    float k_mul, v_mul;  // the current item's FP8 scales
 
     DFX_D StreamAttn(const KArgs& args, uint8_t* smem)
         : Base(args), lds(smem), prefix(reinterpret_cast<int*>(smem)),
@@ -172,7 +182,7 @@ struct StreamAttn : TileMath<HD, NB, NW> {
                 const int p = a.page_shift >= 0 ? (band >> a.page_shift) : (band / a.page_size);
                 int64_t page = p < a.max_pages ? a.block_tables[static_cast<int64_t>(sq) * a.bt_stride + p] : 0;
                 page = page < 0 ? 0 : (page >= a.n_pages ? a.n_pages - 1 : page);
-                b.off = (page * a.c_sp + static_cast<int64_t>(band - p * a.page_size) * a.c_st + kv_head * a.c_sh) * 2;
+                b.off = (page * a.c_sp + static_cast<int64_t>(band - p * a.page_size) * a.c_st + kv_head * a.c_sh) * KVB;
             } else {
                 b.off = ((static_cast<int64_t>(a.cu_new[sq]) + band) * a.kn_st + kv_head * a.kn_sh) * 2;
             }
@@ -192,16 +202,72 @@ struct StreamAttn : TileMath<HD, NB, NW> {
                             static_cast<uint32_t>(uniform(static_cast<int>(b.off)));
         const uint8_t* kbase = (is_ctx ? a.k_cache : reinterpret_cast<const uint8_t*>(a.k_new)) + off;
         const uint8_t* vbase = (is_ctx ? a.v_cache : reinterpret_cast<const uint8_t*>(a.v_new)) + off;
-        const uint32_t row_stride = static_cast<uint32_t>(is_ctx ? a.c_st : a.kn_st) * 2u;
+        const uint32_t row_stride = static_cast<uint32_t>(is_ctx ? a.c_st * KVB : a.kn_st * 2);
         const uint32_t dst = stages_lds + (rel % C::kStages) * C::STAGE_BYTES + wave * (C::IPW * 1024);
 #pragma unroll
         for (int j = 0; j < C::IPW; ++j) {
             const int r = j * C::RPI + lane / C::CPR;  // row inside the band
             const int lds_row = wave * C::ROWS_PER_WAVE + r;
             const int chunk = (lane % C::CPR) ^ C::swizzle(lds_row);
-            const uint32_t voff = static_cast<uint32_t>(min(r, last)) * row_stride + chunk * 16;
+            uint32_t voff = static_cast<uint32_t>(min(r, last)) * row_stride + chunk * 16;
+            // Fresh rows are bf16 and are fetched by widen_unit() itself; the loads are issued all
+            // the same (every lane re-reads the band's first bytes) so that every unit advances
+            // the completion counter by the same amount.
+            if (KVB == 1 && !is_ctx) voff = 0;
             async_load16(kbase, voff, dst + j * 1024);
             async_load16(vbase, voff, dst + C::MAT_BYTES + j * 1024);
+        }
+    }
+
+    // FP8 only: bring unit `rel` into bf16 tile (rel & 1).  A wave widens the rows it loaded itself,
+    // so it only has to wait for its own loads; fresh rows (bf16 in memory) are copied from
+    // global memory here, once per item.
+    DFX_D uint8_t* wide_tile(int rel) const { return lds + C::WIDE_OFF + (rel & 1) * C::WIDE_BYTES; }
+    DFX_D void widen_unit(int rel) const {
+        const BandDesc b = bands[rel * NW + wave];
+        const bool is_ctx = uniform(b.is_ctx) != 0;
+        uint8_t* kt = wide_tile(rel);
+        uint8_t* vt = kt + L::MAT_BYTES;
+        const uint8_t* raw = lds + C::STAGES_OFF + (rel % C::kStages) * C::STAGE_BYTES + wave * (C::IPW * 1024) + lane * 16;
+        if (is_ctx) {
+#pragma unroll
+            for (int j = 0; j < C::IPW; ++j) {
+                const int row = wave * C::ROWS_PER_WAVE + j * C::RPI + lane / C::CPR;
+                const int cc = lane % C::CPR;
+                const u32x4 kc = *reinterpret_cast<const u32x4*>(raw + j * 1024);
+                const u32x4 vc = *reinterpret_cast<const u32x4*>(raw + C::MAT_BYTES + j * 1024);
+                u32x4 lo, hi;
+                widen16(kc, lo, hi);
+                *reinterpret_cast<u32x4*>(kt + L::chunk_offset(row, 2 * cc)) = lo;
+                *reinterpret_cast<u32x4*>(kt + L::chunk_offset(row, 2 * cc + 1)) = hi;
+                widen16(vc, lo, hi);
+                *reinterpret_cast<u32x4*>(vt + L::chunk_offset(row, 2 * cc)) = lo;
+                *reinterpret_cast<u32x4*>(vt + L::chunk_offset(row, 2 * cc + 1)) = hi;
+            }
+        } else {
+            const int last = uniform(b.last);
+            const int64_t off = (static_cast<int64_t>(uniform(static_cast<int>(b.off >> 32))) << 32) |
+                                static_cast<uint32_t>(uniform(static_cast<int>(b.off)));
+            const uint8_t* kbase = reinterpret_cast<const uint8_t*>(a.k_new) + off;
+            const uint8_t* vbase = reinterpret_cast<const uint8_t*>(a.v_new) + off;
+#pragma unroll
+            for (int j = 0; j < C::IPW; ++j) {
+                const int r = j * C::RPI + lane / C::CPR;
+                const int row = wave * C::ROWS_PER_WAVE + r;
+                const int cc = lane % C::CPR;
+                const int64_t voff = static_cast<int64_t>(min(r, last)) * a.kn_st * 2 + cc * 32;
+                const u32x4 k0 = *reinterpret_cast<const u32x4*>(kbase + voff);
+                const u32x4 k1 = *reinterpret_cast<const u32x4*>(kbase + voff + 16);
+                const u32x4 v0 = *reinterpret_cast<const u32x4*>(vbase + voff);
+                const u32x4 v1 = *reinterpret_cast<const u32x4*>(vbase + voff + 16);
+                // Wait here, inside the branch: a wait the compiler places where the two branches
+                // meet again would drain the asynchronous loads in every step.
+                __builtin_amdgcn_s_waitcnt(0x0f70);
+                *reinterpret_cast<u32x4*>(kt + L::chunk_offset(row, 2 * cc)) = k0;
+                *reinterpret_cast<u32x4*>(kt + L::chunk_offset(row, 2 * cc + 1)) = k1;
+                *reinterpret_cast<u32x4*>(vt + L::chunk_offset(row, 2 * cc)) = v0;
+                *reinterpret_cast<u32x4*>(vt + L::chunk_offset(row, 2 * cc + 1)) = v1;
+            }
         }
     }
 
@@ -221,8 +287,31 @@ struct StreamAttn : TileMath<HD, NB, NW> {
         this->kvh = uniform(d.kvh);
         this->q0 = uniform(d.q0);
         this->sh.q_len = uniform(d.q_len);
+        if (KVB == 1) {
+            k_mul = a.k_scale[this->kvh];
+            v_mul = a.v_scale[this->kvh];
+        }
         this->load_queries(uniform(d.rt));
         touch_queries();
+    }
+
+    // Close the item whose last unit of this workgroup's piece is planned unit `last_rel`.
+    DFX_D void finish_run(int last_rel, const WgSplit& split) {
+        const UnitDesc e = units[last_rel];
+        if (!(uniform(e.flags) & kUnitLast)) return;
+        this->outputs_ready();
+        float l_tot[NB];
+        this->row_sums(l_tot);
+        if (uniform(e.flags) & kUnitComplete) this->store_output(uniform(e.rt), l_tot);
+        else finish_cut_item(*this, uniform(e.rt), begin + uniform(e.item_rel), uniform(e.n_tiles), split,
+                             uniform(e.slot), l_tot, misc + kMaxWaves + 1);
+    }
+
+    // Wait until at most `younger` units' loads of this wave are outstanding (younger <= 2).
+    DFX_D static void wait_younger(int younger) {
+        if (younger >= 2) wait_async_loads<2 * C::LOADS_PER_UNIT>();
+        else if (younger == 1) wait_async_loads<C::LOADS_PER_UNIT>();
+        else wait_async_loads<0>();
     }
 };
 
@@ -259,10 +348,7 @@ __global__ void __launch_bounds__(64 * NW, COMPACT ? 2 : 1) paged_attn_stream_ke
             if (flags & kUnitFirst) at.begin_item(d);
             for (; rel < run_end; ++rel) {
                 // the unit must have landed: only younger units may still be outstanding
-                const int younger = issued - rel - 1;
-                if (younger >= 2) wait_async_loads<2 * C::LOADS_PER_UNIT>();
-                else if (younger == 1) wait_async_loads<C::LOADS_PER_UNIT>();
-                else wait_async_loads<0>();
+                at.wait_younger(issued - rel - 1);
                 __builtin_amdgcn_s_barrier();
                 // every wave has finished the previous unit: its stage may be overwritten
                 if (issued < n_units) at.issue_unit(issued++);
@@ -281,15 +367,71 @@ __global__ void __launch_bounds__(64 * NW, COMPACT ? 2 : 1) paged_attn_stream_ke
                 at.template softmax_tile<false>(sc, t, pb, [&] { at.outputs_ready(); });
                 at.accumulate(k_tile + C::MAT_BYTES, pb);
             }
-            const UnitDesc e = at.units[rel - 1];
-            if (uniform(e.flags) & kUnitLast) {
-                at.outputs_ready();
-                float l_tot[NB];
-                at.row_sums(l_tot);
-                if (uniform(e.flags) & kUnitComplete) at.store_output(uniform(e.rt), l_tot);
-                else finish_cut_item(at, uniform(e.rt), begin + uniform(e.item_rel), uniform(e.n_tiles), split,
-                                     uniform(e.slot), l_tot, at.misc + kMaxWaves + 1);
+            at.finish_run(rel - 1, split);
+        }
+    }
+}
+
+// FP8-E4M3 context cache (fresh K/V stay bf16).  The ring stages hold the codes as stored; in
+// step `rel` a wave first widens its own rows of unit rel + 1 into the bf16 tile the matrix
+// instructions of the previous step have just released, then computes unit rel from the other
+// bf16 tile.  The ring needs no barrier (a stage's band is written and read by one wave only);
+// the one barrier per step orders the two bf16 tiles.
+template <int HD, int NW>
+__global__ void __launch_bounds__(64 * NW, 1) paged_attn_stream_fp8_kernel(const KArgs a) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    using C = StreamCfg<HD, 1, NW, false, 1>;
+    StreamAttn<HD, 1, NW, false, 1> at(a, smem);
+    at.per_head = build_unit_prefix<C::RT>(a, at.prefix, at.misc);
+    const int64_t total = static_cast<int64_t>(at.per_head) * a.h_kv;
+    if (total == 0) return;
+    const int w = blockIdx.x;
+    const WgSplit split = make_wg_split(total, a.n_wg);
+    at.begin = split.first(w);
+    at.end = split.first(w + 1);
+    if (at.begin >= at.end) return;
+    const int64_t begin = at.begin, end = at.end;
+
+    for (int64_t chunk = begin; chunk < end; chunk += C::kPlanUnits) {
+        const int n_units = static_cast<int>(min(static_cast<int64_t>(C::kPlanUnits), end - chunk));
+        __syncthreads();  // every wave is done with the previous plan, its stages and bf16 tiles
+        at.plan_units(chunk, n_units);
+        __syncthreads();
+
+        int issued = 0;
+        for (; issued < C::kStages - 1 && issued < n_units; ++issued) at.issue_unit(issued);
+        at.wait_younger(issued - 1);
+        at.widen_unit(0);
+
+        int rel = 0;
+        while (rel < n_units) {
+            const UnitDesc d = at.units[rel];
+            const int flags = uniform(d.flags);
+            const int run_end = min(rel + uniform(d.run), n_units);
+            if (flags & kUnitFirst) at.begin_item(d);
+            for (; rel < run_end; ++rel) {
+                // stage (rel + 3) % 4 held unit rel - 1, which this wave widened a step ago
+                if (issued < n_units) at.issue_unit(issued++);
+                if (rel + 1 < n_units) at.wait_younger(issued - rel - 2);
+                // every wave has widened its rows of unit rel and is done computing unit rel - 1
+                __builtin_amdgcn_s_barrier();
+                if (rel + 1 < n_units) at.widen_unit(rel + 1);
+
+                const UnitDesc u = at.units[rel];
+                TileInfo t;
+                t.base = uniform(u.base);
+                t.limit = uniform(u.limit);
+                t.is_ctx = (uniform(u.flags) & kUnitCtx) != 0;
+                t.c_tile = t.is_ctx ? a.c * at.k_mul : a.c;
+                t.v_mul = t.is_ctx ? at.v_mul : 1.0f;
+                const uint8_t* k_tile = at.wide_tile(rel);
+                f32x16 sc[2][1];
+                at.scores(k_tile, sc);
+                bf16x8 pb[1][2][2];
+                at.template softmax_tile<true>(sc, t, pb, [&] { at.outputs_ready(); });
+                at.accumulate(k_tile + TileLayout<HD>::MAT_BYTES, pb);
             }
+            at.finish_run(rel - 1, split);
         }
     }
 }

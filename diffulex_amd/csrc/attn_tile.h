@@ -17,6 +17,22 @@ namespace dfx {
 
 DFX_D int uniform(int v) { return __builtin_amdgcn_readfirstlane(v); }
 
+// Two e4m3 codes (bytes 0,1 or 2,3 of w) -> two bf16 packed in a dword.  An e4m3 value has 3
+// mantissa bits, so the upper half of its fp32 form is its bf16 form.
+template <bool HI>
+DFX_D uint32_t fp8x2_to_bf16x2(uint32_t w) {
+    const f32x2 f = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(w), HI);
+    return (__float_as_uint(f.x) >> 16) | (__float_as_uint(f.y) & 0xffff0000u);
+}
+
+// 16 e4m3 codes -> 16 bf16 (two 16-byte chunks, in order).
+DFX_D void widen16(u32x4 codes, u32x4& lo, u32x4& hi) {
+    lo = u32x4{fp8x2_to_bf16x2<false>(codes.x), fp8x2_to_bf16x2<true>(codes.x),
+               fp8x2_to_bf16x2<false>(codes.y), fp8x2_to_bf16x2<true>(codes.y)};
+    hi = u32x4{fp8x2_to_bf16x2<false>(codes.z), fp8x2_to_bf16x2<true>(codes.z),
+               fp8x2_to_bf16x2<false>(codes.w), fp8x2_to_bf16x2<true>(codes.w)};
+}
+
 template <int HD>
 struct TileLayout {
     static constexpr int ROWB = HD * 2;                   // bytes per token row

@@ -5,9 +5,9 @@
 // workgroup holds every query row that shares the KV head -- all G = H_q / H_kv heads of
 // every query token, up to 128*NB rows -- so each K/V tile is fetched from HBM once per KV
 // head and reused by the whole GQA group.  Two tile paths feed the same MFMA / online-softmax
-// core (attn_common.h): the streaming path (attn_stream.h: direct-to-LDS loads in a 4-stage
-// ring, bf16 KV, page sizes that are multiples of 16) and the generic path (attn_generic.h:
-// any page size, FP8-E4M3 KV).
+// core (attn_tile.h): the streaming path (attn_stream.h: direct-to-LDS loads in a 4-stage
+// ring; page sizes that are multiples of 16; bf16 KV, or FP8-E4M3 KV with head_dim 128) and
+// the generic path (attn_generic.h: any page size, any layout of the fresh K/V).
 #include "attn_common.h"
 #include "attn_generic.h"
 #include "attn_stream.h"
@@ -50,9 +50,13 @@ int make_plan(const dfx_attn_params* p, Plan& plan) {
     plan.hd = p->head_dim;
     plan.nb = rows <= 32 * kWaves ? 1 : 2;
     plan.fp8 = p->kv_dtype == DFX_KV_FP8_E4M3 && p->k_cache != nullptr;
-    plan.stream = !plan.fp8 && !(p->flags & DFX_ATTN_GENERIC_PATH) &&
-                  (p->k_cache == nullptr || (p->page_size > 0 && p->page_size % 16 == 0));
-    plan.compact = plan.stream && plan.nb == 1 && p->num_seqs <= kCompactMaxSeqs;
+    // The streaming path addresses a K row and its V row with one offset: page size a multiple
+    // of 16, fresh K and V laid out alike.  FP8 streaming exists for head_dim 128.
+    plan.stream = !(p->flags & DFX_ATTN_GENERIC_PATH) &&
+                  (p->k_cache == nullptr || (p->page_size > 0 && p->page_size % 16 == 0)) &&
+                  p->kn_stride_token == p->vn_stride_token && p->kn_stride_head == p->vn_stride_head &&
+                  (!plan.fp8 || p->head_dim == 128);
+    plan.compact = plan.stream && !plan.fp8 && plan.nb == 1 && p->num_seqs <= kCompactMaxSeqs;
     if (p->max_workgroups > 0) {
         plan.n_wg = p->max_workgroups;
     } else {
@@ -75,12 +79,17 @@ int64_t plan_workspace_bytes(const Plan& plan) {
     return counter_bytes(plan) + 2 * static_cast<int64_t>(plan.n_wg) * plan.slot_floats * 4;
 }
 
-// PATH: 0 generic bf16, 1 generic FP8, 2 streaming bf16
+// PATH: 0 generic bf16, 1 generic FP8, 2 streaming bf16, 3 streaming FP8
 template <int HD, int NB, int PATH>
 int launch(const KArgs& ka, const Plan& plan, hipStream_t st) {
     void (*main_k)(const KArgs);
     int lds, threads = kThreads;
-    if constexpr (PATH == 2) {
+    if constexpr (PATH == 3) {
+        constexpr int NW = 4 * NB;
+        main_k = paged_attn_stream_fp8_kernel<HD, NW>;
+        lds = StreamCfg<HD, 1, NW, false, 1>::LDS_BYTES;
+        threads = 64 * NW;
+    } else if constexpr (PATH == 2) {
         // the streaming path gives every wave one 32-row query block: 4 waves for up to 128 rows,
         // 8 waves (two per SIMD, so one wave's softmax overlaps the other's matrix work) for 256
         constexpr int NW = 4 * NB;
@@ -198,6 +207,9 @@ extern "C" int dfx_paged_attn(const dfx_attn_params* p, dfx_stream_t stream) {
     hipStream_t st = static_cast<hipStream_t>(stream);
 #define DFX_ATTN_CASE(HD_, NB_)                                               \
     if (plan.hd == HD_ && plan.nb == NB_) {                                   \
+        if (plan.stream && plan.fp8) {                                        \
+            if constexpr (HD_ == 128) return launch<HD_, NB_, 3>(ka, plan, st); \
+        }                                                                     \
         if (plan.stream) return launch<HD_, NB_, 2>(ka, plan, st);       \
         if (plan.fp8) return launch<HD_, NB_, 1>(ka, plan, st);          \
         return launch<HD_, NB_, 0>(ka, plan, st);                        \

@@ -114,6 +114,45 @@ def test_fp8_kv_against_oracle(dev, over):
         assert max_abs_err(got, want) <= ATOL_FP8
 
 
+FP8_EDGE_CASES = [
+    # 4 waves (at most 128 rows), 8 waves, several row tiles; page sizes that are / are not multiples of 16
+    dict(num_seqs=5, h_q=4, h_kv=2, hd=128, page=16, ctx=[0, 1, 64, 65, 300], q_len=32, dbs=32),
+    dict(num_seqs=4, h_q=14, h_kv=2, hd=128, page=256, ctx=[255, 256, 257, 1000], q_len=32, dbs=32),
+    dict(num_seqs=3, h_q=7, h_kv=1, hd=128, page=48, ctx=[47, 500, 0], q_len=64, dbs=32),
+    dict(num_seqs=2, h_q=8, h_kv=1, hd=128, page=32, ctx=[100, 200], q_len=64, dbs=64),
+    dict(num_seqs=3, h_q=6, h_kv=3, hd=128, page=24, ctx=[23, 24, 100], q_len=32, dbs=32),
+    dict(num_seqs=70, h_q=4, h_kv=1, hd=128, page=64, ctx=(0, 200), q_len=32, dbs=32),   # more units than one plan holds
+]
+
+
+@pytest.mark.parametrize("flags", PATHS)
+@pytest.mark.parametrize("case", FP8_EDGE_CASES)
+@pytest.mark.parametrize("mask", [MASK_FULL, MASK_BLOCK_CAUSAL])
+def test_fp8_edge_cases(dev, case, mask, flags):
+    wl = make_workload("c5", seed=29, mask=mask, **case)
+    want = oracle_fp32(wl)
+    g = wl.to(dev)
+    for max_wg in (1, 5, 0):
+        got = _run(g, max_wg, flags=flags)
+        assert max_abs_err(got, want) <= ATOL_FP8
+
+
+def test_fresh_k_and_v_with_different_strides(dev):
+    """K and V rows cut out of differently shaped parents (the streaming path assumes one layout
+    for both and must hand such calls to the generic path)."""
+    for name in ("c4", "c5"):
+        wl = make_workload(name, num_seqs=3, ctx=(50, 400))
+        want = oracle_fp32(wl)
+        g = wl.to(dev)
+        t, h, d = g.v_new.shape
+        parent = torch.zeros(t, h + 1, d + 64, dtype=g.v_new.dtype, device=dev)
+        parent[:, 1:, :d] = g.v_new
+        g.v_new = parent[:, 1:, :d]
+        assert g.v_new.stride() != g.k_new.stride()
+        got = _run(g)
+        assert max_abs_err(got, want) <= (ATOL_FP8 if name == "c5" else ATOL_BF16)
+
+
 @pytest.mark.parametrize("flags", PATHS)
 def test_d2f_block_causal_small_c4(dev, flags):
     wl = make_workload("c4", num_seqs=3, ctx=(100, 700))

@@ -19,7 +19,8 @@ struct GenericCfg : Shape<HD, NB> {
     // the block-table entries of the piece of an item being processed, so that the tile loop
     // does not chase a table entry in global memory before every row it loads
     static constexpr int kTableEntries = 4096;
-    static constexpr int TABLE_OFF = S::PREFIX_BYTES + S::MISC_BYTES + 2 * STAGE_BYTES;
+    static constexpr int STAGES_OFF = (S::PREFIX_BYTES + S::MISC_BYTES + 255) / 256 * 256;  // tiles start at a multiple of 256
+    static constexpr int TABLE_OFF = STAGES_OFF + 2 * STAGE_BYTES;
     static constexpr int LDS_BYTES = TABLE_OFF + kTableEntries * 4;
     static constexpr int CH16 = S::TN * HD * 2 / 16 / kThreads;  // 16-byte chunks per lane, bf16 tile
     static constexpr int CH8 = S::TN * HD / 16 / kThreads;       // 16-byte chunks per lane, fp8 tile
@@ -72,7 +73,7 @@ struct GenericAttn : TileMath<HD, NB, kWaves> {
         }
     }
 
-    DFX_D uint8_t* k_stage(int b) const { return lds + C::PREFIX_BYTES + C::MISC_BYTES + b * C::STAGE_BYTES; }
+    DFX_D uint8_t* k_stage(int b) const { return lds + C::STAGES_OFF + b * C::STAGE_BYTES; }
     DFX_D uint8_t* v_stage(int b) const { return k_stage(b) + C::K_BYTES; }
 
     DFX_D int64_t cache_row_offset(int tok, bool& ok) const {
@@ -204,7 +205,7 @@ struct GenericAttn : TileMath<HD, NB, kWaves> {
 
 template <int HD, int NB, bool FP8>
 __global__ void __launch_bounds__(kThreads) paged_attn_generic_kernel(const KArgs a) {
-    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    extern __shared__ __attribute__((aligned(256))) uint8_t smem[];
     GenericAttn<HD, NB, FP8> at(a, smem);
     const int per_head = build_unit_prefix<Shape<HD, NB>::RT>(a, at.prefix, at.misc);
     const int64_t total = static_cast<int64_t>(per_head) * a.h_kv;

@@ -71,7 +71,7 @@ struct StreamCfg : Shape<HD, NB, NW> {
     static constexpr int BAND_TABLE_BYTES = kPlanUnits * NW * static_cast<int>(sizeof(BandDesc));
     static constexpr int UNIT_TABLE_OFF = PREFIX_BYTES + S::MISC_BYTES;
     static constexpr int BAND_TABLE_OFF = UNIT_TABLE_OFF + UNIT_TABLE_BYTES;
-    static constexpr int STAGES_OFF = BAND_TABLE_OFF + BAND_TABLE_BYTES;
+    static constexpr int STAGES_OFF = (BAND_TABLE_OFF + BAND_TABLE_BYTES + 255) / 256 * 256;  // tiles start at a multiple of 256
     static constexpr int WIDE_OFF = STAGES_OFF + kStages * STAGE_BYTES;
     static constexpr int WIDE_BYTES = 2 * TileLayout<HD>::MAT_BYTES;  // widened K tile, widened V tile
     static constexpr int LDS_BYTES = WIDE_OFF + (KVB == 1 ? 2 * WIDE_BYTES : 0);
@@ -317,7 +317,7 @@ struct StreamAttn : TileMath<HD, NB, NW> {
 
 template <int HD, int NB, int NW, bool COMPACT>
 __global__ void __launch_bounds__(64 * NW, COMPACT ? 2 : 1) paged_attn_stream_kernel(const KArgs a) {
-    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    extern __shared__ __attribute__((aligned(256))) uint8_t smem[];
     using C = StreamCfg<HD, NB, NW, COMPACT>;
     StreamAttn<HD, NB, NW, COMPACT> at(a, smem);
     at.per_head = build_unit_prefix<C::RT>(a, at.prefix, at.misc);
@@ -379,7 +379,7 @@ __global__ void __launch_bounds__(64 * NW, COMPACT ? 2 : 1) paged_attn_stream_ke
 // the one barrier per step orders the two bf16 tiles.
 template <int HD, int NW>
 __global__ void __launch_bounds__(64 * NW, 1) paged_attn_stream_fp8_kernel(const KArgs a) {
-    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    extern __shared__ __attribute__((aligned(256))) uint8_t smem[];
     using C = StreamCfg<HD, 1, NW, false, 1>;
     StreamAttn<HD, 1, NW, false, 1> at(a, smem);
     at.per_head = build_unit_prefix<C::RT>(a, at.prefix, at.misc);

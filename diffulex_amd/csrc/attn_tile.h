@@ -87,29 +87,48 @@ struct TileMath : AttnState<HD, NB, NW> {
     using Base::o;
     using Base::qf;
 
-    DFX_D explicit TileMath(const KArgs& args) : Base(args) {}
+    // LDS addressing.  A tile starts at a multiple of its row pitch (256 or 128 bytes), so the
+    // chunk swizzle, an XOR on bits 4..7 of the offset, can be applied to the finished address:
+    //   K operand (tb, slab):       ((tile + k_lane) ^ (slab * 32)) + tb * 32 rows
+    //   V operand (tb, sl, db, ii): ((tile + v_lane) ^ (zi * 64)) + (tb * 32 + sl * 16 + ii * 8) rows,
+    //                               zi = db ^ (swizzle(ii * 8) / 4)
+    // with one per-lane constant each.  Per tile that is one addition and a few XORs; the rest
+    // folds into the instructions' immediate offsets.  (swizzle(r0 + x) == swizzle(r0) ^ swizzle(x)
+    // holds for the row splits used here: 32-row blocks, and ii * 8 + (0..7) inside 16 rows.)
+    uint32_t k_lane, v_lane;
 
-    // ---- tile arithmetic -------------------------------------------------------------------
-    DFX_D bf16x8 read_k(const uint8_t* k_tile, int tb, int slab) const {
-        const int row = tb * 32 + col;
-        const int pos = (2 * slab + half) ^ L::swizzle(row);
-        return *reinterpret_cast<const bf16x8*>(k_tile + row * L::ROWB + pos * 16);
+    DFX_D explicit TileMath(const KArgs& args) : Base(args) {
+        k_lane = col * L::ROWB + ((half ^ L::swizzle(col)) * 16);
+        const int g16 = lane >> 4, sl16 = lane & 15;
+        const int lrow = (g16 >> 1) * 4 + (sl16 >> 2);         // 0..7
+        const int c = (g16 & 1) * 2 + ((sl16 & 3) >> 1);       // 0..3
+        v_lane = lrow * L::ROWB + ((c ^ L::swizzle(lrow)) * 16) + (sl16 & 1) * 8;
     }
 
-    // V^T operand for token slab (tb, sl) and d block db.
-    DFX_D bf16x8 read_vt(const uint8_t* v_tile, int tb, int sl, int db) const {
+    DFX_D static uint32_t lds_address(const uint8_t* p) {
+        return static_cast<uint32_t>(reinterpret_cast<uintptr_t>(p));
+    }
+
+    // ---- tile arithmetic -------------------------------------------------------------------
+    // kx: the K tile's address plus k_lane, XORed with slab * 32
+    DFX_D bf16x8 read_k(uint32_t kx, int tb) const {
+        typedef __attribute__((address_space(3))) bf16x8 lds_bf16x8;
+        return *(const lds_bf16x8*)static_cast<uintptr_t>(kx + tb * 32 * L::ROWB);
+    }
+
+    // V^T operand for token slab (tb, sl) and d block db; vx[zi]: the V tile's address plus
+    // v_lane, XORed with zi * 64.
+    static constexpr int kVx = HD == 128 ? 4 : 2;
+    DFX_D bf16x8 read_vt(const uint32_t (&vx)[kVx], int tb, int sl, int db) const {
         typedef short short4v __attribute__((ext_vector_type(4)));
         typedef short short8v __attribute__((ext_vector_type(8)));
         typedef __attribute__((address_space(3))) short4v lds_short4v;
-        const int g16 = lane >> 4, sl16 = lane & 15;
         short4v r[2];
 #pragma unroll
         for (int ii = 0; ii < 2; ++ii) {
-            const int row = tb * 32 + sl * 16 + ii * 8 + (g16 >> 1) * 4 + (sl16 >> 2);
-            const int chunk = db * 4 + (g16 & 1) * 2 + ((sl16 & 3) >> 1);
-            const int pos = chunk ^ L::swizzle(row);
-            const uint8_t* p = v_tile + row * L::ROWB + pos * 16 + (sl16 & 1) * 8;
-            r[ii] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4v*)(p));
+            const int zi = db ^ (L::swizzle(ii * 8) / 4);
+            const uint32_t p = vx[zi] + (tb * 32 + sl * 16 + ii * 8) * L::ROWB;
+            r[ii] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4v*)static_cast<uintptr_t>(p));
         }
         const short8v v = __builtin_shufflevector(r[0], r[1], 0, 1, 2, 3, 4, 5, 6, 7);
         return __builtin_bit_cast(bf16x8, v);
@@ -119,14 +138,16 @@ struct TileMath : AttnState<HD, NB, NW> {
     // current one: being volatile assembly those pin the order, so the LDS latency is hidden
     // only by what the source puts in between.
     DFX_D void scores(const uint8_t* k_tile, f32x16 (&sc)[2][NB]) const {
+        const uint32_t k0 = lds_address(k_tile) + k_lane;
         bf16x8 ka[2][2];
 #pragma unroll
-        for (int tb = 0; tb < 2; ++tb) ka[0][tb] = read_k(k_tile, tb, 0);
+        for (int tb = 0; tb < 2; ++tb) ka[0][tb] = read_k(k0, tb);
 #pragma unroll
         for (int slab = 0; slab < S::NSLAB; ++slab) {
             if (slab + 1 < S::NSLAB) {
+                const uint32_t kx = k0 ^ ((slab + 1) * 32);
 #pragma unroll
-                for (int tb = 0; tb < 2; ++tb) ka[(slab + 1) & 1][tb] = read_k(k_tile, tb, slab + 1);
+                for (int tb = 0; tb < 2; ++tb) ka[(slab + 1) & 1][tb] = read_k(kx, tb);
             }
 #pragma unroll
             for (int tb = 0; tb < 2; ++tb)
@@ -152,15 +173,19 @@ struct TileMath : AttnState<HD, NB, NW> {
 
     DFX_D void accumulate(const uint8_t* v_tile, const bf16x8 (&pb)[NB][2][2]) {
         constexpr int kSteps = 4 * S::NDB;  // (tb, sl, db)
+        uint32_t vx[kVx];
+        vx[0] = lds_address(v_tile) + v_lane;
+#pragma unroll
+        for (int zi = 1; zi < kVx; ++zi) vx[zi] = vx[0] ^ (zi * 64);
         bf16x8 va[3];
-        va[0] = read_vt(v_tile, 0, 0, 0);
-        va[1] = read_vt(v_tile, 0, 0, 1);
+        va[0] = read_vt(vx, 0, 0, 0);
+        va[1] = read_vt(vx, 0, 0, 1);
 #pragma unroll
         for (int st = 0; st < kSteps; ++st) {
             const int tb = st / (2 * S::NDB), sl = (st / S::NDB) & 1, db = st % S::NDB;
             if (st + 2 < kSteps) {
                 const int n = st + 2;
-                va[n % 3] = read_vt(v_tile, n / (2 * S::NDB), (n / S::NDB) & 1, n % S::NDB);
+                va[n % 3] = read_vt(vx, n / (2 * S::NDB), (n / S::NDB) & 1, n % S::NDB);
             }
 #pragma unroll
             for (int qb = 0; qb < NB; ++qb) mfma_output(o[db][qb], va[st % 3], pb[qb][tb][sl]);

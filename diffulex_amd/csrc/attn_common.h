@@ -363,7 +363,8 @@ struct AttnState {
 // workgroup that finishes last merges the stored ones into its own registers and writes the
 // rows (bit-identical whichever piece that is).  Who is last is decided by an arrival counter per item (indexed by the workgroup that
 // owns the item's first unit; a workgroup owns at most one such cut item):
-//   - a workgroup that finds every other piece already arrived merges without storing its own;
+//   - a workgroup that finds every other piece already arrived merges without storing its own
+//     (only the owner of the item's first units looks: the others are early by construction);
 //   - otherwise it stores its piece, waits until the stores have completed, and increments the
 //     counter; if that increment was the last arrival after all, it merges the others.
 // Nobody waits for anybody.  The last arrival resets the counter for the next launch.  Must be
@@ -383,10 +384,16 @@ DFX_D void finish_cut_item(AttnState<HD, NB, NW>& at, int rt, int64_t item_begin
     }
     int* counter = a.arrivals + wa;
 
-    if (threadIdx.x == 0) *flag = __hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    __syncthreads();
-    bool last = *flag == pieces - 1;
-    __syncthreads();
+    // The owner of the item's first units works on them at the end of its range, every other
+    // owner at the start of its own: only the former is likely to find the others arrived, the
+    // others skip the look (a round trip to memory) and go straight to storing.
+    bool last = false;
+    if (me == wa) {
+        if (threadIdx.x == 0) *flag = __hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __syncthreads();
+        last = *flag == pieces - 1;
+        __syncthreads();
+    }
     bool stored = false;
     if (!last || pieces > 2) {
         at.store_partial(my_slot, l_tot);

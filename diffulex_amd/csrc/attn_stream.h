@@ -281,8 +281,9 @@ struct StreamAttn : TileMath<HD, NB, NW> {
             for (int slab = 0; slab < C::NSLAB; ++slab) asm volatile("" : : "v"(qf[qb][slab]));
     }
 
-    // Adopt the item of unit d as the current one and fetch its query rows.
-    DFX_D void begin_item(const UnitDesc& d) {
+    // Adopt the item of unit d as the current one and fetch its query rows.  With wait == false
+    // the caller calls touch_queries() itself before the tile loop.
+    DFX_D void begin_item(const UnitDesc& d, bool wait = true) {
         this->s = uniform(d.s);
         this->kvh = uniform(d.kvh);
         this->q0 = uniform(d.q0);
@@ -292,7 +293,7 @@ struct StreamAttn : TileMath<HD, NB, NW> {
             v_mul = a.v_scale[this->kvh];
         }
         this->load_queries(uniform(d.rt));
-        touch_queries();
+        if (wait) touch_queries();
     }
 
     // Close the item whose last unit of this workgroup's piece is planned unit `last_rel`.
@@ -336,8 +337,13 @@ __global__ void __launch_bounds__(64 * NW, COMPACT ? 2 : 1) paged_attn_stream_ke
         at.plan_units(chunk, n_units);
         __syncthreads();
 
+        // An item that opens with this plan: its query rows are requested ahead of the ring fill,
+        // so that their (cold) latency runs concurrently with that of the first tiles.
+        const bool opens = (uniform(at.units[0].flags) & kUnitFirst) != 0;
+        if (opens) at.begin_item(at.units[0], false);
         int issued = 0;  // ring fill: kStages - 1 units in flight
         for (; issued < C::kStages - 1 && issued < n_units; ++issued) at.issue_unit(issued);
+        at.touch_queries();  // unconditional: the compiler must see no path into the tile loop with these loads pending
 
         int rel = 0;
         while (rel < n_units) {
@@ -345,7 +351,7 @@ __global__ void __launch_bounds__(64 * NW, COMPACT ? 2 : 1) paged_attn_stream_ke
             const UnitDesc d = at.units[rel];
             const int flags = uniform(d.flags);
             const int run_end = min(rel + uniform(d.run), n_units);
-            if (flags & kUnitFirst) at.begin_item(d);
+            if ((flags & kUnitFirst) && rel != 0) at.begin_item(d);
             for (; rel < run_end; ++rel) {
                 // the unit must have landed: only younger units may still be outstanding
                 at.wait_younger(issued - rel - 1);
@@ -398,8 +404,11 @@ __global__ void __launch_bounds__(64 * NW, 1) paged_attn_stream_fp8_kernel(const
         at.plan_units(chunk, n_units);
         __syncthreads();
 
+        const bool opens = (uniform(at.units[0].flags) & kUnitFirst) != 0;
+        if (opens) at.begin_item(at.units[0], false);  // query rows ahead of the ring fill, as in the bf16 kernel
         int issued = 0;
         for (; issued < C::kStages - 1 && issued < n_units; ++issued) at.issue_unit(issued);
+        at.touch_queries();  // unconditional: the compiler must see no path into the tile loop with these loads pending
         at.wait_younger(issued - 1);
         at.widen_unit(0);
 
@@ -408,7 +417,7 @@ __global__ void __launch_bounds__(64 * NW, 1) paged_attn_stream_fp8_kernel(const
             const UnitDesc d = at.units[rel];
             const int flags = uniform(d.flags);
             const int run_end = min(rel + uniform(d.run), n_units);
-            if (flags & kUnitFirst) at.begin_item(d);
+            if ((flags & kUnitFirst) && rel != 0) at.begin_item(d);
             for (; rel < run_end; ++rel) {
                 // stage (rel + 3) % 4 held unit rel - 1, which this wave widened a step ago
                 if (issued < n_units) at.issue_unit(issued++);

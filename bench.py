@@ -30,8 +30,8 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this command, scaled by
-# what the same counters read for a plain copy of known size (profiles/paged_attn_stream_kernel_c3.md).
-MEASURED_TRAFFIC_BYTES = {"c3": 291.5e6}
+# what the same counters read for a plain copy of known size (one summary per workload under profiles/).
+MEASURED_TRAFFIC_BYTES = {"c3": 288.5e6, "c4": 1490.9e6, "c5": 856.8e6}
 
 
 def algorithmic_bytes(wl) -> int:
@@ -231,7 +231,7 @@ def main():
             "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
             "algorithmic_bytes": nbytes, "algorithmic_flops": nflops,
             "mfma_tflops": tflops, "mfma_frac": tflops / MFMA_BF16_PEAK_TFLOPS,
-            "kernel": "paged_attn_stream_kernel / paged_attn_generic_kernel (one launch per step), "
+            "kernel": "paged_attn_stream_kernel (bf16 KV) / paged_attn_stream_fp8_kernel (FP8 KV), one launch per step, "
                       "duration = timed region / steps",
         },
     }

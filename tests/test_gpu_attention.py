@@ -258,3 +258,42 @@ def test_full_size_c4_and_c5_on_sampled_sequences(dev):
             assert max_abs_err(out[cu[s]:cu[s + 1]], w) <= tol
         del wl, out
         torch.cuda.empty_cache()
+
+
+def test_static_decode_in_a_captured_graph(dev):
+    """The block-diffusion runner replays the decode step from a captured graph
+    (strategy/block_diffusion/engine/model_runner.py:206-274): store + attention are captured once,
+    then replayed with new contents in the same tensors.  Every replay is compared with the eager
+    result on the same inputs, with eager launches and synchronisations in between."""
+    wl = make_workload("c3", num_seqs=6, ctx=(300, 900), seed=41).to(dev)   # cut items: partials and counters in use
+    att = dfx.Attention(wl.num_q_heads, wl.head_dim, wl.scale, wl.num_kv_heads)
+    att.k_cache, att.v_cache = wl.k_cache, wl.v_cache
+    md = metadata_for(wl, "static")
+    dfx.set_fetch_fn_for_attn_metadata(lambda: md)
+    t = wl.q.shape[0]
+    q, k, v = (x.reshape(t, -1).clone() for x in (wl.q, wl.k_new, wl.v_new))
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):          # warm-up on the capture stream: its workspace exists before the capture
+        att(q, k, v)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        o_static = att(q, k, v)
+    gen = torch.Generator(device=dev).manual_seed(7)
+    for rep in range(4):
+        for x in (q, k, v):
+            x.copy_(torch.randn(x.shape, generator=gen, device=dev, dtype=torch.float32).to(x.dtype))
+        if rep == 2:   # other contexts, same shapes
+            md.context_lens.copy_(torch.clamp(md.context_lens - 37 * (rep + 1), min=0))
+        graph.replay()
+        torch.cuda.synchronize()
+        got = o_static.clone()
+        eager = att(q, k, v)
+        torch.cuda.synchronize()
+        assert torch.equal(got, eager), f"replay {rep}"
+    wl2 = wl.to("cpu")
+    wl2.q, wl2.k_new, wl2.v_new = (x.view(t, -1, wl.head_dim).cpu() for x in (q, k, v))
+    wl2.context_lens = md.context_lens.cpu()
+    assert max_abs_err(got.view(t, wl.num_q_heads, wl.head_dim), oracle_fp32(wl2)) <= ATOL_BF16

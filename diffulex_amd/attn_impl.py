@@ -22,6 +22,7 @@ class Attention(nn.Module):
         self.scale = scale
         self.num_kv_heads = num_kv_heads
         self.k_cache = self.v_cache = torch.tensor([])
+        self.fuse_kv_store = True  # False: store in a launch of its own, as the reference does
         # looked up at call time so that a later set_fetch_fn_for_attn_metadata() is seen
         self.fetch_attn_metadata = lambda: _metadata.fetch_attn_metadata()
 
@@ -34,16 +35,25 @@ class Attention(nn.Module):
         k_cache, v_cache = self.k_cache, self.v_cache
         is_unified_layout = attn_metadata.kv_cache_layout == "unified"
 
+        # Decode on the unified layout: the store rides in the attention launch (the block being
+        # stored follows the attended context, so the two never touch the same slots).
+        fused_slots = None
         if k_cache.numel() and v_cache.numel():
             if attn_metadata.need_kv_cache_store:
-                store_kvcache = store_kvcache_unified_layout if is_unified_layout else store_kvcache_distinct_layout
-                store_kvcache(k, v, k_cache, v_cache, attn_metadata.slot_mapping, attn_metadata)
+                slots = attn_metadata.slot_mapping
+                if (self.fuse_kv_store and is_unified_layout and not attn_metadata.is_prefill
+                        and slots.is_contiguous() and slots.dtype in (torch.int32, torch.int64)):
+                    fused_slots = slots
+                else:
+                    store_kvcache = store_kvcache_unified_layout if is_unified_layout else store_kvcache_distinct_layout
+                    store_kvcache(k, v, k_cache, v_cache, slots, attn_metadata)
 
         if attn_metadata.is_prefill:
             o = dllm_flash_attn_prefill(q, k, v, self.scale, attn_metadata)
         else:
             if is_unified_layout:
-                o = dllm_flash_attn_decode(q, k, v, k_cache, v_cache, self.scale, attn_metadata)
+                o = dllm_flash_attn_decode(q, k, v, k_cache, v_cache, self.scale, attn_metadata,
+                                           store_slot_mapping=fused_slots)
             else:
                 raise NotImplementedError("Distinct layout is not supported yet...")
 

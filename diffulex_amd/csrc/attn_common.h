@@ -12,6 +12,7 @@
 #pragma once
 
 #include "dfx_common.h"
+#include "fp8_e4m3.h"
 #include "partition.h"
 
 namespace dfx {
@@ -41,6 +42,8 @@ struct KArgs {
     const float* v_scale;
     float* workspace;  // partial-result slots
     int* arrivals;     // one arrival counter per workgroup, zero between launches
+    const void* store_slots;  // fused KV-cache store: slot per fresh row, or null
+    int store_slots_i64;
     int64_t q_st, q_sh, kn_st, kn_sh, vn_st, vn_sh, o_st, o_sh;
     int64_t c_sp, c_st, c_sh;  // cache strides in elements: page, token, head
     int64_t bt_stride, n_pages;
@@ -430,6 +433,42 @@ DFX_D void finish_cut_item(AttnState<HD, NB, NW>& at, int rt, int64_t item_begin
     for (int qb = 0; qb < NB; ++qb) l_all[qb] = at.l_run[qb];
     at.store_output(rt, l_all);
     if (threadIdx.x == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Fused KV-cache store: fresh row t of k_new / v_new goes to cache slot store_slots[t] (what
+// dfx_kv_store_unified does in a launch of its own).  The 16-byte chunks of all rows are dealt
+// round-robin to the threads of the whole grid; every workgroup calls this once.  The slots
+// written are outside every attended context (caller's contract), so nothing in this launch
+// reads them.
+template <int HD, bool FP8>
+DFX_D void store_fresh_rows(const KArgs& a) {
+    if (a.store_slots == nullptr) return;
+    constexpr int kChunksPerHead = HD / 8;
+    const int chunks_per_token = a.h_kv * kChunksPerHead;
+    const int64_t total = static_cast<int64_t>(a.cu_new[a.num_seqs]) * chunks_per_token;
+    const int64_t n_slots = a.n_pages * a.page_size;
+    uint8_t* kc = const_cast<uint8_t*>(a.k_cache);
+    uint8_t* vc = const_cast<uint8_t*>(a.v_cache);
+    for (int64_t idx = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; idx < total;
+         idx += static_cast<int64_t>(gridDim.x) * blockDim.x) {
+        const int64_t t = idx / chunks_per_token;
+        const int r = static_cast<int>(idx - t * chunks_per_token);
+        const int h = r / kChunksPerHead, c = r - h * kChunksPerHead;
+        const int64_t slot = a.store_slots_i64 ? static_cast<const int64_t*>(a.store_slots)[t]
+                                               : static_cast<int64_t>(static_cast<const int32_t*>(a.store_slots)[t]);
+        if (slot < 0 || slot >= n_slots) continue;
+        const u32x4 k8 = *reinterpret_cast<const u32x4*>(a.k_new + t * a.kn_st + h * a.kn_sh + c * 8);
+        const u32x4 v8 = *reinterpret_cast<const u32x4*>(a.v_new + t * a.vn_st + h * a.vn_sh + c * 8);
+        const int64_t page = a.page_shift >= 0 ? (slot >> a.page_shift) : slot / a.page_size;
+        const int64_t dst = page * a.c_sp + (slot - page * a.page_size) * a.c_st + h * a.c_sh + c * 8;  // elements
+        if constexpr (FP8) {
+            *reinterpret_cast<u32x2*>(kc + dst) = quantise8(k8, a.k_scale[h]);
+            *reinterpret_cast<u32x2*>(vc + dst) = quantise8(v8, a.v_scale[h]);
+        } else {
+            *reinterpret_cast<u32x4*>(kc + dst * 2) = k8;
+            *reinterpret_cast<u32x4*>(vc + dst * 2) = v8;
+        }
+    }
 }
 
 // Exclusive prefix of units(s) into prefix[0..num_seqs]; returns the per-head total.

@@ -207,6 +207,7 @@ template <int HD, int NB, bool FP8>
 __global__ void __launch_bounds__(kThreads) paged_attn_generic_kernel(const KArgs a) {
     extern __shared__ __attribute__((aligned(256))) uint8_t smem[];
     GenericAttn<HD, NB, FP8> at(a, smem);
+    store_fresh_rows<HD, FP8>(a);
     const int per_head = build_unit_prefix<Shape<HD, NB>::RT>(a, at.prefix, at.misc);
     const int64_t total = static_cast<int64_t>(per_head) * a.h_kv;
     if (total == 0) return;

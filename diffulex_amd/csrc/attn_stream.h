@@ -323,12 +323,18 @@ __global__ void __launch_bounds__(64 * NW, COMPACT ? 2 : 1) paged_attn_stream_ke
     StreamAttn<HD, NB, NW, COMPACT> at(a, smem);
     at.per_head = build_unit_prefix<C::RT>(a, at.prefix, at.misc);
     const int64_t total = static_cast<int64_t>(at.per_head) * a.h_kv;
-    if (total == 0) return;
+    if (total == 0) {
+        store_fresh_rows<HD, false>(a);
+        return;
+    }
     const int w = blockIdx.x;
     const WgSplit split = make_wg_split(total, a.n_wg);
     at.begin = split.first(w);
     at.end = split.first(w + 1);
-    if (at.begin >= at.end) return;
+    if (at.begin >= at.end) {
+        store_fresh_rows<HD, false>(a);
+        return;
+    }
     const int64_t begin = at.begin, end = at.end;
 
     for (int64_t chunk = begin; chunk < end; chunk += C::kPlanUnits) {
@@ -343,6 +349,8 @@ __global__ void __launch_bounds__(64 * NW, COMPACT ? 2 : 1) paged_attn_stream_ke
         if (opens) at.begin_item(at.units[0], false);
         int issued = 0;  // ring fill: kStages - 1 units in flight
         for (; issued < C::kStages - 1 && issued < n_units; ++issued) at.issue_unit(issued);
+        // the fused cache store runs here, once, while the first tiles and the query rows are on their way
+        if (chunk == begin) store_fresh_rows<HD, false>(a);
         at.touch_queries();  // unconditional: the compiler must see no path into the tile loop with these loads pending
 
         int rel = 0;
@@ -390,12 +398,18 @@ __global__ void __launch_bounds__(64 * NW, 1) paged_attn_stream_fp8_kernel(const
     StreamAttn<HD, 1, NW, false, 1> at(a, smem);
     at.per_head = build_unit_prefix<C::RT>(a, at.prefix, at.misc);
     const int64_t total = static_cast<int64_t>(at.per_head) * a.h_kv;
-    if (total == 0) return;
+    if (total == 0) {
+        store_fresh_rows<HD, true>(a);
+        return;
+    }
     const int w = blockIdx.x;
     const WgSplit split = make_wg_split(total, a.n_wg);
     at.begin = split.first(w);
     at.end = split.first(w + 1);
-    if (at.begin >= at.end) return;
+    if (at.begin >= at.end) {
+        store_fresh_rows<HD, true>(a);
+        return;
+    }
     const int64_t begin = at.begin, end = at.end;
 
     for (int64_t chunk = begin; chunk < end; chunk += C::kPlanUnits) {
@@ -408,6 +422,8 @@ __global__ void __launch_bounds__(64 * NW, 1) paged_attn_stream_fp8_kernel(const
         if (opens) at.begin_item(at.units[0], false);  // query rows ahead of the ring fill, as in the bf16 kernel
         int issued = 0;
         for (; issued < C::kStages - 1 && issued < n_units; ++issued) at.issue_unit(issued);
+        // the fused cache store runs here, once, while the first tiles and the query rows are on their way
+        if (chunk == begin) store_fresh_rows<HD, true>(a);
         at.touch_queries();  // unconditional: the compiler must see no path into the tile loop with these loads pending
         at.wait_younger(issued - 1);
         at.widen_unit(0);

@@ -57,4 +57,18 @@ DFX_HD uint8_t quantise_e4m3(float x, float scale) {
     return f32_to_e4m3fn(y);
 }
 
+DFX_D uint32_t quantise_pair(uint32_t two_bf16, float scale) {
+    const uint8_t lo = quantise_e4m3(bf16_bits_to_f32(static_cast<uint16_t>(two_bf16 & 0xffffu)), scale);
+    const uint8_t hi = quantise_e4m3(bf16_bits_to_f32(static_cast<uint16_t>(two_bf16 >> 16)), scale);
+    return static_cast<uint32_t>(lo) | (static_cast<uint32_t>(hi) << 8);
+}
+
+// 8 bf16 (16 bytes) -> 8 e4m3 codes (8 bytes)
+DFX_D u32x2 quantise8(u32x4 v, float scale) {
+    u32x2 r;
+    r.x = quantise_pair(v.x, scale) | (quantise_pair(v.y, scale) << 16);
+    r.y = quantise_pair(v.z, scale) | (quantise_pair(v.w, scale) << 16);
+    return r;
+}
+
 }  // namespace dfx

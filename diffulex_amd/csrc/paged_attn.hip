@@ -134,6 +134,8 @@ extern "C" int dfx_paged_attn(const dfx_attn_params* p, dfx_stream_t stream) {
     Plan plan;
     const int rc = make_plan(p, plan);
     if (rc != DFX_OK) return rc;
+    // no query rows, no launch: a store asked for with such a call would be skipped silently
+    if (p->store_slot_mapping != nullptr && p->num_seqs > 0 && p->max_seqlen_q == 0) return DFX_ERR_INVALID_ARG;
     if (p->num_seqs == 0 || p->max_seqlen_q == 0) return DFX_OK;
     if (!p->q || !p->k_new || !p->v_new || !p->out || !p->cu_seqlens_q || !p->cu_seqlens_new)
         return DFX_ERR_INVALID_ARG;
@@ -142,6 +144,11 @@ extern "C" int dfx_paged_attn(const dfx_attn_params* p, dfx_stream_t stream) {
     if (has_cache && (!p->block_tables || p->page_size <= 0 || p->max_pages_per_seq < 0 || p->n_pages < 0))
         return DFX_ERR_INVALID_ARG;
     if (plan.fp8 && (!p->k_scale || !p->v_scale)) return DFX_ERR_INVALID_ARG;
+    if (p->store_slot_mapping != nullptr) {
+        if (!has_cache) return DFX_ERR_INVALID_ARG;
+        if (p->store_slot_index_type != DFX_INDEX_I32 && p->store_slot_index_type != DFX_INDEX_I64)
+            return DFX_ERR_INVALID_ARG;
+    }
     if (!(p->scale > 0.0f) || p->diffusion_block_size <= 0) return DFX_ERR_INVALID_ARG;
     if (p->mask_mode != DFX_MASK_FULL && p->mask_mode != DFX_MASK_BLOCK_CAUSAL) return DFX_ERR_INVALID_ARG;
     const int64_t strides8[] = {p->q_stride_token,  p->q_stride_head,   p->kn_stride_token, p->kn_stride_head,
@@ -174,6 +181,8 @@ extern "C" int dfx_paged_attn(const dfx_attn_params* p, dfx_stream_t stream) {
     ka.cu_new = p->cu_seqlens_new;
     ka.k_scale = p->k_scale;
     ka.v_scale = p->v_scale;
+    ka.store_slots = has_cache ? p->store_slot_mapping : nullptr;
+    ka.store_slots_i64 = p->store_slot_index_type == DFX_INDEX_I64;
     ka.arrivals = static_cast<int*>(p->workspace);
     ka.workspace = reinterpret_cast<float*>(static_cast<uint8_t*>(p->workspace) + counter_bytes(plan));
     ka.q_st = p->q_stride_token;

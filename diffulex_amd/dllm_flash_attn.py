@@ -13,7 +13,7 @@ from typing import Optional
 import torch
 
 from . import _lib
-from .kv_cache_kernels import _FP8_DTYPES, _scales, _stream
+from .kv_cache_kernels import _FP8_DTYPES, _index_type, _scales, _stream
 
 _workspaces = {}
 
@@ -30,10 +30,14 @@ def _workspace(device: torch.device, stream: int, nbytes: int) -> torch.Tensor:
 
 def paged_attention(q, k, v, k_cache, v_cache, scale, *, block_tables, context_lens, cu_seqlens_q,
                     cu_seqlens_new, max_seqlen_q, mask_mode=_lib.DFX_MASK_FULL, diffusion_block_size=32,
-                    k_scale=None, v_scale=None, max_workgroups=0, out=None, flags=0) -> torch.Tensor:
+                    k_scale=None, v_scale=None, max_workgroups=0, out=None, flags=0,
+                    store_slot_mapping=None) -> torch.Tensor:
     """Marshal tensors into ``dfx_attn_params`` and launch ``dfx_paged_attn`` on the
     current stream.  q: [T, H_q, hd]; k, v: [T_new, H_kv, hd]; caches
-    [pages, page, H_kv, hd] or None."""
+    [pages, page, H_kv, hd] or None.  ``store_slot_mapping`` ([T_new] int32/int64): the same
+    launch also writes the fresh rows into those cache slots (what
+    ``store_kvcache_unified_layout`` does in a launch of its own); the slots must lie outside
+    every attended context."""
     lib = _lib.load()
     assert q.is_cuda and q.dtype == torch.bfloat16 and k.dtype == torch.bfloat16 and v.dtype == torch.bfloat16
     assert q.dim() == 3 and k.dim() == 3 and v.shape == k.shape
@@ -81,6 +85,12 @@ def paged_attention(q, k, v, k_cache, v_cache, scale, *, block_tables, context_l
     p.max_workgroups = int(max_workgroups)
     p.flags = int(flags)
     p.scale = float(scale)
+    if store_slot_mapping is not None:
+        assert has_cache and store_slot_mapping.is_cuda and store_slot_mapping.is_contiguous()
+        assert store_slot_mapping.numel() == k.shape[0], \
+            f"`N`: {k.shape[0]}, `slot_mapping.numel()`: {store_slot_mapping.numel()}"
+        p.store_slot_mapping = store_slot_mapping.data_ptr()
+        p.store_slot_index_type = _index_type(store_slot_mapping)
     need = lib.dfx_paged_attn_workspace_bytes(C.byref(p))
     if need < 0:
         _lib.check(int(need), "dfx_paged_attn_workspace_bytes")
@@ -119,8 +129,10 @@ def dllm_flash_attn_prefill(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, s
 def dllm_flash_attn_decode(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, k_cache: torch.Tensor,
                            v_cache: torch.Tensor, scale: float, attn_metadata,
                            k_scale: Optional[torch.Tensor] = None,
-                           v_scale: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """dllm_flash_attn.py:599-637.
+                           v_scale: Optional[torch.Tensor] = None,
+                           store_slot_mapping: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """dllm_flash_attn.py:599-637.  ``store_slot_mapping`` (extension): also store the fresh
+    K/V rows into these cache slots in the same launch (see ``paged_attention``).
 
     ``decode_mode == "static"``: ``cu_seqlens_k`` indexes the fresh K/V rows
     (strategy/block_diffusion/engine/model_runner.py:134-139).
@@ -148,4 +160,4 @@ def dllm_flash_attn_decode(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, k_
         context_lens=attn_metadata.context_lens, cu_seqlens_q=attn_metadata.cu_seqlens_q,
         cu_seqlens_new=cu_new, max_seqlen_q=_max_seqlen_q(attn_metadata, attn_metadata.cu_seqlens_q),
         mask_mode=mask, diffusion_block_size=attn_metadata.diffusion_block_size,
-        k_scale=k_scale, v_scale=v_scale)
+        k_scale=k_scale, v_scale=v_scale, store_slot_mapping=store_slot_mapping)

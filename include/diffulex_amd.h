@@ -19,7 +19,7 @@
 extern "C" {
 #endif
 
-#define DFX_ABI_VERSION 1
+#define DFX_ABI_VERSION 2
 
 typedef void* dfx_stream_t; /* a hipStream_t; NULL is the default stream */
 
@@ -166,6 +166,17 @@ typedef struct dfx_attn_params {
     int32_t max_workgroups;      /* 0: one per compute unit; >0: exactly this many persistent workgroups */
     int32_t flags;               /* DFX_ATTN_* bits, 0 by default */
     float scale;
+    /* Fused KV-cache store (the store + decode pair of diffulex/attention/attn_impl.py:54-69 in
+     * one launch).  NULL: attend only.  Otherwise [T_new] slots of type store_slot_index_type:
+     * the launch also writes fresh row t of k_new / v_new to cache slot store_slot_mapping[t],
+     * exactly as dfx_kv_store_unified would (negative and out-of-range slots skipped, FP8 caches
+     * quantised with k_scale / v_scale), through the cache strides given above.  The slots
+     * written must lie outside the context_lens[s] tokens any sequence attends to in this call
+     * (true for the reference's runners, which store the block that follows the context):
+     * other workgroups read those pages while this one writes.  The caches are written
+     * through k_cache / v_cache although the pointers are declared const. */
+    const void* store_slot_mapping;
+    int32_t store_slot_index_type; /* dfx_index_type */
 } dfx_attn_params;
 
 /* Bytes of scratch dfx_paged_attn needs for these shapes (depends on the sizes

@@ -297,3 +297,37 @@ def test_static_decode_in_a_captured_graph(dev):
     wl2.q, wl2.k_new, wl2.v_new = (x.view(t, -1, wl.head_dim).cpu() for x in (q, k, v))
     wl2.context_lens = md.context_lens.cpu()
     assert max_abs_err(got.view(t, wl.num_q_heads, wl.head_dim), oracle_fp32(wl2)) <= ATOL_BF16
+
+
+@pytest.mark.parametrize("flags", PATHS)
+@pytest.mark.parametrize("name,over", [
+    ("c1", {}),
+    ("c3", dict(num_seqs=5, ctx=(200, 700))),
+    ("c4", dict(num_seqs=3, ctx=(100, 500))),
+    ("c5", dict(num_seqs=4, ctx=(200, 900))),
+    ("c5", dict(num_seqs=3, ctx=[256, 0, 511], h_q=8, h_kv=2, hd=64, page=32)),
+])
+def test_store_fused_into_the_attention_launch(dev, name, over, flags):
+    """One launch that stores the fresh block and attends == the store launch followed by the
+    attention launch (diffulex/attention/attn_impl.py:54-69): same cache bits, same output bits."""
+    wl = make_workload(name, seed=53, **over).to(dev)
+    md = metadata_for(wl, "static")
+    for slot_dtype in (torch.int32, torch.int64):
+        slots = wl.slot_mapping.to(slot_dtype).clone()
+        slots[1::7] = -1                                   # rows that are not stored
+        slots[3] = wl.k_cache.shape[0] * wl.k_cache.shape[1] + 5   # out of range: skipped
+        for max_wg in (0, 3, 1000):                        # 1000: more workgroups than units
+            kc_a, vc_a = wl.k_cache.clone(), wl.v_cache.clone()
+            dfx.store_kvcache_unified_layout(wl.k_new, wl.v_new, kc_a, vc_a, slots, md)
+            want = _run(wl, max_wg, flags=flags)
+            kc_b, vc_b = wl.k_cache.clone(), wl.v_cache.clone()
+            args = dict(block_tables=wl.block_tables, context_lens=wl.context_lens, cu_seqlens_q=wl.cu_seqlens_q,
+                        cu_seqlens_new=wl.cu_seqlens_q, max_seqlen_q=wl.q_len, mask_mode=wl.mask_mode,
+                        diffusion_block_size=wl.diffusion_block_size, k_scale=wl.k_scale, v_scale=wl.v_scale,
+                        max_workgroups=max_wg, flags=flags, store_slot_mapping=slots)
+            got = dfx.paged_attention(wl.q, wl.k_new, wl.v_new, kc_b, vc_b, wl.scale, **args)
+            torch.cuda.synchronize()
+            assert torch.equal(got, want)
+            assert torch.equal(kc_b.view(torch.uint8), kc_a.view(torch.uint8))
+            assert torch.equal(vc_b.view(torch.uint8), vc_a.view(torch.uint8))
+            assert not torch.equal(kc_b.view(torch.uint8), wl.k_cache.view(torch.uint8))  # something was stored

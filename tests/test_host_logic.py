@@ -3,6 +3,7 @@ host/device helper code (FP8 quantiser, bf16 rounding) and the work partition.""
 import ctypes as C
 import re
 import os
+import subprocess
 
 import numpy as np
 import pytest
@@ -27,9 +28,18 @@ def test_library_exports_every_declared_symbol():
     assert lib.dfx_status_string(-2) == b"unsupported shape"
 
 
-def test_struct_layout_matches_header():
-    # 14 pointers/int64 + 13 int64 + 12 int32 + 1 float
-    assert C.sizeof(_lib.AttnParams) == 8 * 27 + 4 * 13 + 4   # padded to a multiple of 8
+def test_struct_layout_matches_header(tmp_path):
+    """Size and every field offset of the ctypes mirror against what a C compiler makes of the header."""
+    names = [f[0] for f in _lib.AttnParams._fields_]
+    prints = "".join(f'printf("%zu\\n", offsetof(dfx_attn_params, {n}));' for n in names)
+    src = tmp_path / "layout.c"
+    src.write_text('#include <stdio.h>\n#include <stddef.h>\n#include "diffulex_amd.h"\n'
+                   'int main(void){printf("%zu\\n", sizeof(dfx_attn_params));' + prints + 'return 0;}\n')
+    exe = tmp_path / "layout"
+    subprocess.check_call(["gcc", "-I", os.path.join(ROOT, "include"), "-o", str(exe), str(src)])
+    got = [int(x) for x in subprocess.check_output([str(exe)]).split()]
+    assert got[0] == C.sizeof(_lib.AttnParams)
+    assert got[1:] == [getattr(_lib.AttnParams, n).offset for n in names]
 
 
 def test_argument_errors_do_not_launch():

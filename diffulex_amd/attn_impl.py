@@ -23,6 +23,7 @@ class Attention(nn.Module):
         self.num_kv_heads = num_kv_heads
         self.k_cache = self.v_cache = torch.tensor([])
         self.fuse_kv_store = True  # False: store in a launch of its own, as the reference does
+        self.fuse_kv_store_max_bytes = 6 << 20  # bf16 bytes of fresh K plus V up to which the store is fused
         # looked up at call time so that a later set_fetch_fn_for_attn_metadata() is seen
         self.fetch_attn_metadata = lambda: _metadata.fetch_attn_metadata()
 
@@ -41,7 +42,11 @@ class Attention(nn.Module):
         if k_cache.numel() and v_cache.numel():
             if attn_metadata.need_kv_cache_store:
                 slots = attn_metadata.slot_mapping
+                # (worth it while the block is small: measured on an MI355X the fused form saves a
+                # launch's worth of time up to about 4 MB of fresh K+V and loses beyond 8 MB, where a
+                # store kernel of its own has far more loads in flight than the attention grid)
                 if (self.fuse_kv_store and is_unified_layout and not attn_metadata.is_prefill
+                        and k.numel() * 4 <= self.fuse_kv_store_max_bytes
                         and slots.is_contiguous() and slots.dtype in (torch.int32, torch.int64)):
                     fused_slots = slots
                 else:

@@ -333,6 +333,11 @@ struct AttnState {
 
     // Merge one stored partial into the running state (l_run holds whole-row sums here).
     DFX_D void merge_partial(int slot) {
+        // No fused multiply-add in here: a * wa + b * wb must round both products, or merging a
+        // into b and b into a differ in the last bit (an fma keeps one product exact, and which
+        // one depends on who merges).  __fmul_rn / __fadd_rn would not do: they are plain operators
+        // in this toolchain and fuse like any other.
+#pragma clang fp contract(off)
 #pragma unroll
         for (int qb = 0; qb < NB; ++qb) {
             const __amdgpu_buffer_rsrc_t rs = block_resource(slot, qb);
@@ -345,7 +350,8 @@ struct AttnState {
             const float wb = (mp == -INFINITY) ? 0.0f : fast_exp2(mp - mn);
             // products and sum are rounded separately: merging a into b then gives the same bits as
             // b into a, so it does not matter which of two pieces does the merging
-            l_run[qb] = __fadd_rn(__fmul_rn(l_run[qb], wa), __fmul_rn(lp, wb));
+            const float la = l_run[qb] * wa, lb = lp * wb;
+            l_run[qb] = la + lb;
             m_run[qb] = mn;
 #pragma unroll
             for (int db = 0; db < S::NDB; ++db)
@@ -354,8 +360,10 @@ struct AttnState {
                     const f32x4 v = __builtin_bit_cast(
                         f32x4, __builtin_amdgcn_raw_buffer_load_b128(rs, ((db * 4 + ii) * 64 + lane) * 16, 0, kDeviceScope));
 #pragma unroll
-                    for (int j = 0; j < 4; ++j)
-                        o[db][qb][ii * 4 + j] = __fadd_rn(__fmul_rn(o[db][qb][ii * 4 + j], wa), __fmul_rn(v[j], wb));
+                    for (int j = 0; j < 4; ++j) {
+                        const float oa = o[db][qb][ii * 4 + j] * wa, ob = v[j] * wb;
+                        o[db][qb][ii * 4 + j] = oa + ob;
+                    }
                 }
         }
     }
@@ -444,29 +452,55 @@ template <int HD, bool FP8>
 DFX_D void store_fresh_rows(const KArgs& a) {
     if (a.store_slots == nullptr) return;
     constexpr int kChunksPerHead = HD / 8;
+    constexpr int kBatch = 4;  // chunks a thread has in flight: all loads of a batch are issued before its stores
     const int chunks_per_token = a.h_kv * kChunksPerHead;
     const int64_t total = static_cast<int64_t>(a.cu_new[a.num_seqs]) * chunks_per_token;
     const int64_t n_slots = a.n_pages * a.page_size;
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
     uint8_t* kc = const_cast<uint8_t*>(a.k_cache);
     uint8_t* vc = const_cast<uint8_t*>(a.v_cache);
-    for (int64_t idx = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; idx < total;
-         idx += static_cast<int64_t>(gridDim.x) * blockDim.x) {
-        const int64_t t = idx / chunks_per_token;
-        const int r = static_cast<int>(idx - t * chunks_per_token);
-        const int h = r / kChunksPerHead, c = r - h * kChunksPerHead;
-        const int64_t slot = a.store_slots_i64 ? static_cast<const int64_t*>(a.store_slots)[t]
-                                               : static_cast<int64_t>(static_cast<const int32_t*>(a.store_slots)[t]);
-        if (slot < 0 || slot >= n_slots) continue;
-        const u32x4 k8 = *reinterpret_cast<const u32x4*>(a.k_new + t * a.kn_st + h * a.kn_sh + c * 8);
-        const u32x4 v8 = *reinterpret_cast<const u32x4*>(a.v_new + t * a.vn_st + h * a.vn_sh + c * 8);
-        const int64_t page = a.page_shift >= 0 ? (slot >> a.page_shift) : slot / a.page_size;
-        const int64_t dst = page * a.c_sp + (slot - page * a.page_size) * a.c_st + h * a.c_sh + c * 8;  // elements
-        if constexpr (FP8) {
-            *reinterpret_cast<u32x2*>(kc + dst) = quantise8(k8, a.k_scale[h]);
-            *reinterpret_cast<u32x2*>(vc + dst) = quantise8(v8, a.v_scale[h]);
-        } else {
-            *reinterpret_cast<u32x4*>(kc + dst * 2) = k8;
-            *reinterpret_cast<u32x4*>(vc + dst * 2) = v8;
+    for (int64_t base = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; base < total;
+         base += stride * kBatch) {
+        int64_t slot[kBatch], src_k[kBatch], src_v[kBatch], dst[kBatch];
+        int head[kBatch];
+        u32x4 k8[kBatch], v8[kBatch];
+#pragma unroll
+        for (int j = 0; j < kBatch; ++j) {
+            const int64_t idx = base + j * stride;
+            slot[j] = -1;
+            if (idx < total) {
+                const int64_t t = idx / chunks_per_token;
+                const int r = static_cast<int>(idx - t * chunks_per_token);
+                const int h = r / kChunksPerHead, c = r - h * kChunksPerHead;
+                head[j] = h;
+                src_k[j] = t * a.kn_st + h * a.kn_sh + c * 8;
+                src_v[j] = t * a.vn_st + h * a.vn_sh + c * 8;
+                dst[j] = h * a.c_sh + c * 8;
+                slot[j] = a.store_slots_i64 ? static_cast<const int64_t*>(a.store_slots)[t]
+                                            : static_cast<int64_t>(static_cast<const int32_t*>(a.store_slots)[t]);
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < kBatch; ++j) {
+            if (slot[j] < 0 || slot[j] >= n_slots) {
+                slot[j] = -1;
+                continue;
+            }
+            k8[j] = *reinterpret_cast<const u32x4*>(a.k_new + src_k[j]);
+            v8[j] = *reinterpret_cast<const u32x4*>(a.v_new + src_v[j]);
+        }
+#pragma unroll
+        for (int j = 0; j < kBatch; ++j) {
+            if (slot[j] < 0) continue;
+            const int64_t page = a.page_shift >= 0 ? (slot[j] >> a.page_shift) : slot[j] / a.page_size;
+            const int64_t d = page * a.c_sp + (slot[j] - page * a.page_size) * a.c_st + dst[j];  // elements
+            if constexpr (FP8) {
+                *reinterpret_cast<u32x2*>(kc + d) = quantise8(k8[j], a.k_scale[head[j]]);
+                *reinterpret_cast<u32x2*>(vc + d) = quantise8(v8[j], a.v_scale[head[j]]);
+            } else {
+                *reinterpret_cast<u32x4*>(kc + d * 2) = k8[j];
+                *reinterpret_cast<u32x4*>(vc + d * 2) = v8[j];
+            }
         }
     }
 }

@@ -48,6 +48,7 @@ struct KArgs {
     int64_t c_sp, c_st, c_sh;  // cache strides in elements: page, token, head
     int64_t bt_stride, n_pages;
     int num_seqs, h_kv, group, page_size, page_shift, max_pages, dbs, mask_mode, n_wg;
+    int fixed_wg;  // the caller fixed the number of workgroups: all of them take part
     float c;  // scale * log2(e)
 };
 
@@ -505,14 +506,34 @@ DFX_D void store_fresh_rows(const KArgs& a) {
     }
 }
 
-// Exclusive prefix of units(s) into prefix[0..num_seqs]; returns the per-head total.
+// Exclusive prefix of units(s) into prefix[0..num_seqs]; also the per-head total, the number of
+// items per KV head and the tile count of the longest item.
+struct UnitSummary {
+    int per_head;    // units per KV head
+    int items;       // (sequence, row tile) items per KV head
+    int max_tiles;   // KV tiles of the longest item
+};
+
 template <int RT>
-DFX_D int build_unit_prefix(const KArgs& a, int* prefix, int* scratch) {
+DFX_D UnitSummary build_unit_prefix(const KArgs& a, int* prefix, int* scratch) {
     int carry = 0;
     const int n_threads = blockDim.x;
+    if (threadIdx.x == 0) {
+        scratch[kMaxWaves + 2] = 0;
+        scratch[kMaxWaves + 3] = 0;
+    }
+    __syncthreads();
     for (int base = 0; base < a.num_seqs; base += n_threads) {
         const int sq = base + threadIdx.x;
-        const int u = sq < a.num_seqs ? load_seq_shape(a, sq, RT).units : 0;
+        int u = 0;
+        if (sq < a.num_seqs) {
+            const SeqShape shp = load_seq_shape(a, sq, RT);
+            u = shp.units;
+            if (u > 0) {
+                atomicAdd(&scratch[kMaxWaves + 2], shp.n_row_tiles);
+                atomicMax(&scratch[kMaxWaves + 3], shp.n_tiles);
+            }
+        }
         int tot;
         const int incl = block_inclusive_scan(u, scratch, tot);
         if (sq < a.num_seqs) prefix[sq + 1] = carry + incl;
@@ -520,7 +541,11 @@ DFX_D int build_unit_prefix(const KArgs& a, int* prefix, int* scratch) {
     }
     if (threadIdx.x == 0) prefix[0] = 0;
     __syncthreads();
-    return carry;
+    UnitSummary r;
+    r.per_head = carry;
+    r.items = scratch[kMaxWaves + 2];
+    r.max_tiles = scratch[kMaxWaves + 3];
+    return r;
 }
 
 // The sequence whose unit range contains rem (0 <= rem < per-head total).

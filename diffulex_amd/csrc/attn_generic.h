@@ -208,11 +208,16 @@ __global__ void __launch_bounds__(kThreads) paged_attn_generic_kernel(const KArg
     extern __shared__ __attribute__((aligned(256))) uint8_t smem[];
     GenericAttn<HD, NB, FP8> at(a, smem);
     store_fresh_rows<HD, FP8>(a);
-    const int per_head = build_unit_prefix<Shape<HD, NB>::RT>(a, at.prefix, at.misc);
+    const UnitSummary summary = build_unit_prefix<Shape<HD, NB>::RT>(a, at.prefix, at.misc);
+    const int per_head = summary.per_head;
     const int64_t total = static_cast<int64_t>(per_head) * a.h_kv;
     if (total == 0) return;
     const int w = blockIdx.x;
-    const WgSplit split = make_wg_split(total, a.n_wg);
+    const int n_active = a.fixed_wg ? a.n_wg
+                                    : effective_workgroups(total, static_cast<int64_t>(summary.items) * a.h_kv,
+                                                           summary.max_tiles, a.n_wg);
+    if (w >= n_active) return;
+    const WgSplit split = make_wg_split(total, n_active);
     const int64_t begin = split.first(w);
     const int64_t end = split.first(w + 1);
     if (begin >= end) return;

@@ -321,16 +321,20 @@ __global__ void __launch_bounds__(64 * NW, COMPACT ? 2 : 1) paged_attn_stream_ke
     extern __shared__ __attribute__((aligned(256))) uint8_t smem[];
     using C = StreamCfg<HD, NB, NW, COMPACT>;
     StreamAttn<HD, NB, NW, COMPACT> at(a, smem);
-    at.per_head = build_unit_prefix<C::RT>(a, at.prefix, at.misc);
+    const UnitSummary summary = build_unit_prefix<C::RT>(a, at.prefix, at.misc);
+    at.per_head = summary.per_head;
     const int64_t total = static_cast<int64_t>(at.per_head) * a.h_kv;
     if (total == 0) {
         store_fresh_rows<HD, false>(a);
         return;
     }
     const int w = blockIdx.x;
-    const WgSplit split = make_wg_split(total, a.n_wg);
-    at.begin = split.first(w);
-    at.end = split.first(w + 1);
+    const int n_active = a.fixed_wg ? a.n_wg
+                                    : effective_workgroups(total, static_cast<int64_t>(summary.items) * a.h_kv,
+                                                           summary.max_tiles, a.n_wg);
+    const WgSplit split = make_wg_split(total, n_active);
+    at.begin = w < n_active ? split.first(w) : 0;
+    at.end = w < n_active ? split.first(w + 1) : 0;
     if (at.begin >= at.end) {
         store_fresh_rows<HD, false>(a);
         return;
@@ -396,16 +400,20 @@ __global__ void __launch_bounds__(64 * NW, 1) paged_attn_stream_fp8_kernel(const
     extern __shared__ __attribute__((aligned(256))) uint8_t smem[];
     using C = StreamCfg<HD, 1, NW, false, 1>;
     StreamAttn<HD, 1, NW, false, 1> at(a, smem);
-    at.per_head = build_unit_prefix<C::RT>(a, at.prefix, at.misc);
+    const UnitSummary summary = build_unit_prefix<C::RT>(a, at.prefix, at.misc);
+    at.per_head = summary.per_head;
     const int64_t total = static_cast<int64_t>(at.per_head) * a.h_kv;
     if (total == 0) {
         store_fresh_rows<HD, true>(a);
         return;
     }
     const int w = blockIdx.x;
-    const WgSplit split = make_wg_split(total, a.n_wg);
-    at.begin = split.first(w);
-    at.end = split.first(w + 1);
+    const int n_active = a.fixed_wg ? a.n_wg
+                                    : effective_workgroups(total, static_cast<int64_t>(summary.items) * a.h_kv,
+                                                           summary.max_tiles, a.n_wg);
+    const WgSplit split = make_wg_split(total, n_active);
+    at.begin = w < n_active ? split.first(w) : 0;
+    at.end = w < n_active ? split.first(w + 1) : 0;
     if (at.begin >= at.end) {
         store_fresh_rows<HD, true>(a);
         return;

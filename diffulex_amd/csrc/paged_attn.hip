@@ -211,6 +211,7 @@ extern "C" int dfx_paged_attn(const dfx_attn_params* p, dfx_stream_t stream) {
     ka.dbs = p->diffusion_block_size;
     ka.mask_mode = p->mask_mode;
     ka.n_wg = plan.n_wg;
+    ka.fixed_wg = p->max_workgroups > 0;
     ka.c = p->scale * kLog2e;
 
     hipStream_t st = static_cast<hipStream_t>(stream);

@@ -44,6 +44,22 @@ DFX_HD SeqShape make_seq_shape(int ctx, int q_len, int new_len, int group, int r
     return s;
 }
 
+// How many of the n_wg workgroups of the launch take part.  Cutting an item into p pieces costs
+// a merge whose time grows with p, so a workgroup should own at least about 1.5 * sqrt(tiles of
+// the longest item) units (the point where the time of its own tiles equals the merge time they
+// save), but there is never a reason to use fewer workgroups than there are items.  Small
+// batches with long contexts are the case this matters for.  Integer arithmetic only: every
+// workgroup (and the host-side tests) must arrive at the same number.
+DFX_HD int effective_workgroups(int64_t total_units, int64_t n_items, int max_tiles, int n_wg) {
+    int r = 0;  // floor(1.5 * sqrt(max_tiles))
+    while (static_cast<int64_t>(r + 1) * (r + 1) * 4 <= static_cast<int64_t>(max_tiles) * 9) ++r;
+    const int min_units = r > 4 ? r : 4;
+    int64_t n = (total_units + min_units - 1) / min_units;
+    if (n < n_items) n = n_items;
+    if (n > n_wg) n = n_wg;
+    return n < 1 ? 1 : static_cast<int>(n);
+}
+
 // First unit of workgroup w (w == n_wg gives total).
 DFX_HD int64_t wg_first_unit(int w, int64_t total, int n_wg) { return (static_cast<int64_t>(w) * total) / n_wg; }
 

@@ -163,7 +163,9 @@ typedef struct dfx_attn_params {
     int32_t diffusion_block_size;
     int32_t kv_dtype;            /* dfx_kv_dtype of the caches (k_new/v_new are always bf16) */
     int32_t mask_mode;           /* dfx_mask_mode */
-    int32_t max_workgroups;      /* 0: one per compute unit; >0: exactly this many persistent workgroups */
+    int32_t max_workgroups;      /* 0: up to one (two for small row counts) per compute unit, fewer when the
+                                    batch is small (chosen on the device from the lengths); >0: exactly this
+                                    many persistent workgroups */
     int32_t flags;               /* DFX_ATTN_* bits, 0 by default */
     float scale;
     /* Fused KV-cache store (the store + decode pair of diffulex/attention/attn_impl.py:54-69 in

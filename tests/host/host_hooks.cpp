@@ -20,6 +20,10 @@ void hook_bf16_round(const float* x, uint16_t* out, int64_t n) {
     for (int64_t i = 0; i < n; ++i) out[i] = dfx::f32_to_bf16_bits(x[i]);
 }
 
+int hook_effective_workgroups(int64_t total_units, int64_t n_items, int max_tiles, int n_wg) {
+    return dfx::effective_workgroups(total_units, n_items, max_tiles, n_wg);
+}
+
 // Replays the persistent kernel's walk over its unit range on the host.  For workgroup w it
 // appends one record per segment: {w, kv_head, seq, row_tile, tile0, tile1, complete, slot}.
 // ctx/q_len/new_len: per-sequence lengths.  Returns the number of records (<= cap).

@@ -23,6 +23,8 @@ def load():
     lib.hook_quantise_e4m3.argtypes = [vp, C.c_float, vp, i64]
     lib.hook_e4m3_to_f32.argtypes = [vp, vp, i64]
     lib.hook_bf16_round.argtypes = [vp, vp, i64]
+    lib.hook_effective_workgroups.restype = i32
+    lib.hook_effective_workgroups.argtypes = [i64, i64, i32, i32]
     lib.hook_walk_segments.restype = i64
     lib.hook_walk_segments.argtypes = [vp, vp, vp, i32, i32, i32, i32, i32, vp, i64]
     lib.hook_combine_slots.restype = i32

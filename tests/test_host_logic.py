@@ -152,3 +152,21 @@ def test_partition_covers_every_tile_once_and_combine_finds_the_pieces(seed):
     assert len(seen) == sum(1 for kvh in range(h_kv) for s in range(b)
                             for rt in range(-(-group * int(q_len[s]) // rows_per_tile))
                             if -(-int(ctx[s]) // 64) + -(-int(new_len[s]) // 64) > 0)
+
+
+def test_number_of_participating_workgroups():
+    """Small batches use fewer workgroups (a cut item costs a merge that grows with its pieces),
+    never fewer than there are items, never more than launched; large batches use them all."""
+    f = hosthooks.load().hook_effective_workgroups
+    import math
+    for max_tiles in (1, 2, 9, 33, 129, 513, 5000):
+        r = math.isqrt(9 * max_tiles // 4)                      # floor(1.5 sqrt(max_tiles))
+        min_units = max(4, r)
+        for n_items in (1, 4, 32, 256, 4096):
+            total = n_items * max_tiles
+            for n_wg in (1, 64, 256, 512):
+                want = max(1, min(n_wg, max(n_items, -(-total // min_units))))
+                assert f(total, n_items, max_tiles, n_wg) == want
+    assert f(64 * 4 * 21, 256, 33, 256) == 256        # Dream-7B shape, batch 64: every compute unit
+    assert f(4 * 33, 4, 33, 256) == 17                # batch 1, 2K context: 132 units at >= 8 per workgroup
+    assert f(4 * 513, 4, 513, 256) == 63              # batch 1, 32K context

@@ -62,7 +62,7 @@ struct Shape {
     static constexpr int NSLAB = HD / 16;        // contraction slabs of Q K^T
     static constexpr int NDB = HD / 32;          // 32-row blocks of O^T
     static constexpr int PREFIX_BYTES = (kMaxSeqs + 1) * 4;
-    static constexpr int MISC_BYTES = 64;
+    static constexpr int MISC_BYTES = 128;
     // A partial result is stored per 32-row query block b = wave * NB + qb, whatever the shape of
     // the workgroup that wrote it: NDB * 4 float4 per lane of O^T, then the running maximum and
     // the row sum of the lane's query.
@@ -516,35 +516,48 @@ struct UnitSummary {
 
 template <int RT>
 DFX_D UnitSummary build_unit_prefix(const KArgs& a, int* prefix, int* scratch) {
-    int carry = 0;
+    // scratch: [0, kMaxWaves) is used by the scan, [16, 16 + kMaxWaves) and [24, 24 + kMaxWaves) hold
+    // per-wave item counts and tile maxima (register reductions; atomics on one LDS word from
+    // every lane cost microseconds here)
+    int carry = 0, items = 0, max_tiles = 0;
     const int n_threads = blockDim.x;
-    if (threadIdx.x == 0) {
-        scratch[kMaxWaves + 2] = 0;
-        scratch[kMaxWaves + 3] = 0;
-    }
-    __syncthreads();
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, n_waves = blockDim.x >> 6;
     for (int base = 0; base < a.num_seqs; base += n_threads) {
         const int sq = base + threadIdx.x;
-        int u = 0;
+        int u = 0, rows = 0, tiles = 0;
         if (sq < a.num_seqs) {
             const SeqShape shp = load_seq_shape(a, sq, RT);
             u = shp.units;
             if (u > 0) {
-                atomicAdd(&scratch[kMaxWaves + 2], shp.n_row_tiles);
-                atomicMax(&scratch[kMaxWaves + 3], shp.n_tiles);
+                rows = shp.n_row_tiles;
+                tiles = shp.n_tiles;
             }
         }
+#pragma unroll
+        for (int d = 32; d >= 1; d >>= 1) {
+            rows += __shfl_xor(rows, d);
+            tiles = max(tiles, __shfl_xor(tiles, d));
+        }
+        if (lane == 0) {
+            scratch[16 + wave] = rows;
+            scratch[24 + wave] = tiles;
+        }
         int tot;
-        const int incl = block_inclusive_scan(u, scratch, tot);
+        const int incl = block_inclusive_scan(u, scratch, tot);  // (its barriers also publish the two arrays)
         if (sq < a.num_seqs) prefix[sq + 1] = carry + incl;
         carry += tot;
+        for (int w = 0; w < n_waves; ++w) {
+            items += scratch[16 + w];
+            max_tiles = max(max_tiles, scratch[24 + w]);
+        }
+        if (base + n_threads < a.num_seqs) __syncthreads();  // before the next round overwrites the arrays
     }
     if (threadIdx.x == 0) prefix[0] = 0;
     __syncthreads();
     UnitSummary r;
     r.per_head = carry;
-    r.items = scratch[kMaxWaves + 2];
-    r.max_tiles = scratch[kMaxWaves + 3];
+    r.items = items;
+    r.max_tiles = max_tiles;
     return r;
 }
 

@@ -321,13 +321,13 @@ __global__ void __launch_bounds__(64 * NW, COMPACT ? 2 : 1) paged_attn_stream_ke
     extern __shared__ __attribute__((aligned(256))) uint8_t smem[];
     using C = StreamCfg<HD, NB, NW, COMPACT>;
     StreamAttn<HD, NB, NW, COMPACT> at(a, smem);
+    // The fused cache store comes first, while next to nothing is live in registers: anywhere
+    // later its address arithmetic would push values of the tile loop out of their registers.
+    store_fresh_rows<HD, false>(a);
     const UnitSummary summary = build_unit_prefix<C::RT>(a, at.prefix, at.misc);
     at.per_head = summary.per_head;
     const int64_t total = static_cast<int64_t>(at.per_head) * a.h_kv;
-    if (total == 0) {
-        store_fresh_rows<HD, false>(a);
-        return;
-    }
+    if (total == 0) return;
     const int w = blockIdx.x;
     const int n_active = a.fixed_wg ? a.n_wg
                                     : effective_workgroups(total, static_cast<int64_t>(summary.items) * a.h_kv,
@@ -335,10 +335,7 @@ __global__ void __launch_bounds__(64 * NW, COMPACT ? 2 : 1) paged_attn_stream_ke
     const WgSplit split = make_wg_split(total, n_active);
     at.begin = w < n_active ? split.first(w) : 0;
     at.end = w < n_active ? split.first(w + 1) : 0;
-    if (at.begin >= at.end) {
-        store_fresh_rows<HD, false>(a);
-        return;
-    }
+    if (at.begin >= at.end) return;
     const int64_t begin = at.begin, end = at.end;
 
     for (int64_t chunk = begin; chunk < end; chunk += C::kPlanUnits) {
@@ -353,8 +350,6 @@ __global__ void __launch_bounds__(64 * NW, COMPACT ? 2 : 1) paged_attn_stream_ke
         if (opens) at.begin_item(at.units[0], false);
         int issued = 0;  // ring fill: kStages - 1 units in flight
         for (; issued < C::kStages - 1 && issued < n_units; ++issued) at.issue_unit(issued);
-        // the fused cache store runs here, once, while the first tiles and the query rows are on their way
-        if (chunk == begin) store_fresh_rows<HD, false>(a);
         at.touch_queries();  // unconditional: the compiler must see no path into the tile loop with these loads pending
 
         int rel = 0;
@@ -400,13 +395,11 @@ __global__ void __launch_bounds__(64 * NW, 1) paged_attn_stream_fp8_kernel(const
     extern __shared__ __attribute__((aligned(256))) uint8_t smem[];
     using C = StreamCfg<HD, 1, NW, false, 1>;
     StreamAttn<HD, 1, NW, false, 1> at(a, smem);
+    store_fresh_rows<HD, true>(a);  // first, as in the bf16 kernel
     const UnitSummary summary = build_unit_prefix<C::RT>(a, at.prefix, at.misc);
     at.per_head = summary.per_head;
     const int64_t total = static_cast<int64_t>(at.per_head) * a.h_kv;
-    if (total == 0) {
-        store_fresh_rows<HD, true>(a);
-        return;
-    }
+    if (total == 0) return;
     const int w = blockIdx.x;
     const int n_active = a.fixed_wg ? a.n_wg
                                     : effective_workgroups(total, static_cast<int64_t>(summary.items) * a.h_kv,
@@ -414,10 +407,7 @@ __global__ void __launch_bounds__(64 * NW, 1) paged_attn_stream_fp8_kernel(const
     const WgSplit split = make_wg_split(total, n_active);
     at.begin = w < n_active ? split.first(w) : 0;
     at.end = w < n_active ? split.first(w + 1) : 0;
-    if (at.begin >= at.end) {
-        store_fresh_rows<HD, true>(a);
-        return;
-    }
+    if (at.begin >= at.end) return;
     const int64_t begin = at.begin, end = at.end;
 
     for (int64_t chunk = begin; chunk < end; chunk += C::kPlanUnits) {
@@ -430,8 +420,6 @@ __global__ void __launch_bounds__(64 * NW, 1) paged_attn_stream_fp8_kernel(const
         if (opens) at.begin_item(at.units[0], false);  // query rows ahead of the ring fill, as in the bf16 kernel
         int issued = 0;
         for (; issued < C::kStages - 1 && issued < n_units; ++issued) at.issue_unit(issued);
-        // the fused cache store runs here, once, while the first tiles and the query rows are on their way
-        if (chunk == begin) store_fresh_rows<HD, true>(a);
         at.touch_queries();  // unconditional: the compiler must see no path into the tile loop with these loads pending
         at.wait_younger(issued - 1);
         at.widen_unit(0);

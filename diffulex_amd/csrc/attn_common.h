@@ -114,6 +114,10 @@ struct TileInfo {
     bool is_ctx;
     float c_tile;  // logit -> log2 domain factor (scale * log2 e, times k_scale for FP8 context)
     float v_mul;   // factor applied to P before the PV product (v_scale for FP8 context, else 1)
+    uint64_t holes;  // bit b: tokens base + b * HOLE_ROWS .. + HOLE_ROWS - 1 (HOLE_ROWS: a parameter of
+                     // softmax_tile) sit on a page whose block-table entry is negative or out of range
+                     // and are skipped, as the reference skips such pages
+                     // (diffulex_kernel/python/dllm_flash_attn.py:260-261)
 };
 
 template <int HD, int NB, int NW = kWaves>
@@ -149,6 +153,7 @@ struct AttnState {
         t.limit = t.is_ctx ? shp.ctx : shp.new_len;
         t.c_tile = a.c;
         t.v_mul = 1.0f;
+        t.holes = 0;
         if (fp8 && t.is_ctx) {
             t.c_tile = fmaxf(a.c * a.k_scale[kv_head], 1e-30f);
             t.v_mul = a.v_scale[kv_head];
@@ -194,12 +199,15 @@ struct AttnState {
     // rescales o when a row maximum grows.  pb[qb][tb][sl] is the B operand of the PV product.
     // before_rescale() runs ahead of any vector-ALU access to o (kernels that issue their matrix
     // instructions behind the compiler's back insert the required wait states there).
-    template <bool SCALE_P, typename BeforeRescale>
+    template <bool SCALE_P, int HOLE_ROWS, typename BeforeRescale>
     DFX_D void softmax_tile(f32x16 (&sc)[2][NB], const TileInfo& t, bf16x8 (&pb)[NB][2][2],
                             BeforeRescale&& before_rescale) {
         const bool mask_valid = t.base + S::TN > t.limit;
         const bool mask_bc = !t.is_ctx && a.mask_mode == DFX_MASK_BLOCK_CAUSAL;
-        if (mask_valid || mask_bc) {
+        static_assert(HOLE_ROWS == 1 || HOLE_ROWS % 8 == 0, "a lane's 4 * half offset must stay inside a hole unit");
+        if (mask_valid || mask_bc || t.holes != 0) {
+            // token-granular holes: this lane's tokens sit 4 * half higher
+            const uint64_t holes = (HOLE_ROWS == 1 && half) ? (t.holes >> 4) : t.holes;
 #pragma unroll
             for (int qb = 0; qb < NB; ++qb) {
                 int lim = t.limit;
@@ -208,8 +216,9 @@ struct AttnState {
                 for (int tb = 0; tb < 2; ++tb)
 #pragma unroll
                     for (int e = 0; e < 16; ++e) {
-                        const int tok = t.base + tb * 32 + (e >> 2) * 8 + half * 4 + (e & 3);
-                        if (tok >= lim) sc[tb][qb][e] = -INFINITY;
+                        const int in_tile = tb * 32 + (e >> 2) * 8 + (e & 3);
+                        const int tok = t.base + in_tile + half * 4;
+                        if (tok >= lim || ((holes >> (in_tile / HOLE_ROWS)) & 1)) sc[tb][qb][e] = -INFINITY;
                     }
             }
         }

@@ -172,11 +172,17 @@ struct GenericAttn : TileMath<HD, NB, kWaves> {
 
     // one tile of attention from LDS
     DFX_D void compute(int buf, int tile) {
-        const TileInfo t = this->tile_info(sh, kvh, tile, FP8);
+        TileInfo t = this->tile_info(sh, kvh, tile, FP8);
+        if (t.is_ctx) {  // tokens on pages without a valid block-table entry are skipped: one token per lane
+            const int tok = t.base + this->lane;
+            bool ok = true;
+            if (tok < t.limit) cache_row_offset(tok, ok);
+            t.holes = __ballot(!ok);
+        }
         f32x16 sc[2][NB];
         this->scores(k_stage(buf), sc);
         bf16x8 pb[NB][2][2];
-        this->template softmax_tile<FP8>(sc, t, pb, [&] { this->outputs_ready(); });
+        this->template softmax_tile<FP8, 1>(sc, t, pb, [&] { this->outputs_ready(); });
         this->accumulate(v_stage(buf), pb);
     }
 

@@ -41,7 +41,7 @@ struct BandDesc {
     int32_t last;  // last valid row of the band; later rows re-read it
     int32_t is_ctx;
 };
-enum : int32_t { kUnitCtx = 1, kUnitFirst = 2, kUnitLast = 4, kUnitComplete = 8 };
+enum : int32_t { kUnitCtx = 1, kUnitFirst = 2, kUnitLast = 4, kUnitComplete = 8, kUnitHoleShift = 8 };
 
 // COMPACT: a configuration small enough (2 stages, short plan, at most kCompactMaxSeqs sequences)
 // for two workgroups to share a compute unit.  Items with at most 128 rows run with four waves,
@@ -176,11 +176,14 @@ struct StreamAttn : TileMath<HD, NB, NW> {
             }
             // Rows past the end re-read the last valid rows (finite data; their scores are masked).
             int band = base + w * C::ROWS_PER_WAVE;
-            if (band >= limit) band = ((limit - 1) / C::ROWS_PER_WAVE) * C::ROWS_PER_WAVE;
+            const bool past_end = band >= limit;
+            if (past_end) band = ((limit - 1) / C::ROWS_PER_WAVE) * C::ROWS_PER_WAVE;
             BandDesc b;
+            bool hole = false;  // the band's page has no valid block-table entry: its tokens are skipped
             if (is_ctx) {
                 const int p = a.page_shift >= 0 ? (band >> a.page_shift) : (band / a.page_size);
-                int64_t page = p < a.max_pages ? a.block_tables[static_cast<int64_t>(sq) * a.bt_stride + p] : 0;
+                int64_t page = p < a.max_pages ? a.block_tables[static_cast<int64_t>(sq) * a.bt_stride + p] : -1;
+                hole = !past_end && (page < 0 || page >= a.n_pages);
                 page = page < 0 ? 0 : (page >= a.n_pages ? a.n_pages - 1 : page);
                 b.off = (page * a.c_sp + static_cast<int64_t>(band - p * a.page_size) * a.c_st + kv_head * a.c_sh) * KVB;
             } else {
@@ -189,6 +192,10 @@ struct StreamAttn : TileMath<HD, NB, NW> {
             b.last = limit - 1 - band;
             b.is_ctx = is_ctx ? 1 : 0;
             bands[slot_in_ring * NW + w] = b;
+            // the NW lanes of a unit are neighbours in a wave: its holes as a bit per band
+            const uint64_t votes = __ballot(hole);
+            const int holes = static_cast<int>((votes >> ((threadIdx.x & 63) & ~(NW - 1))) & ((1u << NW) - 1));
+            if (w == 0 && holes != 0) units[slot_in_ring].flags |= holes << kUnitHoleShift;
         }
     }
 
@@ -371,13 +378,14 @@ __global__ void __launch_bounds__(64 * NW, COMPACT ? 2 : 1) paged_attn_stream_ke
                 t.base = uniform(u.base);
                 t.limit = uniform(u.limit);
                 t.is_ctx = (uniform(u.flags) & kUnitCtx) != 0;
+                t.holes = static_cast<uint32_t>(uniform(u.flags)) >> kUnitHoleShift;  // a bit per band of rows
                 t.c_tile = a.c;
                 t.v_mul = 1.0f;
                 const uint8_t* k_tile = smem + C::STAGES_OFF + (rel % C::kStages) * C::STAGE_BYTES;
                 f32x16 sc[2][NB];
                 at.scores(k_tile, sc);
                 bf16x8 pb[NB][2][2];
-                at.template softmax_tile<false>(sc, t, pb, [&] { at.outputs_ready(); });
+                at.template softmax_tile<false, C::ROWS_PER_WAVE>(sc, t, pb, [&] { at.outputs_ready(); });
                 at.accumulate(k_tile + C::MAT_BYTES, pb);
             }
             at.finish_run(rel - 1, split);
@@ -443,13 +451,14 @@ __global__ void __launch_bounds__(64 * NW, 1) paged_attn_stream_fp8_kernel(const
                 t.base = uniform(u.base);
                 t.limit = uniform(u.limit);
                 t.is_ctx = (uniform(u.flags) & kUnitCtx) != 0;
+                t.holes = static_cast<uint32_t>(uniform(u.flags)) >> kUnitHoleShift;  // a bit per band of rows
                 t.c_tile = t.is_ctx ? a.c * at.k_mul : a.c;
                 t.v_mul = t.is_ctx ? at.v_mul : 1.0f;
                 const uint8_t* k_tile = at.wide_tile(rel);
                 f32x16 sc[2][1];
                 at.scores(k_tile, sc);
                 bf16x8 pb[1][2][2];
-                at.template softmax_tile<true>(sc, t, pb, [&] { at.outputs_ready(); });
+                at.template softmax_tile<true, C::ROWS_PER_WAVE>(sc, t, pb, [&] { at.outputs_ready(); });
                 at.accumulate(k_tile + TileLayout<HD>::MAT_BYTES, pb);
             }
             at.finish_run(rel - 1, split);

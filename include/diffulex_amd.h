@@ -141,7 +141,8 @@ typedef struct dfx_attn_params {
     const void* k_cache;         /* [n_pages, page_size, num_kv_heads, head_dim]; NULL: no cached context */
     const void* v_cache;
     void* out;                   /* [T_q, num_q_heads, head_dim] bf16 */
-    const int32_t* block_tables; /* [num_seqs, block_table_stride]; entries < 0 are never dereferenced */
+    const int32_t* block_tables; /* [num_seqs, block_table_stride]; a page whose entry is < 0 (or >= n_pages) is
+                                    skipped: its tokens take no part, as in the reference (dllm_flash_attn.py:260-261) */
     const int32_t* context_lens; /* [num_seqs]; NULL means 0 everywhere */
     const int32_t* cu_seqlens_q;   /* [num_seqs + 1] */
     const int32_t* cu_seqlens_new; /* [num_seqs + 1] offsets of the fresh K/V rows */

@@ -100,7 +100,7 @@ def paged_attention_fp32(q, k_new, v_new, k_cache, v_cache, block_tables, contex
         if ctx > 0:
             kc = gather_context(k_cache, block_tables[s], ctx, page)
             vc = gather_context(v_cache, block_tables[s], ctx, page)
-            assert kc.shape[0] == ctx
+            ctx = kc.shape[0]  # fewer than context_len if pages were skipped (negative table entries)
             if k_cache.element_size() == 1:
                 kc, vc = _dequant(kc, k_scale), _dequant(vc, v_scale)
             kk = torch.cat([kc.float(), k_new[n0:n1].float()], 0)
@@ -142,6 +142,7 @@ def paged_attention_sdpa(q, k_new, v_new, k_cache, v_cache, block_tables, contex
         if ctx > 0:
             kc = gather_context(k_cache, block_tables[s], ctx, page)
             vc = gather_context(v_cache, block_tables[s], ctx, page)
+            ctx = kc.shape[0]  # fewer than context_len if pages were skipped
             if k_cache.element_size() == 1:
                 kc, vc = _dequant(kc, k_scale), _dequant(vc, v_scale)
             ks = torch.cat([kc.to(dt), ks], 0)

@@ -353,3 +353,33 @@ def test_store_fused_into_the_attention_launch(dev, name, over, flags):
             assert torch.equal(kc_b.view(torch.uint8), kc_a.view(torch.uint8))
             assert torch.equal(vc_b.view(torch.uint8), vc_a.view(torch.uint8))
             assert not torch.equal(kc_b.view(torch.uint8), wl.k_cache.view(torch.uint8))  # something was stored
+
+
+@pytest.mark.parametrize("flags", PATHS)
+@pytest.mark.parametrize("name,over", [
+    ("c1", dict(num_seqs=3, ctx=[100, 64, 37])),                       # page 16: four pages per tile
+    ("c3", dict(num_seqs=4, ctx=[700, 256, 1000, 90], page=32)),
+    ("c3", dict(num_seqs=3, ctx=[700, 513, 1000])),                    # page 256: whole tiles vanish
+    ("c5", dict(num_seqs=3, ctx=[700, 513, 1000])),
+    ("c4", dict(num_seqs=2, ctx=[300, 95], page=48)),
+])
+def test_pages_with_negative_table_entries_are_skipped(dev, name, over, flags):
+    """The reference skips a page whose block-table entry is negative: its tokens take no part
+    (diffulex_kernel/python/dllm_flash_attn.py:260-261; the oracle follows
+    tests/python/kernel/test_dllm_flash_attn_decode_kernel.py:63-76)."""
+    wl = make_workload(name, seed=61, **over)
+    bt = wl.block_tables.clone()
+    page = wl.page_size
+    for s in range(wl.num_seqs):
+        n_ctx_pages = -(-int(wl.context_lens[s]) // page)
+        for p in range(n_ctx_pages):
+            if (p + s) % 3 == 1:
+                bt[s, p] = -1
+    bt[0, 0] = wl.k_cache.shape[0] + 7        # out of range counts as missing too
+    wl.block_tables = bt
+    want = oracle_fp32(wl, block_tables=torch.where(bt >= wl.k_cache.shape[0], torch.full_like(bt, -1), bt))
+    g = wl.to(dev)
+    tol = ATOL_FP8 if name == "c5" else ATOL_BF16
+    for max_wg in (0, 3):
+        got = _run(g, max_wg, flags=flags)
+        assert max_abs_err(got, want) <= tol

@@ -90,6 +90,34 @@ def test_permuting_physical_pages_with_the_table_is_a_no_op():
     assert torch.equal(got, base)
 
 
+@pytest.mark.parametrize("mask", [MASK_FULL, MASK_BLOCK_CAUSAL])
+def test_a_skipped_page_is_the_same_as_a_shorter_context_without_it(mask):
+    """Negative table entries drop their page's tokens (dllm_flash_attn.py:260-261): the result is
+    that of a sequence whose context simply lacks those tokens (table compacted, length reduced)."""
+    wl = make_workload("c4", num_seqs=2, ctx=[100, 70], page=16, mask=mask, seed=13)
+    bt = wl.block_tables.clone()
+    bt[0, 1] = -1
+    bt[0, 4] = -1
+    bt[1, 0] = -1
+    holed = _run_fp32(wl, block_tables=bt)
+    # the same thing spelled without holes: drop the entries, shorten the contexts by whole pages
+    bt2 = torch.full_like(bt, -1)
+    ctx2 = wl.context_lens.clone()
+    for s in range(2):
+        n_ctx_pages = -(-int(wl.context_lens[s]) // 16)
+        kept = [int(x) for x in bt[s, :n_ctx_pages] if x >= 0]
+        assert int(wl.context_lens[s]) % 16 != 0 and bt[s, n_ctx_pages - 1] >= 0   # the partial last page stays last
+        bt2[s, :len(kept)] = torch.tensor(kept, dtype=bt.dtype)
+        ctx2[s] -= 16 * (n_ctx_pages - len(kept))
+    plain = _run_fp32(wl, block_tables=bt2, context_lens=ctx2)
+    assert torch.equal(holed, plain)
+    assert not torch.equal(holed, _run_fp32(wl))
+    lib = oat.paged_attention_sdpa(wl.q, wl.k_new, wl.v_new, wl.k_cache, wl.v_cache, bt, wl.context_lens,
+                                   wl.cu_seqlens_q, wl.cu_seqlens_q, wl.scale, mask_mode=mask,
+                                   dbs=wl.diffusion_block_size, compute_dtype=torch.float32)
+    assert float((lib - holed).abs().max()) < 2e-5
+
+
 def test_repaging_the_same_context_is_a_no_op():
     wl = make_workload("c1")          # page 16
     base = _run_fp32(wl)

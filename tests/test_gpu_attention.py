@@ -383,3 +383,31 @@ def test_pages_with_negative_table_entries_are_skipped(dev, name, over, flags):
     for max_wg in (0, 3):
         got = _run(g, max_wg, flags=flags)
         assert max_abs_err(got, want) <= tol
+
+
+@pytest.mark.parametrize("name,over,tol", [
+    # more sequences than the two-workgroups-per-CU variant plans for (1023): the one-per-CU variants
+    ("c3", dict(num_seqs=1500, ctx=(0, 150), h_q=8, h_kv=2), ATOL_BF16),
+    ("c1", dict(num_seqs=1100, ctx=(0, 90), h_q=4, h_kv=4), ATOL_BF16),
+    ("c5", dict(num_seqs=1200, ctx=(0, 200), h_q=8, h_kv=2), ATOL_FP8),
+    # the largest batch the kernels take
+    ("c3", dict(num_seqs=4095, ctx=(0, 40), h_q=4, h_kv=1, q_len=32), ATOL_BF16),
+])
+def test_many_short_sequences(dev, name, over, tol):
+    wl = make_workload(name, seed=71, **over)
+    g = wl.to(dev)
+    seqs = [0, 1, wl.num_seqs // 2, wl.num_seqs - 2, wl.num_seqs - 1]
+    want = oracle_fp32(wl, seqs=seqs)
+    cu = wl.cu_seqlens_q.tolist()
+    for flags in PATHS:
+        got = _run(g, flags=flags)
+        assert torch.isfinite(got.float()).all()
+        for s, w in zip(seqs, want):
+            assert max_abs_err(got[cu[s]:cu[s + 1]], w) <= tol
+    assert max_abs_err(_run(g), _run(g, max_workgroups=64)) <= 1e-2   # another partition: rounding differences only
+
+
+def test_batch_above_the_limit_is_refused(dev):
+    wl = make_workload("c1", num_seqs=4096, ctx=(0, 20), seed=3).to(dev)
+    with pytest.raises(Exception):
+        _run(wl)

@@ -49,6 +49,7 @@ struct KArgs {
     int64_t bt_stride, n_pages;
     int num_seqs, h_kv, group, page_size, page_shift, max_pages, dbs, mask_mode, n_wg;
     int fixed_wg;  // the caller fixed the number of workgroups: all of them take part
+    int busy_waves;  // streaming kernels: waves from this one on have query rows in no item of the launch
     float c;  // scale * log2(e)
 };
 

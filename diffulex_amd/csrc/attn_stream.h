@@ -382,11 +382,13 @@ __global__ void __launch_bounds__(64 * NW, COMPACT ? 2 : 1) paged_attn_stream_ke
                 t.c_tile = a.c;
                 t.v_mul = 1.0f;
                 const uint8_t* k_tile = smem + C::STAGES_OFF + (rel % C::kStages) * C::STAGE_BYTES;
-                f32x16 sc[2][NB];
-                at.scores(k_tile, sc);
-                bf16x8 pb[NB][2][2];
-                at.template softmax_tile<false, C::ROWS_PER_WAVE>(sc, t, pb, [&] { at.outputs_ready(); });
-                at.accumulate(k_tile + C::MAT_BYTES, pb);
+                if (at.wave < a.busy_waves) {  // waves whose 32 rows exist in no item of this launch only fetch
+                    f32x16 sc[2][NB];
+                    at.scores(k_tile, sc);
+                    bf16x8 pb[NB][2][2];
+                    at.template softmax_tile<false, C::ROWS_PER_WAVE>(sc, t, pb, [&] { at.outputs_ready(); });
+                    at.accumulate(k_tile + C::MAT_BYTES, pb);
+                }
             }
             at.finish_run(rel - 1, split);
         }
@@ -455,11 +457,13 @@ __global__ void __launch_bounds__(64 * NW, 1) paged_attn_stream_fp8_kernel(const
                 t.c_tile = t.is_ctx ? a.c * at.k_mul : a.c;
                 t.v_mul = t.is_ctx ? at.v_mul : 1.0f;
                 const uint8_t* k_tile = at.wide_tile(rel);
-                f32x16 sc[2][1];
-                at.scores(k_tile, sc);
-                bf16x8 pb[1][2][2];
-                at.template softmax_tile<true, C::ROWS_PER_WAVE>(sc, t, pb, [&] { at.outputs_ready(); });
-                at.accumulate(k_tile + TileLayout<HD>::MAT_BYTES, pb);
+                if (at.wave < a.busy_waves) {
+                    f32x16 sc[2][1];
+                    at.scores(k_tile, sc);
+                    bf16x8 pb[1][2][2];
+                    at.template softmax_tile<true, C::ROWS_PER_WAVE>(sc, t, pb, [&] { at.outputs_ready(); });
+                    at.accumulate(k_tile + TileLayout<HD>::MAT_BYTES, pb);
+                }
             }
             at.finish_run(rel - 1, split);
         }

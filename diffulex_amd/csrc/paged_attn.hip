@@ -212,6 +212,10 @@ extern "C" int dfx_paged_attn(const dfx_attn_params* p, dfx_stream_t stream) {
     ka.mask_mode = p->mask_mode;
     ka.n_wg = plan.n_wg;
     ka.fixed_wg = p->max_workgroups > 0;
+    {
+        const int64_t rows = static_cast<int64_t>(ka.group) * p->max_seqlen_q;
+        ka.busy_waves = static_cast<int>(rows >= 32 * kMaxWaves ? kMaxWaves : (rows + 31) / 32);
+    }
     ka.c = p->scale * kLog2e;
 
     hipStream_t st = static_cast<hipStream_t>(stream);

@@ -1,4 +1,5 @@
-// Streaming tile path of the paged-attention kernel (bf16 KV, page_size a multiple of 16).
+// Streaming tile path of the paged-attention kernels (page_size a multiple of 16; bf16 KV, or
+// FP8-E4M3 KV with head_dim 128: see the second kernel below).
 //
 // K/V tiles go HBM -> LDS directly (global_load_lds_dwordx4, 16 bytes per lane, never through
 // registers) into a ring of kStages stages, so several tiles are in flight per compute unit
@@ -7,7 +8,7 @@
 // item is finished.
 //
 // Everything data dependent about a unit (which sequence / head / tile it is, where its rows
-// start in memory, whether it opens or closes an item) is worked out ahead of time by all 256
+// start in memory, whether it opens or closes an item) is worked out ahead of time by all
 // lanes in parallel and kept in a small LDS table, kPlanUnits units at a time.  The tile loop
 // itself reads that table and issues nothing to memory but the asynchronous tile loads, so
 // their in-order completion counter can be waited on exactly.
@@ -26,8 +27,8 @@
 
 namespace dfx {
 
-// One unit of the plan: wave-uniform facts (UnitDesc) and the start of each wave's 16-row
-// band of the tile in memory (BandDesc).
+// One unit of the plan: wave-uniform facts (UnitDesc) and the start of each wave's band of
+// rows of the tile in memory (BandDesc; 64 / waves rows per band).
 struct UnitDesc {
     int32_t s, kvh, rt, q0;
     int32_t q_len, base, limit, flags;
@@ -200,7 +201,7 @@ struct StreamAttn : TileMath<HD, NB, NW> {
     }
 
     // ---- loads -----------------------------------------------------------------------------
-    // Start the loads of planned unit `rel` (this wave's 16-row band of K and V) into its ring stage.
+    // Start the loads of planned unit `rel` (this wave's band of K and V rows) into its ring stage.
     DFX_D void issue_unit(int rel) const {
         const BandDesc b = bands[rel * NW + wave];
         const int last = uniform(b.last);

@@ -6,8 +6,9 @@
 //     units(s) = n_tiles(s) * n_row_tiles(s)
 // consecutive units (row-tile major), the sequences follow each other, and the whole list is
 // repeated for every KV head.  The linear unit space [0, total) is cut into n_wg equal
-// ranges, one per persistent workgroup; wherever a cut falls inside a (sequence, head, row
-// tile) item the two sides produce partial results that a combine pass merges.
+// ranges, one per participating workgroup; wherever a cut falls inside a (sequence, head, row
+// tile) item the sides produce partial results, which the workgroup that finishes its piece
+// last merges.
 #pragma once
 
 #include <stdint.h>

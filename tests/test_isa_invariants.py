@@ -1,0 +1,78 @@
+"""What the compiler made of the streaming kernels' tile loops (CPU test: hipcc cross-compiles).
+
+The asynchronous tile loads are waited for by hand (exact ``s_waitcnt vmcnt(n)``), which only
+works while the compiler has no reason to wait inside the loop itself: a load of its own that is
+pending on some path into the loop, or a register spilled to scratch, makes it drain the load
+queue in every iteration.  Such regressions cost 10-30 % and change no result, so they are
+checked on the generated code: per tile loop the expected matrix instructions, no scratch access, and no
+``vmcnt`` wait beyond the hand-placed ones.
+"""
+import collections
+import re
+import shutil
+import subprocess
+from pathlib import Path
+
+import pytest
+
+from diffulex_amd import build as dbuild
+
+ROOT = Path(__file__).resolve().parent.parent
+
+
+@pytest.fixture(scope="module")
+def isa(tmp_path_factory):
+    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not Path(hipcc).exists():
+        pytest.skip("hipcc not available")
+    out = tmp_path_factory.mktemp("isa") / "paged_attn.s"
+    cmd = [hipcc, *dbuild.HIP_FLAGS, "-I", str(ROOT / "include"), "-S", "--cuda-device-only", "-x", "hip",
+           str(ROOT / "diffulex_amd" / "csrc" / "paged_attn.hip"), "-o", str(out)]
+    subprocess.run(cmd, check=True, capture_output=True)
+    return out.read_text()
+
+
+def _tile_loop(isa_text, mangled_prefix):
+    """Instructions of the innermost loop that contains every matrix instruction of the kernel."""
+    m = re.search(r"^(%s\w*):" % re.escape(mangled_prefix), isa_text, re.M)
+    assert m, mangled_prefix
+    body = [l.strip() for l in isa_text[m.start():isa_text.index("s_endpgm", m.start())].split("\n")]
+    mfma = [i for i, l in enumerate(body) if l.startswith("v_mfma")]
+    labels = {mm.group(1): i for i, l in enumerate(body) for mm in [re.match(r"^(\.LBB\d+_\d+):", l)] if mm}
+    best = None
+    for i, l in enumerate(body):
+        mm = re.search(r"s_c?branch\S*\s+(\.LBB\d+_\d+)", l)
+        if mm and mm.group(1) in labels:
+            t = labels[mm.group(1)]
+            if t < mfma[0] and i > mfma[-1] and (best is None or i - t < best[1] - best[0]):
+                best = (t, i)
+    assert best, "no loop around the matrix instructions"
+    return [l for l in body[best[0]:best[1] + 1] if l and not l.startswith((";", "."))]
+
+
+# kernel, hand-placed vmcnt waits in its loop (three alternatives of wait_younger; the FP8 kernel
+# also waits inside the branch that copies fresh bf16 rows, once per load round of a wave)
+KERNELS = [
+    ("_ZN3dfx24paged_attn_stream_kernelILi128ELi1ELi8ELb0E", 3),
+    ("_ZN3dfx24paged_attn_stream_kernelILi128ELi1ELi4ELb1E", 3),
+    ("_ZN3dfx24paged_attn_stream_kernelILi128ELi1ELi4ELb0E", 3),
+    ("_ZN3dfx24paged_attn_stream_kernelILi64ELi1ELi8ELb0E", 3),
+    ("_ZN3dfx24paged_attn_stream_kernelILi64ELi1ELi4ELb1E", 3),
+    ("_ZN3dfx28paged_attn_stream_fp8_kernelILi128ELi8E", 3 + 2),
+    ("_ZN3dfx28paged_attn_stream_fp8_kernelILi128ELi4E", 3 + 3),
+]
+
+
+@pytest.mark.parametrize("kernel,max_waits", KERNELS)
+def test_tile_loop_has_no_spills_and_no_compiler_waits(isa, kernel, max_waits):
+    loop = _tile_loop(isa, kernel)
+    ops = collections.Counter(l.split()[0] for l in loop)
+    assert ops["v_mfma_f32_32x32x16_bf16"] == (32 if "ILi128E" in kernel else 16)   # head_dim / 4 per 64-token tile
+    assert not [l for l in loop if l.startswith("scratch_")], "a register of the tile loop lives in scratch"
+    waits = [l for l in loop if l.startswith("s_waitcnt") and "vmcnt" in l]
+    assert len(waits) <= max_waits, waits
+    # nothing may wait for memory between the barrier and the end of the step in the bf16 kernels
+    if "fp8" not in kernel:
+        after_barrier = loop[max(i for i, l in enumerate(loop) if l.startswith("s_barrier")):]
+        assert not [l for l in after_barrier if "vmcnt" in l]
+    assert ops["global_load_lds_dwordx4"] in (2, 4, 8)   # a wave's share of the 64 * head_dim * elt * 2 bytes of a tile

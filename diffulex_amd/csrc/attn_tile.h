@@ -38,9 +38,21 @@ struct TileLayout {
     static constexpr int ROWB = HD * 2;                   // bytes per token row
     static constexpr int CPR = ROWB / 16;                 // 16-byte chunks per row
     static constexpr int MAT_BYTES = kTileTokens * ROWB;  // one K (or V) tile
-    // chunk position = chunk index ^ swizzle(row); 16 consecutive rows of one chunk column hit
-    // 16 different 16-byte bank groups (the LDS has 64 banks)
-    DFX_HD static int swizzle(int row) { return HD == 128 ? (row & 15) : ((row >> 1) & 7); }
+    // chunk position = chunk index ^ swizzle(row).  The swizzle is a permutation of row bits chosen
+    // for both operand reads:
+    //   ds_read_b128 (K): 16 lanes = 16 consecutive rows of one chunk column per 256-byte LDS cycle
+    //     -> the low four row bits (three plus the row's 128-byte half for head_dim 64) must give
+    //     16 different positions: any bijection does;
+    //   ds_read_b64_tr_b16 (V^T): 32 lanes = 4 consecutive rows x 4 consecutive chunks x 2 halves
+    //     per cycle -> the rows' two low bits must move the chunk by multiples of 4, or the four
+    //     rows land on the same 16 banks (a plain `row & 15` does that: 4-way conflicts, 8 cycles
+    //     per instruction instead of 2).
+    // Hence: row bits 0,1 -> position bits 2,3 and row bits 2,3 -> position bits 0,1 (head_dim
+    // 128); for 128-byte rows the odd rows already sit 64 banks further, so row bit 1 -> position
+    // bit 2 and row bits 2,3 -> position bits 0,1.
+    DFX_HD static int swizzle(int row) {
+        return HD == 128 ? (((row & 3) << 2) | ((row >> 2) & 3)) : ((((row >> 1) & 1) << 2) | ((row >> 2) & 3));
+    }
     // byte offset of 16-byte chunk c of token row r inside a tile
     DFX_HD static int chunk_offset(int r, int c) { return r * ROWB + ((c ^ swizzle(r)) * 16); }
 };
@@ -90,8 +102,8 @@ struct TileMath : AttnState<HD, NB, NW> {
     // LDS addressing.  A tile starts at a multiple of its row pitch (256 or 128 bytes), so the
     // chunk swizzle, an XOR on bits 4..7 of the offset, can be applied to the finished address:
     //   K operand (tb, slab):       ((tile + k_lane) ^ (slab * 32)) + tb * 32 rows
-    //   V operand (tb, sl, db, ii): ((tile + v_lane) ^ (zi * 64)) + (tb * 32 + sl * 16 + ii * 8) rows,
-    //                               zi = db ^ (swizzle(ii * 8) / 4)
+    //   V operand (tb, sl, db, ii): ((tile + v_lane) ^ (z * 16)) + (tb * 32 + sl * 16 + ii * 8) rows,
+    //                               z = (db * 4) ^ swizzle(ii * 8)
     // with one per-lane constant each.  Per tile that is one addition and a few XORs; the rest
     // folds into the instructions' immediate offsets.  (swizzle(r0 + x) == swizzle(r0) ^ swizzle(x)
     // holds for the row splits used here: 32-row blocks, and ii * 8 + (0..7) inside 16 rows.)
@@ -116,9 +128,9 @@ struct TileMath : AttnState<HD, NB, NW> {
         return *(const lds_bf16x8*)static_cast<uintptr_t>(kx + tb * 32 * L::ROWB);
     }
 
-    // V^T operand for token slab (tb, sl) and d block db; vx[zi]: the V tile's address plus
-    // v_lane, XORed with zi * 64.
-    static constexpr int kVx = HD == 128 ? 4 : 2;
+    // V^T operand for token slab (tb, sl) and d block db; vx[db * 2 + ii]: the V tile's address
+    // plus v_lane, XORed with ((db * 4) ^ swizzle(ii * 8)) * 16.
+    static constexpr int kVx = S::NDB * 2;
     DFX_D bf16x8 read_vt(const uint32_t (&vx)[kVx], int tb, int sl, int db) const {
         typedef short short4v __attribute__((ext_vector_type(4)));
         typedef short short8v __attribute__((ext_vector_type(8)));
@@ -126,8 +138,7 @@ struct TileMath : AttnState<HD, NB, NW> {
         short4v r[2];
 #pragma unroll
         for (int ii = 0; ii < 2; ++ii) {
-            const int zi = db ^ (L::swizzle(ii * 8) / 4);
-            const uint32_t p = vx[zi] + (tb * 32 + sl * 16 + ii * 8) * L::ROWB;
+            const uint32_t p = vx[db * 2 + ii] + (tb * 32 + sl * 16 + ii * 8) * L::ROWB;
             r[ii] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4v*)static_cast<uintptr_t>(p));
         }
         const short8v v = __builtin_shufflevector(r[0], r[1], 0, 1, 2, 3, 4, 5, 6, 7);
@@ -176,7 +187,7 @@ struct TileMath : AttnState<HD, NB, NW> {
         uint32_t vx[kVx];
         vx[0] = lds_address(v_tile) + v_lane;
 #pragma unroll
-        for (int zi = 1; zi < kVx; ++zi) vx[zi] = vx[0] ^ (zi * 64);
+        for (int z = 1; z < kVx; ++z) vx[z] = vx[0] ^ ((((z >> 1) * 4) ^ L::swizzle((z & 1) * 8)) * 16);
         bf16x8 va[3];
         va[0] = read_vt(vx, 0, 0, 0);
         va[1] = read_vt(vx, 0, 0, 1);

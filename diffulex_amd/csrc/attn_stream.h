@@ -389,6 +389,8 @@ __global__ void __launch_bounds__(64 * NW, COMPACT ? 2 : 1) paged_attn_stream_ke
                     bf16x8 pb[NB][2][2];
                     at.template softmax_tile<false, C::ROWS_PER_WAVE>(sc, t, pb, [&] { at.outputs_ready(); });
                     at.accumulate(k_tile + C::MAT_BYTES, pb);
+                } else {
+                    at.outputs_untouched();
                 }
             }
             at.finish_run(rel - 1, split);
@@ -464,6 +466,8 @@ __global__ void __launch_bounds__(64 * NW, 1) paged_attn_stream_fp8_kernel(const
                     bf16x8 pb[1][2][2];
                     at.template softmax_tile<true, C::ROWS_PER_WAVE>(sc, t, pb, [&] { at.outputs_ready(); });
                     at.accumulate(k_tile + TileLayout<HD>::MAT_BYTES, pb);
+                } else {
+                    at.outputs_untouched();
                 }
             }
             at.finish_run(rel - 1, split);

@@ -182,6 +182,17 @@ struct TileMath : AttnState<HD, NB, NW> {
         }
     }
 
+    // For the path of a branch that leaves the accumulators alone: names them as matrix-instruction
+    // operands there too, so that where the paths meet both values already live in the
+    // accumulation registers and none is carried through ordinary registers around the loop.
+    DFX_D void outputs_untouched() {
+#pragma unroll
+        for (int qb = 0; qb < NB; ++qb) {
+            if constexpr (S::NDB == 4) asm volatile("" : "+a"(o[0][qb]), "+a"(o[1][qb]), "+a"(o[2][qb]), "+a"(o[3][qb]));
+            else asm volatile("" : "+a"(o[0][qb]), "+a"(o[1][qb]));
+        }
+    }
+
     DFX_D void accumulate(const uint8_t* v_tile, const bf16x8 (&pb)[NB][2][2]) {
         constexpr int kSteps = 4 * S::NDB;  // (tb, sl, db)
         uint32_t vx[kVx];

@@ -17,12 +17,12 @@ namespace dfx {
 
 DFX_D int uniform(int v) { return __builtin_amdgcn_readfirstlane(v); }
 
-// Two e4m3 codes (bytes 0,1 or 2,3 of w) -> two bf16 packed in a dword.  An e4m3 value has 3
-// mantissa bits, so the upper half of its fp32 form is its bf16 form.
+// Two e4m3 codes (bytes 0,1 or 2,3 of w) -> two bf16 packed in a dword, in one instruction
+// (v_cvt_scalef32_pk_bf16_fp8 with scale 1).  An e4m3 value has 3 mantissa bits, so the widening is
+// exact; checked against v_cvt_pk_f32_fp8 + truncation for all 65 536 pairs of codes.
 template <bool HI>
 DFX_D uint32_t fp8x2_to_bf16x2(uint32_t w) {
-    const f32x2 f = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(w), HI);
-    return (__float_as_uint(f.x) >> 16) | (__float_as_uint(f.y) & 0xffff0000u);
+    return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w, 1.0f, HI));
 }
 
 // 16 e4m3 codes -> 16 bf16 (two 16-byte chunks, in order).

@@ -72,7 +72,16 @@ struct Shape {
     static constexpr int SLOT_FLOATS = BLOCKS * BLOCK_FLOATS;
 };
 
-DFX_D float wave_xor32_max(float x) { return fmaxf(x, __shfl_xor(x, 32)); }
+// max(x of lane i, x of lane i ^ 32): v_permlane32_swap exchanges the halves of a wave inside the
+// vector ALU (a __shfl_xor is an LDS instruction with a round trip of its own per tile).
+DFX_D float wave_xor32_max(float x) {
+    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+DFX_D float wave_xor32_sum(float x) {
+    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
 
 DFX_D float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
@@ -272,7 +281,7 @@ struct AttnState {
 
     DFX_D void row_sums(float (&l_tot)[NB]) const {
 #pragma unroll
-        for (int qb = 0; qb < NB; ++qb) l_tot[qb] = l_run[qb] + __shfl_xor(l_run[qb], 32);
+        for (int qb = 0; qb < NB; ++qb) l_tot[qb] = wave_xor32_sum(l_run[qb]);
     }
 
     // Normalised rows: accumulator 4*i + j of block db is element d = 32*db + 8*i + 4*half + j.

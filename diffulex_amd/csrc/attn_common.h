@@ -284,28 +284,43 @@ struct AttnState {
         for (int qb = 0; qb < NB; ++qb) l_tot[qb] = wave_xor32_sum(l_run[qb]);
     }
 
+    // Whether the 32 rows of block qb of this wave exist in row tile rt of the current item.
+    DFX_D bool block_has_rows(int rt, int qb) const {
+        return rt * S::RT + (wave * NB + qb) * 32 < a.group * sh.q_len;
+    }
+
     // Normalised rows: accumulator 4*i + j of block db is element d = 32*db + 8*i + 4*half + j.
+    // The two lanes of a row (half 0 and 1) hold the two halves of every 16-byte chunk of the
+    // row; they exchange them (v_permlane32_swap) so that each stores whole chunks: the lower
+    // lane the even ones, the upper lane the odd ones.
     DFX_D void store_output(int rt, const float (&l_tot)[NB]) const {
 #pragma unroll
         for (int qb = 0; qb < NB; ++qb) {
             const int r = row_of(rt, qb);
-            if (r >= a.group * sh.q_len) continue;
-            const int g = r / sh.q_len;
-            const int i = r - g * sh.q_len;
+            const bool valid = r < a.group * sh.q_len;
+            const int g = valid ? r / sh.q_len : 0;
+            const int i = valid ? r - g * sh.q_len : 0;
             const float inv = 1.0f / l_tot[qb];
-            uint16_t* op = a.out + (q0 + i) * a.o_st + (kvh * a.group + g) * a.o_sh + half * 4;
+            uint16_t* op = a.out + (q0 + i) * a.o_st + (kvh * a.group + g) * a.o_sh + half * 8;
 #pragma unroll
             for (int db = 0; db < S::NDB; ++db)
 #pragma unroll
-                for (int ii = 0; ii < 4; ++ii) {
-                    const bf16x2 lo = __builtin_convertvector(
-                        f32x2{o[db][qb][ii * 4 + 0] * inv, o[db][qb][ii * 4 + 1] * inv}, bf16x2);
-                    const bf16x2 hi = __builtin_convertvector(
-                        f32x2{o[db][qb][ii * 4 + 2] * inv, o[db][qb][ii * 4 + 3] * inv}, bf16x2);
-                    u32x2 w;
-                    w.x = __builtin_bit_cast(uint32_t, lo);
-                    w.y = __builtin_bit_cast(uint32_t, hi);
-                    *reinterpret_cast<u32x2*>(op + db * 32 + ii * 8) = w;
+                for (int pair = 0; pair < 2; ++pair) {
+                    uint32_t w[2][2];  // [chunk of the pair][dword of this lane's half of it]
+#pragma unroll
+                    for (int c = 0; c < 2; ++c) {
+                        const int ii = pair * 2 + c;
+                        w[c][0] = __builtin_bit_cast(uint32_t, __builtin_convertvector(
+                            f32x2{o[db][qb][ii * 4 + 0] * inv, o[db][qb][ii * 4 + 1] * inv}, bf16x2));
+                        w[c][1] = __builtin_bit_cast(uint32_t, __builtin_convertvector(
+                            f32x2{o[db][qb][ii * 4 + 2] * inv, o[db][qb][ii * 4 + 3] * inv}, bf16x2));
+                    }
+                    // afterwards x[0] is the lower-half dword and x[1] the upper-half dword of
+                    // chunk `half` of the pair
+                    const auto x0 = __builtin_amdgcn_permlane32_swap(w[0][0], w[1][0], false, false);
+                    const auto x1 = __builtin_amdgcn_permlane32_swap(w[0][1], w[1][1], false, false);
+                    const u32x4 chunk = {x0[0], x1[0], x0[1], x1[1]};
+                    if (valid) *reinterpret_cast<u32x4*>(op + db * 32 + pair * 16) = chunk;
                 }
         }
     }
@@ -331,6 +346,7 @@ struct AttnState {
     // 32-row block: accumulators 4*ii .. 4*ii+3 of d block db as 16 bytes at ((db * 4 + ii) * 64
     // + lane) * 16, then the maxima and the row sums (one float per lane each).
     DFX_D void store_partial(int slot, const float (&l_tot)[NB]) const {
+        if (wave >= a.busy_waves) return;  // no rows in any item of the launch: merge_partial skips it too
 #pragma unroll
         for (int qb = 0; qb < NB; ++qb) {
             const __amdgpu_buffer_rsrc_t rs = block_resource(slot, qb);
@@ -358,6 +374,7 @@ struct AttnState {
         // one depends on who merges).  __fmul_rn / __fadd_rn would not do: they are plain operators
         // in this toolchain and fuse like any other.
 #pragma clang fp contract(off)
+        if (wave >= a.busy_waves) return;
 #pragma unroll
         for (int qb = 0; qb < NB; ++qb) {
             const __amdgpu_buffer_rsrc_t rs = block_resource(slot, qb);

@@ -10,7 +10,7 @@ from pathlib import Path
 
 LIB_PATH = Path(__file__).resolve().parent / "libdiffulex_amd.so"
 
-DFX_ABI_VERSION = 2
+DFX_ABI_VERSION = 3
 DFX_OK = 0
 DFX_KV_BF16, DFX_KV_FP8_E4M3 = 0, 1
 DFX_MASK_FULL, DFX_MASK_BLOCK_CAUSAL = 0, 1
@@ -19,7 +19,7 @@ DFX_ATTN_GENERIC_PATH = 1
 
 EXPORTS = (
     "dfx_abi_version", "dfx_status_string", "dfx_kv_store_unified", "dfx_kv_store_distinct",
-    "dfx_kv_load", "dfx_paged_attn_workspace_bytes", "dfx_paged_attn",
+    "dfx_kv_load", "dfx_paged_attn_workspace_bytes", "dfx_paged_attn", "dfx_rope_kv_store",
 )
 
 
@@ -43,6 +43,21 @@ class AttnParams(C.Structure):
         ("diffusion_block_size", C.c_int32), ("kv_dtype", C.c_int32), ("mask_mode", C.c_int32),
         ("max_workgroups", C.c_int32), ("flags", C.c_int32), ("scale", C.c_float),
         ("store_slot_mapping", C.c_void_p), ("store_slot_index_type", C.c_int32),
+    ]
+
+
+class RopeParams(C.Structure):
+    """Mirror of ``dfx_rope_params``."""
+    _fields_ = [
+        ("q", C.c_void_p), ("k", C.c_void_p), ("v", C.c_void_p), ("q_out", C.c_void_p), ("k_out", C.c_void_p),
+        ("q_stride_token", C.c_int64), ("k_stride_token", C.c_int64), ("v_stride_token", C.c_int64),
+        ("q_out_stride_token", C.c_int64), ("k_out_stride_token", C.c_int64),
+        ("positions", C.c_void_p), ("position_index_type", C.c_int32),
+        ("cos_sin_cache", C.c_void_p), ("max_position", C.c_int64), ("n_tokens", C.c_int64),
+        ("num_q_heads", C.c_int32), ("num_kv_heads", C.c_int32), ("head_dim", C.c_int32), ("kv_dtype", C.c_int32),
+        ("k_cache", C.c_void_p), ("v_cache", C.c_void_p),
+        ("slot_mapping", C.c_void_p), ("slot_index_type", C.c_int32), ("n_slots", C.c_int64),
+        ("k_scale", C.c_void_p), ("v_scale", C.c_void_p),
     ]
 
 
@@ -79,6 +94,8 @@ def load() -> C.CDLL:
     lib.dfx_paged_attn_workspace_bytes.argtypes = [C.POINTER(AttnParams)]
     lib.dfx_paged_attn.restype = i32
     lib.dfx_paged_attn.argtypes = [C.POINTER(AttnParams), vp]
+    lib.dfx_rope_kv_store.restype = i32
+    lib.dfx_rope_kv_store.argtypes = [C.POINTER(RopeParams), vp]
     if lib.dfx_abi_version() != DFX_ABI_VERSION:
         raise ImportError(f"{LIB_PATH} has ABI {lib.dfx_abi_version()}, expected {DFX_ABI_VERSION}: rebuild it")
     _lib = lib

@@ -19,7 +19,7 @@
 extern "C" {
 #endif
 
-#define DFX_ABI_VERSION 2
+#define DFX_ABI_VERSION 3
 
 typedef void* dfx_stream_t; /* a hipStream_t; NULL is the default stream */
 
@@ -191,6 +191,59 @@ typedef struct dfx_attn_params {
 int64_t dfx_paged_attn_workspace_bytes(const dfx_attn_params* params);
 
 int dfx_paged_attn(const dfx_attn_params* params, dfx_stream_t stream);
+
+/*
+ * Rotary position embedding of the fresh Q and K rows, optionally fused with the
+ * unified-layout KV-cache store of the rotated K and of V.
+ * Replaces: RotaryEmbedding.forward + apply_rotary_emb
+ *           (diffulex/layer/rotary_embedding.py:39-66, :7-17), called on the
+ *           projections right before the attention layer
+ *           (diffulex/model/dream.py:94-99), and, with slot_mapping != NULL, the
+ *           store_kvcache_unified_layout launch that follows it
+ *           (diffulex/attention/attn_impl.py:54-57).
+ *
+ * For token t with p = positions[t], head h and i < head_dim / 2:
+ *   c = cos_sin_cache[p, i], s = cos_sin_cache[p, head_dim / 2 + i]
+ *   out[t, h, i]                = bf16(x[t, h, i] * c - x[t, h, head_dim / 2 + i] * s)
+ *   out[t, h, head_dim / 2 + i] = bf16(x[t, h, head_dim / 2 + i] * c + x[t, h, i] * s)
+ * in fp32 with every product and sum rounded separately (no fused multiply-add),
+ * then rounded to nearest even: the bits of the reference's eager evaluation.
+ * q_out / k_out may be q / k (in place) or separate buffers.  Positions outside
+ * [0, max_position) are a caller error (clamped, so nothing is read out of bounds).
+ *
+ * slot_mapping != NULL: token t's rotated K row and its V row also go to cache
+ * slot slot_mapping[t] exactly as dfx_kv_store_unified would put them (slots < 0
+ * or >= n_slots skipped; FP8 caches quantise the bf16-rounded rotated K).
+ * slot_mapping == NULL: v, k_cache, v_cache, k_scale, v_scale must be NULL.
+ *
+ * Supported: head_dim a multiple of 16; heads dense inside a token row; strides
+ * (elements) multiples of 8; every pointer 16-byte aligned.
+ */
+typedef struct dfx_rope_params {
+    const void* q;      /* [n_tokens, num_q_heads, head_dim] bf16 */
+    const void* k;      /* [n_tokens, num_kv_heads, head_dim] bf16 */
+    const void* v;      /* [n_tokens, num_kv_heads, head_dim] bf16, read only for the store */
+    void* q_out;        /* rotated q */
+    void* k_out;        /* rotated k */
+    int64_t q_stride_token, k_stride_token, v_stride_token;
+    int64_t q_out_stride_token, k_out_stride_token;
+    const void* positions; /* [n_tokens] */
+    int32_t position_index_type; /* dfx_index_type */
+    const float* cos_sin_cache;  /* [max_position, head_dim] fp32: cosines, then sines */
+    int64_t max_position;
+    int64_t n_tokens;
+    int32_t num_q_heads, num_kv_heads, head_dim;
+    int32_t kv_dtype;            /* dfx_kv_dtype of the caches */
+    void* k_cache;               /* [n_slots, num_kv_heads, head_dim] dense */
+    void* v_cache;
+    const void* slot_mapping;    /* [n_tokens] or NULL */
+    int32_t slot_index_type;     /* dfx_index_type */
+    int64_t n_slots;
+    const float* k_scale;        /* fp32[num_kv_heads], FP8 caches only */
+    const float* v_scale;
+} dfx_rope_params;
+
+int dfx_rope_kv_store(const dfx_rope_params* params, dfx_stream_t stream);
 
 #ifdef __cplusplus
 }

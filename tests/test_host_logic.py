@@ -28,18 +28,49 @@ def test_library_exports_every_declared_symbol():
     assert lib.dfx_status_string(-2) == b"unsupported shape"
 
 
-def test_struct_layout_matches_header(tmp_path):
+@pytest.mark.parametrize("ctype,mirror", [("dfx_attn_params", _lib.AttnParams), ("dfx_rope_params", _lib.RopeParams)])
+def test_struct_layout_matches_header(tmp_path, ctype, mirror):
     """Size and every field offset of the ctypes mirror against what a C compiler makes of the header."""
-    names = [f[0] for f in _lib.AttnParams._fields_]
-    prints = "".join(f'printf("%zu\\n", offsetof(dfx_attn_params, {n}));' for n in names)
+    names = [f[0] for f in mirror._fields_]
+    prints = "".join(f'printf("%zu\\n", offsetof({ctype}, {n}));' for n in names)
     src = tmp_path / "layout.c"
     src.write_text('#include <stdio.h>\n#include <stddef.h>\n#include "diffulex_amd.h"\n'
-                   'int main(void){printf("%zu\\n", sizeof(dfx_attn_params));' + prints + 'return 0;}\n')
+                   f'int main(void){{printf("%zu\\n", sizeof({ctype}));' + prints + 'return 0;}\n')
     exe = tmp_path / "layout"
     subprocess.check_call(["gcc", "-I", os.path.join(ROOT, "include"), "-o", str(exe), str(src)])
     got = [int(x) for x in subprocess.check_output([str(exe)]).split()]
-    assert got[0] == C.sizeof(_lib.AttnParams)
-    assert got[1:] == [getattr(_lib.AttnParams, n).offset for n in names]
+    assert got[0] == C.sizeof(mirror)
+    assert got[1:] == [getattr(mirror, n).offset for n in names]
+
+
+def test_rope_argument_errors_do_not_launch():
+    lib = _lib.load()
+    assert lib.dfx_rope_kv_store(None, None) == -1
+    p = _lib.RopeParams()
+    p.n_tokens, p.num_q_heads, p.num_kv_heads, p.head_dim, p.max_position = 0, 28, 4, 128, 4096
+    assert lib.dfx_rope_kv_store(C.byref(p), None) == 0          # no tokens: nothing to do
+    p.n_tokens = 8
+    assert lib.dfx_rope_kv_store(C.byref(p), None) == -1         # null pointers
+    p.head_dim = 24
+    assert lib.dfx_rope_kv_store(C.byref(p), None) == -2         # head_dim not a multiple of 16
+    p.head_dim = 128
+    p.q = p.k = p.q_out = p.k_out = p.positions = p.cos_sin_cache = 4096
+    p.q_stride_token = p.q_out_stride_token = 28 * 128
+    p.k_stride_token = p.k_out_stride_token = 4 * 128 - 8
+    assert lib.dfx_rope_kv_store(C.byref(p), None) == -1         # key rows overlap
+    p.k_stride_token = p.k_out_stride_token = 4 * 128
+    p.k_cache = 4096
+    assert lib.dfx_rope_kv_store(C.byref(p), None) == -1         # cache without slot_mapping
+    p.k_cache = None
+    p.q = 4100
+    assert lib.dfx_rope_kv_store(C.byref(p), None) == -1         # misaligned
+    p.q = 4096
+    p.position_index_type = 5
+    assert lib.dfx_rope_kv_store(C.byref(p), None) == -1
+    p.position_index_type = 0
+    p.slot_mapping, p.v, p.v_stride_token, p.k_cache, p.v_cache, p.n_slots = 4096, 4096, 512, 4096, 4096, 64
+    p.kv_dtype = 1
+    assert lib.dfx_rope_kv_store(C.byref(p), None) == -1         # FP8 cache without scales
 
 
 def test_argument_errors_do_not_launch():

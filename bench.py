@@ -31,7 +31,7 @@ HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this command, scaled by
 # what the same counters read for a plain copy of known size (one summary per workload under profiles/).
-MEASURED_TRAFFIC_BYTES = {"c3": 288.0e6, "c4": 1491.5e6, "c5": 857.1e6}
+MEASURED_TRAFFIC_BYTES = {"c3": 279.7e6, "c4": 1476.0e6, "c5": 848.6e6}
 
 
 def algorithmic_bytes(wl) -> int:
@@ -149,6 +149,72 @@ def bench_kv_cache(args, dev):
     }))
 
 
+def bench_rope(args, dev):
+    """Rotary embedding of the C3-shaped Q/K projections fused with the KV-cache store (one launch
+    through the C ABI, outputs preallocated).  Eight sets of buffers are used in turn so that the
+    rows come from HBM rather than from the 256 MB last-level cache."""
+    import ctypes as C
+    from diffulex_amd import _lib
+    from diffulex_amd.rotary_embedding import RotaryEmbedding
+    lib = _lib.load()
+    T, hq, hkv, hd, max_pos, n_sets = 2048, 28, 4, 128, 8192, 8
+    g = torch.Generator("cpu").manual_seed(6)
+    rope = RotaryEmbedding(hd, hd, max_pos, 1.0e6).to(dev)
+    pos = torch.randint(0, max_pos, (T,), generator=g).to(dev)
+    pages, page = 64, 256
+    slots = torch.randperm(pages * page, generator=g)[:T].to(torch.int32).to(dev)
+    sets = []
+    for _ in range(n_sets):
+        qkv = torch.randn(T, (hq + 2 * hkv) * hd, generator=g).to(torch.bfloat16).to(dev)
+        sets.append((qkv, torch.empty(T, hq * hd, dtype=torch.bfloat16, device=dev),
+                     torch.empty(T, hkv * hd, dtype=torch.bfloat16, device=dev),
+                     torch.zeros(pages, page, hkv, hd, dtype=torch.bfloat16, device=dev),
+                     torch.zeros(pages, page, hkv, hd, dtype=torch.bfloat16, device=dev)))
+    st = torch.cuda.current_stream().cuda_stream
+    params = []
+    for qkv, qo, ko, kc, vc in sets:
+        p = _lib.RopeParams()
+        p.q, p.k, p.v = qkv.data_ptr(), qkv.data_ptr() + hq * hd * 2, qkv.data_ptr() + (hq + hkv) * hd * 2
+        p.q_out, p.k_out = qo.data_ptr(), ko.data_ptr()
+        p.q_stride_token = p.k_stride_token = p.v_stride_token = qkv.stride(0)
+        p.q_out_stride_token, p.k_out_stride_token = qo.stride(0), ko.stride(0)
+        p.positions, p.position_index_type = pos.data_ptr(), _lib.DFX_INDEX_I64
+        p.cos_sin_cache, p.max_position = rope.cos_sin_cache.data_ptr(), max_pos
+        p.n_tokens, p.num_q_heads, p.num_kv_heads, p.head_dim = T, hq, hkv, hd
+        p.kv_dtype, p.k_cache, p.v_cache = _lib.DFX_KV_BF16, kc.data_ptr(), vc.data_ptr()
+        p.slot_mapping, p.slot_index_type, p.n_slots = slots.data_ptr(), _lib.DFX_INDEX_I32, pages * page
+        params.append(p)
+
+    def step(i):
+        _lib.check(lib.dfx_rope_kv_store(C.byref(params[i % n_sets]), st), "dfx_rope_kv_store")
+
+    n_spin = spin_up(step)
+    for i in range(args.warmup):
+        step(i)
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for i in range(args.steps):
+        step(i)
+    stop.record()
+    torch.cuda.synchronize()
+    ms = start.elapsed_time(stop) / args.steps
+    # q and k read and written, v read, k and v written to the cache, one table row per token
+    nbytes = T * hd * 2 * (2 * hq + 2 * hkv + hkv + 2 * hkv) + T * hd * 4
+    gbs = nbytes / (ms * 1e-3) / 1e9
+    print(json.dumps({
+        "metric": "rotary embedding + KV-cache store, tokens per second and achieved HBM GB/s, 1 GPU",
+        "value": T / (ms * 1e-3), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": f"rope: {T} tokens, H_q={hq}, H_kv={hkv}, head_dim={hd}, rotated and stored into a "
+                               f"{pages}x{page}-slot bf16 cache in one launch", "spin_up_launches": n_spin},
+        "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS,
+                     "traffic": None, "algorithmic_bytes": nbytes,
+                     "kernel": "rope_kv_store_kernel, duration = timed region / steps"},
+    }))
+
+
 SPIN_UP_SECONDS = 0.25
 
 
@@ -172,7 +238,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="c3", choices=["c3", "c4", "c5", "c1", "c2"])
+    ap.add_argument("--workload", default="c3", choices=["c3", "c4", "c5", "c1", "c2", "rope"])
     ap.add_argument("--copies", type=int, default=4, help="independent KV-cache copies rotated between steps")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -201,6 +267,9 @@ def main():
         return
     if args.workload == "c2":
         bench_kv_cache(args, dev)
+        return
+    if args.workload == "rope":
+        bench_rope(args, dev)
         return
     wl = make_workload(args.workload, device=dev)
     caches = [(wl.k_cache, wl.v_cache)]

@@ -114,7 +114,7 @@ DFX_D SeqShape load_seq_shape(const KArgs& a, int s, int rows_per_tile) {
     const int ctx = (a.context_lens != nullptr && a.k_cache != nullptr) ? a.context_lens[s] : 0;
     const int q_len = a.cu_q[s + 1] - a.cu_q[s];
     const int new_len = a.cu_new[s + 1] - a.cu_new[s];
-    return make_seq_shape(ctx, q_len, new_len, a.group, rows_per_tile);
+    return make_seq_shape(ctx, q_len, new_len, a.group, rows_per_tile, a.mask_mode == DFX_MASK_BLOCK_CAUSAL, a.dbs);
 }
 
 // What the softmax needs to know about one KV tile.

@@ -186,8 +186,9 @@ struct GenericAttn : TileMath<HD, NB, kWaves> {
         this->accumulate(v_stage(buf), pb);
     }
 
-    DFX_D void run_segment(int rt, int tile0, int tile1, int64_t item_begin, const WgSplit& split, int slot) {
-        const bool complete = tile0 == 0 && tile1 == this->sh.n_tiles;
+    DFX_D void run_segment(int rt, int tile0, int tile1, int item_tiles, int64_t item_begin, const WgSplit& split,
+                           int slot) {
+        const bool complete = tile0 == 0 && tile1 == item_tiles;
         this->load_queries(rt);
         __syncthreads();  // the previous segment's last tile and block-table entries may still be read from LDS
         cache_block_table(tile0, tile1);
@@ -205,7 +206,7 @@ struct GenericAttn : TileMath<HD, NB, kWaves> {
         float l_tot[NB];
         this->row_sums(l_tot);
         if (complete) this->store_output(rt, l_tot);
-        else finish_cut_item(*this, rt, item_begin, this->sh.n_tiles, split, slot, l_tot, misc + kMaxWaves + 1);
+        else finish_cut_item(*this, rt, item_begin, item_tiles, split, slot, l_tot, misc + kMaxWaves + 1);
     }
 };
 
@@ -235,12 +236,11 @@ __global__ void __launch_bounds__(kThreads) paged_attn_generic_kernel(const KArg
     int64_t pos = begin;
     while (pos < end) {
         at.set_sequence(s, kvh);
-        const int n_tiles = at.sh.n_tiles;
-        const int rt = u / n_tiles;
-        const int tile0 = u - rt * n_tiles;
+        int rt, tile0, n_tiles;
+        locate_unit(at.sh, u, rt, tile0, n_tiles);
         const int64_t seg_end = min(pos + (n_tiles - tile0), end);
         const int tile1 = tile0 + static_cast<int>(seg_end - pos);
-        at.run_segment(rt, tile0, tile1, pos - tile0, split, partial_slot(w, pos, begin));
+        at.run_segment(rt, tile0, tile1, n_tiles, pos - tile0, split, partial_slot(w, pos, begin));
         u += tile1 - tile0;
         pos = seg_end;
         if (pos >= end) break;

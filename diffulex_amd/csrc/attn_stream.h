@@ -148,15 +148,15 @@ struct StreamAttn : TileMath<HD, NB, NW> {
             const int sq = lo;
             const SeqShape shp = load_seq_shape(a, sq, C::RT);
             const int u = rem - prefix[sq];
-            const int rt = u / shp.n_tiles;
-            const int tile = u - rt * shp.n_tiles;
+            int rt, tile, item_tiles;
+            locate_unit(shp, u, rt, tile, item_tiles);
             const bool is_ctx = tile < shp.n_ctx_tiles;
             const int base = (is_ctx ? tile : tile - shp.n_ctx_tiles) * C::TN;
             const int limit = is_ctx ? shp.ctx : shp.new_len;
             // the piece of the item this workgroup owns
             const int64_t before = pos - begin, after = end - pos;
             const int tile0 = before >= tile ? 0 : tile - static_cast<int>(before);
-            const int tile1 = after >= shp.n_tiles - tile ? shp.n_tiles : tile + static_cast<int>(after);
+            const int tile1 = after >= item_tiles - tile ? item_tiles : tile + static_cast<int>(after);
             if (w == 0) {
                 UnitDesc d;
                 d.s = sq;
@@ -168,11 +168,11 @@ struct StreamAttn : TileMath<HD, NB, NW> {
                 d.limit = limit;
                 d.flags = (is_ctx ? kUnitCtx : 0) | (tile == tile0 ? kUnitFirst : 0) |
                           (tile == tile1 - 1 ? kUnitLast : 0) |
-                          (tile0 == 0 && tile1 == shp.n_tiles ? kUnitComplete : 0);
+                          (tile0 == 0 && tile1 == item_tiles ? kUnitComplete : 0);
                 d.slot = partial_slot(static_cast<int>(blockIdx.x), pos - (tile - tile0), begin);
                 d.run = tile1 - tile;
                 d.item_rel = static_cast<int>(pos - tile - begin);
-                d.n_tiles = shp.n_tiles;
+                d.n_tiles = item_tiles;
                 units[slot_in_ring] = d;
             }
             // Rows past the end re-read the last valid rows (finite data; their scores are masked).

@@ -4,7 +4,8 @@
 // Work is measured in "units": one unit is one KV tile (kTileTokens tokens of one KV head of
 // one sequence) processed for one row tile of that sequence's queries.  Sequence s owns
 //     units(s) = n_tiles(s) * n_row_tiles(s)
-// consecutive units (row-tile major), the sequences follow each other, and the whole list is
+// consecutive units (row-tile major) -- fewer under the block-causal mask, where a row tile owns
+// no fresh tile that none of its queries can see -- the sequences follow each other, and the whole list is
 // repeated for every KV head.  The linear unit space [0, total) is cut into n_wg equal
 // ranges, one per participating workgroup; wherever a cut falls inside a (sequence, head, row
 // tile) item the sides produce partial results, which the workgroup that finishes its piece
@@ -31,18 +32,75 @@ struct SeqShape {
     int n_tiles;    // KV tiles: context tiles then fresh tiles (never mixed in one tile)
     int n_row_tiles;
     int units;
+    // Block-causal mask with row tiles that do not straddle query heads (rph > 0): row tile k of a
+    // head holds queries k * RT .. (k + 1) * RT - 1, which see no fresh token from (k + 1) * RT on,
+    // so that row tile owns only its context tiles and its first min(n_new_tiles, (k + 1) * step)
+    // fresh tiles.  rph == 0: every row tile owns all n_tiles.
+    int rph;        // row tiles per query head, or 0
+    int step;       // fresh tiles that become visible per row tile (RT / kTileTokens)
+    int n_new_tiles;
+    int ramp;       // row tiles of a head that see fewer than n_new_tiles fresh tiles
 };
 
-DFX_HD SeqShape make_seq_shape(int ctx, int q_len, int new_len, int group, int rows_per_tile) {
+// Units of the first k row tiles of one query head (rph > 0).
+DFX_HD int units_before_row_tile(const SeqShape& s, int k) {
+    const int kr = k < s.ramp ? k : s.ramp;  // the ramp: step, 2 * step, ... fresh tiles
+    return k * s.n_ctx_tiles + s.step * (kr * (kr + 1) / 2) + (k - kr) * s.n_new_tiles;
+}
+
+// KV tiles row tile rt of the sequence owns.
+DFX_HD int tiles_of_row_tile(const SeqShape& s, int rt) {
+    if (s.rph == 0) return s.n_tiles;
+    const int k = rt % s.rph;
+    return s.n_ctx_tiles + (k < s.ramp ? (k + 1) * s.step : s.n_new_tiles);
+}
+
+DFX_HD SeqShape make_seq_shape(int ctx, int q_len, int new_len, int group, int rows_per_tile,
+                               bool block_causal = false, int dbs = 0) {
     SeqShape s;
     s.ctx = ctx > 0 ? ctx : 0;
     s.q_len = q_len > 0 ? q_len : 0;
     s.new_len = new_len > 0 ? new_len : 0;
     s.n_ctx_tiles = ceil_div(s.ctx, kTileTokens);
-    s.n_tiles = s.n_ctx_tiles + ceil_div(s.new_len, kTileTokens);
+    s.n_new_tiles = ceil_div(s.new_len, kTileTokens);
+    s.n_tiles = s.n_ctx_tiles + s.n_new_tiles;
     s.n_row_tiles = ceil_div(group * s.q_len, rows_per_tile);
     s.units = s.n_tiles * s.n_row_tiles;
+    s.rph = 0;
+    s.step = rows_per_tile / kTileTokens;
+    s.ramp = 0;
+    if (block_causal && dbs > 0 && s.q_len > 0 && s.q_len % rows_per_tile == 0 && rows_per_tile % dbs == 0 &&
+        rows_per_tile % kTileTokens == 0) {
+        s.rph = s.q_len / rows_per_tile;
+        // row tile k sees (k + 1) * step fresh tiles while that is fewer than all of them
+        const int full_from = ceil_div(s.n_new_tiles, s.step) - 1;  // first k that sees every fresh tile
+        s.ramp = full_from < 0 ? 0 : (full_from < s.rph ? full_from : s.rph);
+        s.units = group * units_before_row_tile(s, s.rph);
+    }
     return s;
+}
+
+// Unit u of a sequence (0 <= u < units) -> its row tile, its tile inside that row tile's item and
+// the number of tiles of that item.
+DFX_HD void locate_unit(const SeqShape& s, int u, int& rt, int& tile, int& item_tiles) {
+    if (s.rph == 0) {
+        rt = u / s.n_tiles;
+        tile = u - rt * s.n_tiles;
+        item_tiles = s.n_tiles;
+        return;
+    }
+    const int per_head = units_before_row_tile(s, s.rph);
+    const int g = u / per_head;
+    const int v = u - g * per_head;
+    int lo = 0, hi = s.rph - 1;  // the largest k with units_before_row_tile(k) <= v
+    while (lo < hi) {
+        const int mid = (lo + hi + 1) >> 1;
+        if (units_before_row_tile(s, mid) <= v) lo = mid;
+        else hi = mid - 1;
+    }
+    rt = g * s.rph + lo;
+    tile = v - units_before_row_tile(s, lo);
+    item_tiles = tiles_of_row_tile(s, rt);
 }
 
 // How many of the n_wg workgroups of the launch take part.  Cutting an item into p pieces costs

@@ -27,13 +27,33 @@ int hook_effective_workgroups(int64_t total_units, int64_t n_items, int max_tile
 // Replays the persistent kernel's walk over its unit range on the host.  For workgroup w it
 // appends one record per segment: {w, kv_head, seq, row_tile, tile0, tile1, complete, slot}.
 // ctx/q_len/new_len: per-sequence lengths.  Returns the number of records (<= cap).
+int64_t hook_walk_segments_masked(const int* ctx, const int* q_len, const int* new_len, int num_seqs, int h_kv,
+                                  int group, int rows_per_tile, int n_wg, int block_causal, int dbs, int64_t* rec,
+                                  int64_t cap);
+
 int64_t hook_walk_segments(const int* ctx, const int* q_len, const int* new_len, int num_seqs, int h_kv, int group,
                            int rows_per_tile, int n_wg, int64_t* rec, int64_t cap) {
+    return hook_walk_segments_masked(ctx, q_len, new_len, num_seqs, h_kv, group, rows_per_tile, n_wg, 0, 0, rec, cap);
+}
+
+// Every unit of one sequence in order: out[3 * u + {0, 1, 2}] = row tile, tile inside the item,
+// tiles of the item.  Returns the number of units (<= cap entries are written).
+int hook_enumerate_units(int ctx, int q_len, int new_len, int group, int rows_per_tile, int block_causal, int dbs,
+                         int* out, int cap) {
+    using namespace dfx;
+    const SeqShape sh = make_seq_shape(ctx, q_len, new_len, group, rows_per_tile, block_causal != 0, dbs);
+    for (int u = 0; u < sh.units && u < cap; ++u) locate_unit(sh, u, out[3 * u], out[3 * u + 1], out[3 * u + 2]);
+    return sh.units;
+}
+
+int64_t hook_walk_segments_masked(const int* ctx, const int* q_len, const int* new_len, int num_seqs, int h_kv,
+                                  int group, int rows_per_tile, int n_wg, int block_causal, int dbs, int64_t* rec,
+                                  int64_t cap) {
     using namespace dfx;
     std::vector<SeqShape> sh(num_seqs);
     std::vector<int> prefix(num_seqs + 1, 0);
     for (int s = 0; s < num_seqs; ++s) {
-        sh[s] = make_seq_shape(ctx[s], q_len[s], new_len[s], group, rows_per_tile);
+        sh[s] = make_seq_shape(ctx[s], q_len[s], new_len[s], group, rows_per_tile, block_causal != 0, dbs);
         prefix[s + 1] = prefix[s] + sh[s].units;
     }
     const int per_head = prefix[num_seqs];
@@ -52,8 +72,8 @@ int64_t hook_walk_segments(const int* ctx, const int* q_len, const int* new_len,
         int u = rem - prefix[s];
         int64_t pos = begin;
         while (pos < end) {
-            const int n_tiles = sh[s].n_tiles;
-            const int rt = u / n_tiles, tile0 = u - rt * n_tiles;
+            int rt, tile0, n_tiles;
+            locate_unit(sh[s], u, rt, tile0, n_tiles);
             const int64_t seg_end = pos + (n_tiles - tile0) < end ? pos + (n_tiles - tile0) : end;
             const int tile1 = tile0 + static_cast<int>(seg_end - pos);
             const bool complete = tile0 == 0 && tile1 == n_tiles;

@@ -27,6 +27,10 @@ def load():
     lib.hook_effective_workgroups.argtypes = [i64, i64, i32, i32]
     lib.hook_walk_segments.restype = i64
     lib.hook_walk_segments.argtypes = [vp, vp, vp, i32, i32, i32, i32, i32, vp, i64]
+    lib.hook_walk_segments_masked.restype = i64
+    lib.hook_walk_segments_masked.argtypes = [vp, vp, vp, i32, i32, i32, i32, i32, i32, i32, vp, i64]
+    lib.hook_enumerate_units.restype = i32
+    lib.hook_enumerate_units.argtypes = [i32, i32, i32, i32, i32, i32, i32, vp, i32]
     lib.hook_combine_slots.restype = i32
     lib.hook_combine_slots.argtypes = [vp, vp, vp, i32, i32, i32, i32, i32, i32, i32, i32, vp, i32]
     return lib

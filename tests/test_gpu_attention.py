@@ -411,3 +411,40 @@ def test_batch_above_the_limit_is_refused(dev):
     wl = make_workload("c1", num_seqs=4096, ctx=(0, 20), seed=3).to(dev)
     with pytest.raises(Exception):
         _run(wl)
+
+
+@pytest.mark.parametrize("over", [
+    dict(num_seqs=3, h_q=7, h_kv=1, q_len=512, ctx=[0, 0, 0]),              # prefill shape: 2 row tiles per head
+    dict(num_seqs=2, h_q=2, h_kv=2, q_len=512, ctx=[200, 0]),               # one head per KV head, cached prefix
+    dict(num_seqs=2, h_q=14, h_kv=2, q_len=1024, ctx=[0, 333], hd=64),      # 4 row tiles per head, head_dim 64
+    dict(num_seqs=2, h_q=4, h_kv=4, q_len=256, ctx=[300, 70]),              # one row tile per head: nothing to skip
+    dict(num_seqs=2, h_q=6, h_kv=2, q_len=200, ctx=[0, 90]),                # row tiles straddle heads: every tile kept
+])
+@pytest.mark.parametrize("flags", PATHS)
+@pytest.mark.parametrize("max_wg", [0, 5])
+def test_block_causal_row_tiles_skip_the_fresh_tiles_they_cannot_see(dev, over, flags, max_wg):
+    """Row tiles of long block-causal sequences own only the fresh tiles some of their rows can
+    see; the result is the oracle's, whatever the partition."""
+    wl = make_workload("c4", seed=31, page=64, **over)
+    want = oracle_fp32(wl)
+    got = _run(wl.to(dev), max_workgroups=max_wg, flags=flags)
+    assert torch.isfinite(got.float()).all()
+    assert max_abs_err(got, want) <= ATOL_BF16
+
+
+def test_block_causal_prefill_without_a_cache(dev):
+    B, L, hq, hkv, hd = 2, 768, 8, 2, 128
+    g = torch.Generator().manual_seed(17)
+    q = torch.randn(B * L, hq, hd, generator=g).to(torch.bfloat16)
+    k = torch.randn(B * L, hkv, hd, generator=g).to(torch.bfloat16)
+    v = torch.randn(B * L, hkv, hd, generator=g).to(torch.bfloat16)
+    cu = torch.arange(0, B * L + 1, L, dtype=torch.int32)
+    from oracle import attention as oat
+    want = oat.paged_attention_fp32(q, k, v, None, None, None, None, cu, cu, hd ** -0.5,
+                                    mask_mode=MASK_BLOCK_CAUSAL, dbs=32)
+    for flags in PATHS:
+        got = dfx.paged_attention(q.to(dev), k.to(dev), v.to(dev), None, None, hd ** -0.5, block_tables=None,
+                                  context_lens=None, cu_seqlens_q=cu.to(dev), cu_seqlens_new=cu.to(dev),
+                                  max_seqlen_q=L, mask_mode=MASK_BLOCK_CAUSAL, diffusion_block_size=32, flags=flags)
+        torch.cuda.synchronize()
+        assert max_abs_err(got, want) <= ATOL_BF16

@@ -201,3 +201,84 @@ def test_number_of_participating_workgroups():
     assert f(64 * 4 * 21, 256, 33, 256) == 256        # Dream-7B shape, batch 64: every compute unit
     assert f(4 * 33, 4, 33, 256) == 12                # batch 1, 2K context: 132 units at >= 11 per workgroup
     assert f(4 * 513, 4, 513, 256) == 46              # batch 1, 32K context: >= 45 per workgroup
+
+
+def _visible_tiles(ctx, q_len, new_len, group, rows_per_tile, rt, block_causal, dbs):
+    """Brute force: context tiles plus every fresh tile that some query row of row tile rt can see."""
+    n_ctx = -(-ctx // 64)
+    n_new = -(-new_len // 64)
+    if not block_causal:
+        return n_ctx + n_new
+    rows = range(rt * rows_per_tile, min((rt + 1) * rows_per_tile, group * q_len))
+    limit = max(min(new_len, ((r % q_len) // dbs + 1) * dbs) for r in rows)
+    return n_ctx + sum(1 for t in range(n_new) if t * 64 < limit)
+
+
+@pytest.mark.parametrize("ctx,q_len,new_len,group,rpt,dbs", [
+    (0, 512, 512, 1, 128, 32), (300, 1024, 1024, 7, 256, 32), (0, 2048, 2048, 2, 256, 64), (70, 256, 256, 4, 256, 32),
+    (0, 512, 700, 3, 128, 32), (0, 768, 300, 2, 256, 32), (100, 512, 0, 2, 128, 32), (0, 128, 128, 5, 128, 128),
+])
+def test_block_causal_row_tiles_own_exactly_the_tiles_they_can_see(ctx, q_len, new_len, group, rpt, dbs):
+    hooks = hosthooks.load()
+    cap = 200000
+    out = np.zeros((cap, 3), dtype=np.int32)
+    n = hooks.hook_enumerate_units(ctx, q_len, new_len, group, rpt, 1, dbs, out.ctypes.data, cap)
+    want = []
+    for rt in range(-(-group * q_len // rpt)):
+        nt = _visible_tiles(ctx, q_len, new_len, group, rpt, rt, True, dbs)
+        want += [(rt, t, nt) for t in range(nt)]
+    assert n == len(want)
+    assert out[:n].tolist() == [list(w) for w in want]
+    full = hooks.hook_enumerate_units(ctx, q_len, new_len, group, rpt, 0, dbs, out.ctypes.data, 0)
+    assert n <= full
+    if new_len >= 2 * rpt and q_len >= 2 * rpt:
+        assert n < full        # something is skipped
+
+
+@pytest.mark.parametrize("ctx,q_len,new_len,group,rpt,dbs", [
+    (0, 200, 200, 2, 128, 32),      # row tiles straddle heads
+    (0, 512, 512, 2, 128, 48),      # block size does not divide the row tile
+    (10, 96, 96, 1, 128, 32),       # one partial row tile (the D2F decode shape)
+])
+def test_block_causal_shapes_outside_the_schedule_keep_every_tile(ctx, q_len, new_len, group, rpt, dbs):
+    hooks = hosthooks.load()
+    out = np.zeros((100000, 3), dtype=np.int32)
+    n = hooks.hook_enumerate_units(ctx, q_len, new_len, group, rpt, 1, dbs, out.ctypes.data, 100000)
+    n_tiles = -(-ctx // 64) + -(-new_len // 64)
+    assert n == n_tiles * -(-group * q_len // rpt)
+    for rt in range(-(-group * q_len // rpt)):   # and that is never fewer than what the rows can see
+        assert _visible_tiles(ctx, q_len, new_len, group, rpt, rt, True, dbs) <= n_tiles
+    assert out[:n, 2].min() == n_tiles
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_masked_partition_covers_every_visible_tile_once(seed):
+    hooks = hosthooks.load()
+    rng = np.random.default_rng(100 + seed)
+    b = int(rng.integers(1, 12))
+    h_kv, group = int(rng.integers(1, 4)), int(rng.choice([1, 2, 7]))
+    rpt = int(rng.choice([128, 256]))
+    n_wg = int(rng.choice([1, 3, 64, 256]))
+    q_len = rng.choice([0, 96, 256, 512, 1024], b)
+    new_len = q_len.copy()
+    ctx = rng.integers(0, 400, b)
+    ctx32, q32, new32 = (np.ascontiguousarray(a, dtype=np.int32) for a in (ctx, q_len, new_len))
+    cap = 400000
+    rec = np.zeros((cap, 8), dtype=np.int64)
+    n = hooks.hook_walk_segments_masked(ctx32.ctypes.data, q32.ctypes.data, new32.ctypes.data, b, h_kv, group, rpt,
+                                        n_wg, 1, 32, rec.ctypes.data, cap)
+    assert 0 <= n <= cap
+    seen = {}
+    for w, kvh, s, rt, t0, t1, complete, slot in rec[:n].tolist():
+        nt = _visible_tiles(int(ctx[s]), int(q_len[s]), int(new_len[s]), group, rpt, rt, True, 32)
+        assert 0 <= t0 < t1 <= nt and bool(complete) == (t0 == 0 and t1 == nt)
+        seen.setdefault((kvh, s, rt), []).append((t0, t1))
+    for kvh in range(h_kv):
+        for s in range(b):
+            for rt in range(-(-group * int(q_len[s]) // rpt)):
+                nt = _visible_tiles(int(ctx[s]), int(q_len[s]), int(new_len[s]), group, rpt, rt, True, 32)
+                if nt == 0:
+                    continue
+                pieces = sorted(seen[(kvh, s, rt)])
+                assert pieces[0][0] == 0 and pieces[-1][1] == nt
+                assert all(a[1] == bb[0] for a, bb in zip(pieces, pieces[1:]))

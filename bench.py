@@ -215,6 +215,53 @@ def bench_rope(args, dev):
     }))
 
 
+def bench_prefill(args, dev):
+    """Block-attention prefill (the reference's dllm_flash_attn_prefill with attn_type
+    "block_attention"): B=8 prompts of 2048 tokens, Dream-7B heads, block-causal mask with 32-token
+    blocks, no cache.  Compute bound: the roofline is the bf16 matrix rate, counted on the score
+    elements the mask lets through."""
+    import diffulex_amd as dfx
+    from diffulex_amd import _lib
+    B, L, hq, hkv, hd, dbs = 8, 2048, 28, 4, 128, 32
+    g = torch.Generator("cpu").manual_seed(7)
+    q = torch.randn(B * L, hq, hd, generator=g).to(torch.bfloat16).to(dev)
+    k = torch.randn(B * L, hkv, hd, generator=g).to(torch.bfloat16).to(dev)
+    v = torch.randn(B * L, hkv, hd, generator=g).to(torch.bfloat16).to(dev)
+    cu = torch.arange(0, B * L + 1, L, dtype=torch.int32, device=dev)
+    out = torch.empty_like(q)
+
+    def step(_):
+        dfx.paged_attention(q, k, v, None, None, hd ** -0.5, block_tables=None, context_lens=None, cu_seqlens_q=cu,
+                            cu_seqlens_new=cu, max_seqlen_q=L, mask_mode=_lib.DFX_MASK_BLOCK_CAUSAL,
+                            diffusion_block_size=dbs, out=out)
+
+    n_spin = spin_up(step)
+    for i in range(args.warmup):
+        step(i)
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for i in range(args.steps):
+        step(i)
+    stop.record()
+    torch.cuda.synchronize()
+    ms = start.elapsed_time(stop) / args.steps
+    visible = sum(min(L, (i // dbs + 1) * dbs) for i in range(L))
+    nflops = 4 * hq * hd * visible * B
+    tflops = nflops / (ms * 1e-3) / 1e12
+    print(json.dumps({
+        "metric": "block-attention prefill, query-tokens/sec and achieved bf16 TFLOP/s, 1 GPU",
+        "value": B * L / (ms * 1e-3), "unit": "query-tokens/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"prefill: B={B} prompts of {L} tokens, H_q={hq}, H_kv={hkv}, head_dim={hd}, "
+                               f"block-causal mask, {dbs}-token blocks, no cache", "spin_up_launches": n_spin},
+        "roofline": {"bound": "mfma", "achieved": tflops, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": tflops / MFMA_BF16_PEAK_TFLOPS, "traffic": None, "algorithmic_flops": nflops,
+                     "kernel": "paged_attn_stream_kernel<128, 1, 8, false>, duration = timed region / steps"},
+    }))
+
+
 SPIN_UP_SECONDS = 0.25
 
 
@@ -238,7 +285,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="c3", choices=["c3", "c4", "c5", "c1", "c2", "rope"])
+    ap.add_argument("--workload", default="c3", choices=["c3", "c4", "c5", "c1", "c2", "rope", "prefill"])
     ap.add_argument("--copies", type=int, default=4, help="independent KV-cache copies rotated between steps")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -270,6 +317,9 @@ def main():
         return
     if args.workload == "rope":
         bench_rope(args, dev)
+        return
+    if args.workload == "prefill":
+        bench_prefill(args, dev)
         return
     wl = make_workload(args.workload, device=dev)
     caches = [(wl.k_cache, wl.v_cache)]

@@ -448,3 +448,34 @@ def test_block_causal_prefill_without_a_cache(dev):
                                   max_seqlen_q=L, mask_mode=MASK_BLOCK_CAUSAL, diffusion_block_size=32, flags=flags)
         torch.cuda.synchronize()
         assert max_abs_err(got, want) <= ATOL_BF16
+
+
+# the shapes of the reference's prefill kernel tests (tests/python/kernel/test_dllm_flash_attn_prefill_kernel.py
+# :162-310): (sequences, query heads, KV heads, head_dim, length, block attention, diffusion block size)
+REF_PREFILL_CASES = [
+    (1, 32, 8, 128, 192, False, 32), (4, 32, 8, 128, 256, False, 32), (2, 32, 8, 128, 256, True, 32),
+    (3, 32, 8, 128, 320, True, 32), (2, 32, 8, 128, 256, True, 64), (2, 32, 4, 128, 192, False, 32),
+    (2, 32, 4, 128, 256, True, 32), (2, 32, 8, 64, 192, False, 32),
+]
+
+
+@pytest.mark.parametrize("case", REF_PREFILL_CASES)
+def test_reference_prefill_test_shapes(dev, case):
+    """Through the operator, against the fp32 oracle; the reference compares with atol = rtol = 1e-2."""
+    from oracle import attention as oat
+    B, hq, hkv, hd, L, block_attn, dbs = case
+    g = torch.Generator().manual_seed(B * 1000 + L + dbs)
+    q = torch.randn(B * L, hq, hd, generator=g).to(torch.bfloat16)
+    k = torch.randn(B * L, hkv, hd, generator=g).to(torch.bfloat16)
+    v = torch.randn(B * L, hkv, hd, generator=g).to(torch.bfloat16)
+    cu = torch.arange(0, (B + 1) * L, L, dtype=torch.int32)
+    scale = 1.0 / (hd ** 0.5)
+    mask = MASK_BLOCK_CAUSAL if block_attn else MASK_FULL
+    want = oat.paged_attention_fp32(q, k, v, None, None, None, None, cu, cu, scale, mask_mode=mask, dbs=dbs)
+    md = dfx.PagedAttnMetaData(is_prefill=True, cu_seqlens_q=cu.to(dev), cu_seqlens_k=cu.to(dev), max_seqlen_q=L,
+                               max_seqlen_k=L, attn_type="block_attention" if block_attn else "full_attention",
+                               diffusion_block_size=dbs)
+    got = dfx.dllm_flash_attn_prefill(q.to(dev), k.to(dev), v.to(dev), scale, md)
+    torch.cuda.synchronize()
+    assert got.shape == q.shape and got.dtype == torch.bfloat16
+    assert max_abs_err(got, want) <= 1e-2

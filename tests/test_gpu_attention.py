@@ -479,3 +479,12 @@ def test_reference_prefill_test_shapes(dev, case):
     torch.cuda.synchronize()
     assert got.shape == q.shape and got.dtype == torch.bfloat16
     assert max_abs_err(got, want) <= 1e-2
+
+
+@pytest.mark.parametrize("flags", PATHS)
+def test_block_causal_long_queries_on_an_fp8_cache(dev, flags):
+    wl = make_workload("c5", seed=33, num_seqs=2, h_q=8, h_kv=2, q_len=512, ctx=[700, 130], mask=MASK_BLOCK_CAUSAL)
+    want = oracle_fp32(wl)
+    for max_wg in (0, 7):
+        got = _run(wl.to(dev), max_workgroups=max_wg, flags=flags)
+        assert max_abs_err(got, want) <= ATOL_FP8

@@ -65,8 +65,8 @@ struct Shape {
     static constexpr int PREFIX_BYTES = (kMaxSeqs + 1) * 4;
     static constexpr int MISC_BYTES = 128;
     // A partial result is stored per 32-row query block b = wave * NB + qb, whatever the shape of
-    // the workgroup that wrote it: NDB * 4 float4 per lane of O^T, then the running maximum and
-    // the row sum of the lane's query.
+    // the workgroup that wrote it, in an area of BLOCK_FLOATS floats (the format, which uses a
+    // little over half of it, is described at AttnState::store_partial).
     static constexpr int BLOCKS = NB * NW;
     static constexpr int BLOCK_FLOATS = 64 * (NDB * 16 + 2);
     static constexpr int SLOT_FLOATS = BLOCKS * BLOCK_FLOATS;
@@ -342,32 +342,90 @@ struct AttnState {
         return __builtin_amdgcn_make_buffer_rsrc(bp, 0, S::BLOCK_FLOATS * 4, 0x00020000);
     }
 
-    // Unnormalised accumulators, running maxima and row sums of a piece of an item.  Layout of a
-    // 32-row block: accumulators 4*ii .. 4*ii+3 of d block db as 16 bytes at ((db * 4 + ii) * 64
-    // + lane) * 16, then the maxima and the row sums (one float per lane each).
+    // A stored piece of an item: per 32-row block the unnormalised accumulators as fp16 relative to
+    // a power of two per query row (the exponent of the row's largest magnitude, so scaling is
+    // exact and every value lands in (-2, 2)), then per lane 16 bytes {running maximum, row sum,
+    // that power of two, 0} in fp32.  Chunk c (accumulators 8 * (c & 1) .. + 7 of d block c >> 1)
+    // is 16 bytes at (c * 64 + lane) * 16, the statistics at kStatsOff + lane * 16.  Half the
+    // bytes of an fp32 copy: moving a piece is limited by the memory path of one compute unit.
+    // The rounding (2^-12 of the row's largest accumulator) is an eighth of what the bf16 output
+    // rounding adds afterwards.
+    typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+    static constexpr int kChunks = S::NDB * 2;
+    static constexpr int kStatsOff = kChunks * 64 * 16;
+    static_assert(kStatsOff + 64 * 16 <= S::BLOCK_FLOATS * 4, "a block fits its slot");
+
+    // 2^-(exponent of mx) and its inverse (1 for zero); mx >= 0.
+    DFX_D static void row_scale(float mx, float& down, float& up) {
+        const uint32_t e = (__float_as_uint(mx) >> 23) & 0xffu;
+        uint32_t d = e == 0 ? 127u : 254u - e;
+        d = d < 1u ? 1u : d;
+        down = __uint_as_float(d << 23);
+        up = __uint_as_float((254u - d) << 23);
+    }
+
+    // The largest magnitude among the accumulators of the lane's query row (both lanes of the row).
+    DFX_D float row_magnitude(int qb) const {
+        float mx = 0.0f;
+#pragma unroll
+        for (int db = 0; db < S::NDB; ++db)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) mx = fmaxf(mx, fabsf(o[db][qb][e]));
+        return wave_xor32_max(mx);
+    }
+
+    DFX_D static uint32_t to_f16x2(float x, float y) {
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2{x, y}, f16x2));
+    }
+    DFX_D static f32x2 from_f16x2(uint32_t w) {
+        return __builtin_convertvector(__builtin_bit_cast(f16x2, w), f32x2);
+    }
+
     DFX_D void store_partial(int slot, const float (&l_tot)[NB]) const {
         if (wave >= a.busy_waves) return;  // no rows in any item of the launch: merge_partial skips it too
 #pragma unroll
         for (int qb = 0; qb < NB; ++qb) {
             const __amdgpu_buffer_rsrc_t rs = block_resource(slot, qb);
+            float down, up;
+            row_scale(row_magnitude(qb), down, up);
 #pragma unroll
-            for (int db = 0; db < S::NDB; ++db)
-#pragma unroll
-                for (int ii = 0; ii < 4; ++ii) {
-                    const f32x4 v = {o[db][qb][ii * 4 + 0], o[db][qb][ii * 4 + 1], o[db][qb][ii * 4 + 2],
-                                     o[db][qb][ii * 4 + 3]};
-                    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4v, v), rs,
-                                                           ((db * 4 + ii) * 64 + lane) * 16, 0, kDeviceScope);
-                }
-            const int ml = S::NDB * 16 * 64 * 4;
-            __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, m_run[qb]), rs, ml + lane * 4, 0,
-                                                  kDeviceScope);
-            __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, l_tot[qb]), rs, ml + 256 + lane * 4, 0,
-                                                  kDeviceScope);
+            for (int c = 0; c < kChunks; ++c) {
+                const int db = c >> 1, e0 = (c & 1) * 8;
+                u32x4v w;
+                w.x = to_f16x2(o[db][qb][e0 + 0] * down, o[db][qb][e0 + 1] * down);
+                w.y = to_f16x2(o[db][qb][e0 + 2] * down, o[db][qb][e0 + 3] * down);
+                w.z = to_f16x2(o[db][qb][e0 + 4] * down, o[db][qb][e0 + 5] * down);
+                w.w = to_f16x2(o[db][qb][e0 + 6] * down, o[db][qb][e0 + 7] * down);
+                __builtin_amdgcn_raw_buffer_store_b128(w, rs, (c * 64 + lane) * 16, 0, kDeviceScope);
+            }
+            const f32x4 st = {m_run[qb], l_tot[qb], up, 0.0f};
+            __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4v, st), rs, kStatsOff + lane * 16, 0,
+                                                   kDeviceScope);
         }
     }
 
-    // Merge one stored partial into the running state (l_run holds whole-row sums here).
+    // Round the accumulators to what store_partial() would have stored.  A workgroup that merges a
+    // stored piece into its own piece does this first: had the two arrived in the other order,
+    // the other side would have read this piece in its stored form, and the result must not
+    // depend on who merges.
+    DFX_D void round_to_stored_form() {
+        if (wave >= a.busy_waves) return;
+#pragma unroll
+        for (int qb = 0; qb < NB; ++qb) {
+            float down, up;
+            row_scale(row_magnitude(qb), down, up);
+#pragma unroll
+            for (int db = 0; db < S::NDB; ++db)
+#pragma unroll
+                for (int e = 0; e < 16; e += 2) {
+                    const f32x2 v = from_f16x2(to_f16x2(o[db][qb][e] * down, o[db][qb][e + 1] * down));
+                    o[db][qb][e] = v.x * up;
+                    o[db][qb][e + 1] = v.y * up;
+                }
+        }
+    }
+
+    // Merge one stored piece into the running state (l_run holds whole-row sums here).
     DFX_D void merge_partial(int slot) {
         // No fused multiply-add in here: a * wa + b * wb must round both products, or merging a
         // into b and b into a differ in the last bit (an fma keeps one product exact, and which
@@ -378,10 +436,9 @@ struct AttnState {
 #pragma unroll
         for (int qb = 0; qb < NB; ++qb) {
             const __amdgpu_buffer_rsrc_t rs = block_resource(slot, qb);
-            const int ml = S::NDB * 16 * 64 * 4;
-            const float mp = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rs, ml + lane * 4, 0, kDeviceScope));
-            const float lp =
-                __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rs, ml + 256 + lane * 4, 0, kDeviceScope));
+            const f32x4 st = __builtin_bit_cast(
+                f32x4, __builtin_amdgcn_raw_buffer_load_b128(rs, kStatsOff + lane * 16, 0, kDeviceScope));
+            const float mp = st[0], lp = st[1], up = st[2];
             const float mn = fmaxf(m_run[qb], mp);
             const float wa = (m_run[qb] == -INFINITY) ? 0.0f : fast_exp2(m_run[qb] - mn);
             const float wb = (mp == -INFINITY) ? 0.0f : fast_exp2(mp - mn);
@@ -391,17 +448,20 @@ struct AttnState {
             l_run[qb] = la + lb;
             m_run[qb] = mn;
 #pragma unroll
-            for (int db = 0; db < S::NDB; ++db)
+            for (int c = 0; c < kChunks; ++c) {
+                const int db = c >> 1, e0 = (c & 1) * 8;
+                const u32x4v w = __builtin_amdgcn_raw_buffer_load_b128(rs, (c * 64 + lane) * 16, 0, kDeviceScope);
+                const uint32_t ws[4] = {w.x, w.y, w.z, w.w};
 #pragma unroll
-                for (int ii = 0; ii < 4; ++ii) {
-                    const f32x4 v = __builtin_bit_cast(
-                        f32x4, __builtin_amdgcn_raw_buffer_load_b128(rs, ((db * 4 + ii) * 64 + lane) * 16, 0, kDeviceScope));
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        const float oa = o[db][qb][ii * 4 + j] * wa, ob = v[j] * wb;
-                        o[db][qb][ii * 4 + j] = oa + ob;
-                    }
+                for (int j = 0; j < 4; ++j) {
+                    const f32x2 h = from_f16x2(ws[j]);
+                    const float b0 = h.x * up, b1 = h.y * up;  // exact: a power of two
+                    const float oa0 = o[db][qb][e0 + 2 * j] * wa, ob0 = b0 * wb;
+                    const float oa1 = o[db][qb][e0 + 2 * j + 1] * wa, ob1 = b1 * wb;
+                    o[db][qb][e0 + 2 * j] = oa0 + ob0;
+                    o[db][qb][e0 + 2 * j + 1] = oa1 + ob1;
                 }
+            }
         }
     }
 };
@@ -466,6 +526,7 @@ DFX_D void finish_cut_item(AttnState<HD, NB, NW>& at, int rt, int64_t item_begin
     } else {
 #pragma unroll
         for (int qb = 0; qb < NB; ++qb) at.l_run[qb] = l_tot[qb];
+        at.round_to_stored_form();
     }
     for (int w = wa; w <= wb; ++w) {
         const int64_t ws = split.first(w);

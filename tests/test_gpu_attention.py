@@ -488,3 +488,33 @@ def test_block_causal_long_queries_on_an_fp8_cache(dev, flags):
     for max_wg in (0, 7):
         got = _run(wl.to(dev), max_workgroups=max_wg, flags=flags)
         assert max_abs_err(got, want) <= ATOL_FP8
+
+
+def _random_case(rng):
+    """A random but valid attention problem: shapes the operators accept, drawn from a seeded generator."""
+    hd = int(rng.choice([64, 128]))
+    h_kv = int(rng.choice([1, 2, 4, 8]))
+    group = int(rng.choice([1, 2, 4, 7, 8]))
+    page = int(rng.choice([16, 32, 48, 64, 256, 24, 1]))     # 24 and 1: pages the streaming path does not take
+    dbs = int(rng.choice([16, 32, 64]))
+    q_len = int(rng.choice([dbs, 2 * dbs, 3 * dbs, 8 * dbs]))
+    b = int(rng.integers(1, 7))
+    ctx = [int(x) for x in rng.choice([0, 1, 15, 63, 64, 65, 200, 511, 777], b)]
+    mask = MASK_BLOCK_CAUSAL if rng.random() < 0.5 else MASK_FULL
+    fp8 = bool(rng.random() < 0.3)
+    return dict(num_seqs=b, h_q=h_kv * group, h_kv=h_kv, hd=hd, page=page, ctx=ctx, q_len=q_len, dbs=dbs, mask=mask), fp8
+
+
+@pytest.mark.parametrize("seed", range(40))
+def test_random_shapes_against_oracle(dev, seed):
+    rng = np.random.default_rng(1000 + seed)
+    over, fp8 = _random_case(rng)
+    wl = make_workload("c5" if fp8 else "c1", seed=seed, **over)
+    want = oracle_fp32(wl)
+    tol = ATOL_FP8 if fp8 else ATOL_BF16
+    g = wl.to(dev)
+    for max_wg in (0, int(rng.integers(1, 40))):
+        for flags in PATHS:
+            got = _run(g, max_workgroups=max_wg, flags=flags)
+            assert torch.isfinite(got.float()).all(), (over, fp8, max_wg, flags)
+            assert max_abs_err(got, want) <= tol, (over, fp8, max_wg, flags)

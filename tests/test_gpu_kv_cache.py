@@ -173,3 +173,30 @@ def test_fp8_store_all_bf16_patterns_bit_exact(dev):
         dfx.store_kvcache_unified_layout(key.to(dev), key.to(dev), kc, vc, slots.to(dev), None,
                                          k_scale=ks.to(dev), v_scale=ks.to(dev))
         assert torch.equal(_bits(kc), _bits(want_k)) and torch.equal(_bits(vc), _bits(want_v))
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_random_shapes_store_and_load_bit_exact(dev, seed):
+    """Seeded random shapes (heads, head_dim, page sizes, ragged and empty contexts, bf16 and FP8):
+    store the fresh block, then gather; both against the oracle, bit for bit."""
+    rng = np.random.default_rng(500 + seed)
+    h_kv = int(rng.choice([1, 2, 4, 8]))
+    over = dict(num_seqs=int(rng.integers(1, 9)), h_q=h_kv, h_kv=h_kv, hd=int(rng.choice([64, 128])),
+                page=int(rng.choice([16, 32, 64, 256])), q_len=int(rng.choice([32, 64, 96])))
+    over["ctx"] = [int(x) for x in rng.choice([0, 1, 31, 32, 33, 255, 256, 257, 600], over["num_seqs"])]
+    fp8 = bool(rng.random() < 0.4)
+    wl = make_workload("c5" if fp8 else "c2", seed=seed, **over)
+    slots = wl.slot_mapping.clone()
+    slots[rng.random(slots.numel()) < 0.2] = -1
+    want_kc, want_vc = wl.k_cache.clone(), wl.v_cache.clone()
+    okv.store_unified(wl.k_new, wl.v_new, want_kc, want_vc, slots, wl.k_scale, wl.v_scale)
+    want_k, want_v = okv.load(want_kc, want_vc, wl.block_tables, wl.context_lens, wl.seq_lens_new,
+                              wl.cu_seqlens_q, wl.cu_seqlens_k, wl.k_new, wl.v_new, wl.k_scale, wl.v_scale)
+    g = wl.to(dev)
+    md = metadata_for(g, decode_mode="varlen")
+    dfx.store_kvcache_unified_layout(g.k_new, g.v_new, g.k_cache, g.v_cache,
+                                     slots.to(dev).to(torch.int64 if seed % 2 else torch.int32), md)
+    k_out, v_out = dfx.load_kvcache(g.k_cache, g.v_cache, md, g.k_new, g.v_new)
+    torch.cuda.synchronize()
+    assert torch.equal(_bits(g.k_cache), _bits(want_kc)) and torch.equal(_bits(g.v_cache), _bits(want_vc))
+    assert torch.equal(_bits(k_out), _bits(want_k)) and torch.equal(_bits(v_out), _bits(want_v))

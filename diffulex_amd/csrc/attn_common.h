@@ -467,78 +467,83 @@ struct AttnState {
 };
 
 // Epilogue of a piece of an item that the partition cut into pieces owned by consecutive
-// workgroups.  Every piece but the last one to finish is stored as a partial result; the
-// workgroup that finishes last merges the stored ones into its own registers and writes the
-// rows (bit-identical whichever piece that is).  Who is last is decided by an arrival counter per item (indexed by the workgroup that
-// owns the item's first unit; a workgroup owns at most one such cut item):
-//   - a workgroup that finds every other piece already arrived merges without storing its own
-//     (only the owner of the item's first units looks: the others are early by construction);
-//   - otherwise it stores its piece, waits until the stores have completed, and increments the
-//     counter; if that increment was the last arrival after all, it merges the others.
-// Nobody waits for anybody.  The last arrival resets the counter for the next launch.  Must be
-// called by every thread of the workgroup; l_tot are whole-row sums; `flag` is one int of LDS.
+// workgroups.  The pieces are merged pairwise up a fixed binary tree; nobody waits for anybody.
+//
+// Pieces are numbered from the item's end: piece 0 is the one its owner works on at the very
+// start of its range (the earliest to finish), piece p - 1 the one its owner reaches at the end of
+// its range (the latest).  At the level with subtrees of `half` pieces, the node that starts at
+// piece f (a multiple of 2 * half) joins subtree [f, f + half) with subtree [f + half, f + 2 *
+// half) if the latter exists; a subtree without a sibling moves up unchanged.  Whoever carries a
+// subtree's state arrives at the node through its arrival counter: the first of the two stores
+// the state (in the partial-result slot of the subtree's first piece, whose earlier contents have
+// been consumed by then) and leaves; the second merges the stored state into its own and carries
+// the result up; at the root it writes the rows.  The carrier of the later half looks at the
+// counter first and, if the other half is already there (the usual case), does not store at all.
+// Every merge takes both operands in their stored (rounded) form and is commutative bit for bit
+// (see merge_partial), and the tree is fixed, so the rows do not depend on the order of arrival.
+// With the late pieces at the high end, the workgroup that reaches its piece last has the fewest
+// merges left to do: the others have met lower in the tree, while they had time to spare.
+//
+// The counter of the node whose second subtree starts at piece r is the one indexed by the
+// workgroup that owns piece r (r >= 1: those workgroups own the item's units but not its last
+// ones, and no two items share such a workgroup).  Must be called by every thread of the
+// workgroup; l_tot are whole-row sums; `flag` is one int of LDS.  Returns whether this workgroup
+// wrote the rows.
 template <int HD, int NB, int NW>
-DFX_D void finish_cut_item(AttnState<HD, NB, NW>& at, int rt, int64_t item_begin, int n_tiles, const WgSplit& split,
+DFX_D bool finish_cut_item(AttnState<HD, NB, NW>& at, int rt, int64_t item_begin, int n_tiles, const WgSplit& split,
                            int my_slot, const float (&l_tot)[NB], int* flag) {
     const KArgs& a = at.a;
     const int me = static_cast<int>(blockIdx.x);
+    const int64_t item_last = item_begin + n_tiles - 1;
+    // with fewer units than workgroups every workgroup owns one unit or none: each unit is a piece
+    const bool sparse = split.q == 0;
+    const int64_t total = split.q * split.n_wg + split.r;
     int wa, wb;
-    owners_of_units(split, me, item_begin, item_begin + n_tiles - 1, wa, wb);
-    int pieces = wb - wa + 1;
-    if (split.q == 0) {  // fewer units than workgroups: some ranges are empty
-        pieces = 0;
-        for (int w = wa; w <= wb; ++w)
-            if (split.first(w) < split.first(w + 1)) ++pieces;
-    }
-    int* counter = a.arrivals + wa;
-
-    // The owner of the item's first units works on them at the end of its range, every other
-    // owner at the start of its own: only the former is likely to find the others arrived, the
-    // others skip the look (a round trip to memory) and go straight to storing.
-    bool last = false;
-    if (me == wa) {
-        if (threadIdx.x == 0) *flag = __hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __syncthreads();
-        last = *flag == pieces - 1;
-        __syncthreads();
-    }
-    bool stored = false;
-    if (!last || pieces > 2) {
-        at.store_partial(my_slot, l_tot);
-        __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this thread's write-through stores have completed
-        stored = true;
-    }
-    if (!last) {
-        __syncthreads();
-        if (threadIdx.x == 0) *flag = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __syncthreads();
-        last = *flag == pieces - 1;
-        __syncthreads();
-        if (!last) return;
-    }
-    // The result must not depend on which piece arrives last.  Two pieces: the merge is
-    // commutative bit for bit (see merge_partial).  More (rare): every piece, this one included,
-    // is merged from memory in workgroup order, starting from the empty state.
-    const bool from_memory = pieces > 2;
-    if (from_memory) {
-        __syncthreads();  // every thread's stores of this piece have completed
-        at.reset_accumulators();
-    } else {
-#pragma unroll
-        for (int qb = 0; qb < NB; ++qb) at.l_run[qb] = l_tot[qb];
-        at.round_to_stored_form();
-    }
-    for (int w = wa; w <= wb; ++w) {
+    owners_of_units(split, me, item_begin, item_last, wa, wb);
+    const int p = sparse ? n_tiles : wb - wa + 1;
+    auto owner_of_piece = [&](int j) { return sparse ? wg_of_unit(item_last - j, total, split.n_wg) : wb - j; };
+    auto slot_of_piece = [&](int j) {
+        const int w = owner_of_piece(j);
         const int64_t ws = split.first(w);
-        if ((w == me && !from_memory) || ws >= split.first(w + 1)) continue;
-        at.merge_partial(partial_slot(w, ws > item_begin ? ws : item_begin, ws));
+        return partial_slot(w, ws > item_begin ? ws : item_begin, ws);
+    };
+    int j = sparse ? static_cast<int>(item_last - split.first(me)) : wb - me;  // the first piece of the subtree carried
+    (void)my_slot;  // == slot_of_piece(j)
+#pragma unroll
+    for (int qb = 0; qb < NB; ++qb) at.l_run[qb] = l_tot[qb];
+
+    for (int half = 1; half < p; half <<= 1) {
+        const bool later_half = (j & half) != 0;
+        const int second = (j & ~(2 * half - 1)) + half;  // first piece of the node's second subtree
+        if (!later_half && second >= p) continue;         // no sibling at this level
+        int* counter = a.arrivals + owner_of_piece(second);
+        bool sibling_there = false;
+        if (later_half) {
+            if (threadIdx.x == 0) *flag = __hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __syncthreads();
+            sibling_there = *flag == 1;
+            __syncthreads();
+        }
+        if (!sibling_there) {
+            at.store_partial(slot_of_piece(j), at.l_run);
+            __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this thread's write-through stores have completed
+            __syncthreads();
+            if (threadIdx.x == 0) *flag = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __syncthreads();
+            sibling_there = *flag == 1;
+            __syncthreads();
+            if (!sibling_there) return false;  // the sibling's carrier will find this state
+        }
+        at.round_to_stored_form();
+        at.merge_partial(slot_of_piece(later_half ? second - half : second));
+        if (threadIdx.x == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        j &= ~(2 * half - 1);
     }
-    (void)stored;
     float l_all[NB];
 #pragma unroll
     for (int qb = 0; qb < NB; ++qb) l_all[qb] = at.l_run[qb];
     at.store_output(rt, l_all);
-    if (threadIdx.x == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return true;
 }
 
 // Fused KV-cache store: fresh row t of k_new / v_new goes to cache slot store_slots[t] (what

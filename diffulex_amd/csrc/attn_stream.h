@@ -305,15 +305,19 @@ struct StreamAttn : TileMath<HD, NB, NW> {
     }
 
     // Close the item whose last unit of this workgroup's piece is planned unit `last_rel`.
-    DFX_D void finish_run(int last_rel, const WgSplit& split) {
+    // Returns 0 (the run goes on in the next plan), 1 (rows written), 2 (piece stored), 3 (pieces merged).
+    DFX_D int finish_run(int last_rel, const WgSplit& split) {
         const UnitDesc e = units[last_rel];
-        if (!(uniform(e.flags) & kUnitLast)) return;
+        if (!(uniform(e.flags) & kUnitLast)) return 0;
         this->outputs_ready();
         float l_tot[NB];
         this->row_sums(l_tot);
-        if (uniform(e.flags) & kUnitComplete) this->store_output(uniform(e.rt), l_tot);
-        else finish_cut_item(*this, uniform(e.rt), begin + uniform(e.item_rel), uniform(e.n_tiles), split,
-                             uniform(e.slot), l_tot, misc + kMaxWaves + 1);
+        if (uniform(e.flags) & kUnitComplete) {
+            this->store_output(uniform(e.rt), l_tot);
+            return 1;
+        }
+        return finish_cut_item(*this, uniform(e.rt), begin + uniform(e.item_rel), uniform(e.n_tiles), split,
+                               uniform(e.slot), l_tot, misc + kMaxWaves + 1) ? 3 : 2;
     }
 
     // Wait until at most `younger` units' loads of this wave are outstanding (younger <= 2).
@@ -329,11 +333,26 @@ __global__ void __launch_bounds__(64 * NW, COMPACT ? 2 : 1) paged_attn_stream_ke
     extern __shared__ __attribute__((aligned(256))) uint8_t smem[];
     using C = StreamCfg<HD, NB, NW, COMPACT>;
     StreamAttn<HD, NB, NW, COMPACT> at(a, smem);
+#ifdef DFX_TRACE
+    // Development build: thread 0 accumulates phase times (100 MHz clock) in LDS and leaves them
+    // in the unused upper part of the counter area: [0] entry, [1] prefix built, [2] first plan
+    // done, [3] ring filled and queries in, [4] exit, [5] tile loops, [6] tiles, [7..9] time of
+    // epilogues that wrote rows / stored a piece / merged, [10..12] their counts, [13] begin_item.
+    long long* tr = reinterpret_cast<long long*>(smem + C::LDS_BYTES);
+    if (threadIdx.x == 0) {
+        for (int i = 0; i < 16; ++i) tr[i] = 0;
+        tr[0] = wall_clock64();
+    }
+#define DFX_T(i) do { if (threadIdx.x == 0) tr[i] = wall_clock64(); } while (0)
+#else
+#define DFX_T(i) do {} while (0)
+#endif
     // The fused cache store comes first, while next to nothing is live in registers: anywhere
     // later its address arithmetic would push values of the tile loop out of their registers.
     store_fresh_rows<HD, false>(a);
     const UnitSummary summary = build_unit_prefix<C::RT>(a, at.prefix, at.misc);
     at.per_head = summary.per_head;
+    DFX_T(1);
     const int64_t total = static_cast<int64_t>(at.per_head) * a.h_kv;
     if (total == 0) return;
     const int w = blockIdx.x;
@@ -351,6 +370,9 @@ __global__ void __launch_bounds__(64 * NW, COMPACT ? 2 : 1) paged_attn_stream_ke
         __syncthreads();  // every wave is done with the previous plan and its stages
         at.plan_units(chunk, n_units);
         __syncthreads();
+#ifdef DFX_TRACE
+        if (chunk == begin) DFX_T(2);
+#endif
 
         // An item that opens with this plan: its query rows are requested ahead of the ring fill,
         // so that their (cold) latency runs concurrently with that of the first tiles.
@@ -359,6 +381,9 @@ __global__ void __launch_bounds__(64 * NW, COMPACT ? 2 : 1) paged_attn_stream_ke
         int issued = 0;  // ring fill: kStages - 1 units in flight
         for (; issued < C::kStages - 1 && issued < n_units; ++issued) at.issue_unit(issued);
         at.touch_queries();  // unconditional: the compiler must see no path into the tile loop with these loads pending
+#ifdef DFX_TRACE
+        if (chunk == begin) DFX_T(3);
+#endif
 
         int rel = 0;
         while (rel < n_units) {
@@ -366,7 +391,19 @@ __global__ void __launch_bounds__(64 * NW, COMPACT ? 2 : 1) paged_attn_stream_ke
             const UnitDesc d = at.units[rel];
             const int flags = uniform(d.flags);
             const int run_end = min(rel + uniform(d.run), n_units);
+#ifdef DFX_TRACE
+            long long tb = 0;
+            if (threadIdx.x == 0) tb = wall_clock64();
+#endif
             if ((flags & kUnitFirst) && rel != 0) at.begin_item(d);
+#ifdef DFX_TRACE
+            long long ts = 0;
+            if (threadIdx.x == 0) {
+                ts = wall_clock64();
+                tr[13] += ts - tb;
+                tr[6] += run_end - rel;
+            }
+#endif
             for (; rel < run_end; ++rel) {
                 // the unit must have landed: only younger units may still be outstanding
                 at.wait_younger(issued - rel - 1);
@@ -393,9 +430,29 @@ __global__ void __launch_bounds__(64 * NW, COMPACT ? 2 : 1) paged_attn_stream_ke
                     at.outputs_untouched();
                 }
             }
+#ifdef DFX_TRACE
+            long long te = 0;
+            if (threadIdx.x == 0) {
+                te = wall_clock64();
+                tr[5] += te - ts;
+            }
+            const int kind = at.finish_run(rel - 1, split);
+            if (threadIdx.x == 0 && kind > 0) {
+                tr[6 + kind] += wall_clock64() - te;
+                tr[9 + kind] += 1;
+            }
+#else
             at.finish_run(rel - 1, split);
+#endif
         }
     }
+#ifdef DFX_TRACE
+    if (threadIdx.x == 0) {
+        tr[4] = wall_clock64();
+        long long* out = reinterpret_cast<long long*>(a.arrivals + 16384) + blockIdx.x * 16;
+        for (int i = 0; i < 16; ++i) out[i] = tr[i];
+    }
+#endif
 }
 
 // FP8-E4M3 context cache (fresh K/V stay bf16).  The ring stages hold the codes as stored; in

@@ -99,6 +99,9 @@ int launch(const KArgs& ka, const Plan& plan, hipStream_t st) {
         } else {
             main_k = paged_attn_stream_kernel<HD, 1, NW, false>;
             lds = StreamCfg<HD, 1, NW, false>::LDS_BYTES;
+#ifdef DFX_TRACE
+            lds += 128;  // the phase timers of the development build
+#endif
         }
         threads = 64 * NW;
     } else {

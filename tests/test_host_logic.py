@@ -282,3 +282,65 @@ def test_masked_partition_covers_every_visible_tile_once(seed):
                 pieces = sorted(seen[(kvh, s, rt)])
                 assert pieces[0][0] == 0 and pieces[-1][1] == nt
                 assert all(a[1] == bb[0] for a, bb in zip(pieces, pieces[1:]))
+
+
+def _simulate_tree_merge(p, order_rng):
+    """Model of the pairwise arrival protocol of finish_cut_item (csrc/attn_common.h): p pieces,
+    each carried by its own workgroup, interleaved at the granularity of their memory operations
+    in a random order.  Returns (pieces in the state that reached the root, rows written, counters)."""
+    counters = {}
+    slots = {}            # first piece of a subtree -> frozenset of the pieces in the stored state
+    written = []
+
+    def worker(j):
+        state = frozenset([j])
+        half = 1
+        while half < p:
+            later = (j & half) != 0
+            second = (j & ~(2 * half - 1)) + half
+            if not later and second >= p:
+                half <<= 1
+                continue
+            there = False
+            if later:
+                yield
+                there = counters.get(second, 0) == 1
+            if not there:
+                yield
+                slots[j] = state
+                yield
+                old = counters.get(second, 0)
+                counters[second] = old + 1
+                there = old == 1
+                if not there:
+                    return
+            yield
+            sib = second - half if later else second
+            other = slots[sib]
+            assert not (other & state), "a piece merged twice"
+            lo = j & ~(2 * half - 1)
+            assert other == frozenset(range(sib, min(sib + half, p))), "sibling state is not its subtree"
+            state = state | other
+            yield
+            counters[second] = 0
+            j = lo
+            half <<= 1
+        written.append(state)
+
+    live = [worker(j) for j in range(p)]
+    while live:
+        g = live[order_rng.integers(len(live))]
+        try:
+            next(g)
+        except StopIteration:
+            live.remove(g)
+    return written, counters
+
+
+@pytest.mark.parametrize("p", [2, 3, 4, 5, 6, 7, 8, 9, 13, 16, 33])
+def test_pairwise_merge_protocol_model(p):
+    for seed in range(200):
+        written, counters = _simulate_tree_merge(p, np.random.default_rng(seed * 1000 + p))
+        assert len(written) == 1, "the rows are written exactly once"
+        assert written[0] == frozenset(range(p)), "every piece reaches the root"
+        assert all(v == 0 for v in counters.values()), "every counter is left at zero"

@@ -104,14 +104,14 @@ DFX_HD void locate_unit(const SeqShape& s, int u, int& rt, int& tile, int& item_
 }
 
 // How many of the n_wg workgroups of the launch take part.  Cutting an item into p pieces costs
-// a merge whose time grows with p, so a workgroup should own at least about 2 * sqrt(tiles of
-// the longest item) units (near the point where the time of its own tiles equals the merge time
-// they save; the factor is the best of 0.75 .. 2.5 measured for batches of 1 .. 32 at 2K .. 32K), but there is never a reason to use fewer workgroups than there are items.  Small
-// batches with long contexts are the case this matters for.  Integer arithmetic only: every
-// workgroup (and the host-side tests) must arrive at the same number.
+// log2(p) rounds of a pairwise merge on top of the pieces' own tiles, so a workgroup should own at
+// least about sqrt(tiles of the longest item) units (the best of 0.35 .. 2 times that, measured
+// for batches of 1 .. 32 at 2K .. 32K), but there is never a reason to use fewer workgroups than
+// there are items.  Small batches with long contexts are the case this matters for.  Integer
+// arithmetic only: every workgroup (and the host-side tests) must arrive at the same number.
 DFX_HD int effective_workgroups(int64_t total_units, int64_t n_items, int max_tiles, int n_wg) {
-    int r = 0;  // floor(2 * sqrt(max_tiles))
-    while (static_cast<int64_t>(r + 1) * (r + 1) <= static_cast<int64_t>(max_tiles) * 4) ++r;
+    int r = 0;  // floor(sqrt(max_tiles))
+    while (static_cast<int64_t>(r + 1) * (r + 1) <= static_cast<int64_t>(max_tiles)) ++r;
     const int min_units = r > 4 ? r : 4;
     int64_t n = (total_units + min_units - 1) / min_units;
     if (n < n_items) n = n_items;

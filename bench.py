@@ -31,7 +31,7 @@ HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this command, scaled by
 # what the same counters read for a plain copy of known size (one summary per workload under profiles/).
-MEASURED_TRAFFIC_BYTES = {"c3": 252.9e6, "c4": 1455.3e6, "c5": 821.6e6}
+MEASURED_TRAFFIC_BYTES = {"c3": 251.5e6, "c4": 1455.4e6, "c5": 821.6e6}
 
 
 def algorithmic_bytes(wl) -> int:

@@ -130,3 +130,64 @@ def test_empty_input_is_a_no_op(dev):
     k = torch.empty(0, 4 * 128, dtype=torch.bfloat16, device=dev)
     got_q, got_k = rope(torch.empty(0, dtype=torch.int64, device=dev), q, k)
     assert got_q.shape == q.shape and got_k.shape == k.shape
+
+
+def test_layer_step_rope_store_attention_eager_and_in_a_graph(dev):
+    """One decode step of an attention layer as the reference's model runs it
+    (diffulex/model/dream.py:94-99): rotate q and k, store the rotated k and v, attend.  The fused
+    rope + store launch followed by attention without its own store, eagerly and replayed from a
+    captured graph, against the oracle pipeline (rotary -> store -> attention)."""
+    import diffulex_amd as dfx
+    from diffulex_amd.workloads import make_workload
+    from oracle import attention as oat
+    wl = make_workload("c3", num_seqs=5, ctx=(200, 900), seed=23)
+    t, hq, hkv, hd = wl.q.shape[0], wl.num_q_heads, wl.num_kv_heads, wl.head_dim
+    gen = torch.Generator().manual_seed(24)
+    # each fresh token sits right behind its sequence's context
+    pos = torch.cat([wl.context_lens[s] + torch.arange(wl.q_len) for s in range(wl.num_seqs)]).long()
+    tab = orot.cos_sin_cache(hd, MAXPOS, BASE)
+    q2, k2, v2 = wl.q.reshape(t, -1), wl.k_new.reshape(t, -1), wl.v_new.reshape(t, -1)
+    rq, rk = orot.apply_rotary(q2, pos, tab, hd), orot.apply_rotary(k2, pos, tab, hd)
+    want_kc, want_vc = wl.k_cache.clone(), wl.v_cache.clone()
+    okv.store_unified(rk.view(t, hkv, hd), wl.v_new, want_kc, want_vc, wl.slot_mapping)
+    want = oat.paged_attention_fp32(rq.view(t, hq, hd), rk.view(t, hkv, hd), wl.v_new, wl.k_cache, wl.v_cache,
+                                    wl.block_tables, wl.context_lens, wl.cu_seqlens_q, wl.cu_seqlens_q, wl.scale)
+
+    g = wl.to(dev)
+    rope = _rope(hd, dev)
+    att = dfx.Attention(hq, hd, g.scale, hkv)
+    att.k_cache, att.v_cache = g.k_cache, g.v_cache
+    md = dfx.PagedAttnMetaData(cu_seqlens_q=g.cu_seqlens_q, cu_seqlens_k=g.cu_seqlens_q, max_seqlen_q=g.q_len,
+                               slot_mapping=g.slot_mapping, context_lens=g.context_lens, block_tables=g.block_tables,
+                               page_block_size=g.page_size, decode_mode="static", need_kv_cache_store=False)
+    dfx.set_fetch_fn_for_attn_metadata(lambda: md)
+    gq, gk, gv, gpos = q2.to(dev), k2.to(dev), v2.to(dev), pos.to(dev)
+
+    def layer():
+        q_r, k_r = rope.forward_and_store(gpos, gq, gk, gv, att.k_cache, att.v_cache, md.slot_mapping, md)
+        return att(q_r, k_r, gv)
+
+    out = layer()
+    torch.cuda.synchronize()
+    assert torch.equal(_bits(g.k_cache), _bits(want_kc)) and torch.equal(_bits(g.v_cache), _bits(want_vc))
+    assert float((out.view(t, hq, hd).float().cpu() - want).abs().max()) <= 2e-2
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        layer()                                   # the capture stream's workspace exists before the capture
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        o_static = layer()
+    dgen = torch.Generator(device=dev).manual_seed(9)
+    for rep in range(3):
+        for x in (gq, gk, gv):
+            x.copy_(torch.randn(x.shape, generator=dgen, device=dev, dtype=torch.float32).to(x.dtype))
+        graph.replay()
+        torch.cuda.synchronize()
+        got = o_static.clone()
+        eager = layer()
+        torch.cuda.synchronize()
+        assert torch.equal(got, eager), f"replay {rep}"

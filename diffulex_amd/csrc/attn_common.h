@@ -357,9 +357,9 @@ struct AttnState {
 
     // 2^-(exponent of mx) and its inverse (1 for zero); mx >= 0.
     DFX_D static void row_scale(float mx, float& down, float& up) {
-        const uint32_t e = (__float_as_uint(mx) >> 23) & 0xffu;
-        uint32_t d = e == 0 ? 127u : 254u - e;
-        d = d < 1u ? 1u : d;
+        uint32_t e = (__float_as_uint(mx) >> 23) & 0xffu;
+        e = e > 253u ? 253u : e;  // infinities and NaNs stay what they are in fp16 whatever the scale
+        const uint32_t d = e == 0 ? 127u : 254u - e;
         down = __uint_as_float(d << 23);
         up = __uint_as_float((254u - d) << 23);
     }

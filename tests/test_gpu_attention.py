@@ -518,3 +518,26 @@ def test_random_shapes_against_oracle(dev, seed):
             got = _run(g, max_workgroups=max_wg, flags=flags)
             assert torch.isfinite(got.float()).all(), (over, fp8, max_wg, flags)
             assert max_abs_err(got, want) <= tol, (over, fp8, max_wg, flags)
+
+
+@pytest.mark.parametrize("flags", PATHS)
+def test_non_finite_inputs_stay_inside_their_sequence(dev, flags):
+    """A NaN in one sequence's cached V and an infinity in another's fresh K make those sequences'
+    rows non-finite (as in the oracle) and leave every other sequence exactly as without them,
+    whatever the partition."""
+    wl = make_workload("c3", seed=51, num_seqs=5, ctx=(300, 900))
+    g = wl.to(dev)
+    clean = {mw: _run(g, max_workgroups=mw, flags=flags) for mw in (0, 9)}
+    page = int(wl.block_tables[1, 0])
+    g.v_cache[page, 3, 1, 17] = float("nan")                   # sequence 1, context token 3
+    t3 = int(wl.cu_seqlens_q[3])
+    g.k_new[t3 + 5, 2, 40] = float("inf")                      # sequence 3, fresh token 5
+    cu = wl.cu_seqlens_q.tolist()
+    for mw in (0, 9):
+        got = _run(g, max_workgroups=mw, flags=flags)
+        for s in range(wl.num_seqs):
+            rows = slice(cu[s], cu[s + 1])
+            if s in (1, 3):
+                assert not torch.isfinite(got[rows].float()).all()
+            else:
+                assert torch.equal(got[rows], clean[mw][rows])

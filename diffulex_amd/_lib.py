@@ -10,12 +10,13 @@ from pathlib import Path
 
 LIB_PATH = Path(__file__).resolve().parent / "libdiffulex_amd.so"
 
-DFX_ABI_VERSION = 3
+DFX_ABI_VERSION = 4
 DFX_OK = 0
 DFX_KV_BF16, DFX_KV_FP8_E4M3 = 0, 1
 DFX_MASK_FULL, DFX_MASK_BLOCK_CAUSAL = 0, 1
 DFX_INDEX_I32, DFX_INDEX_I64 = 0, 1
 DFX_ATTN_GENERIC_PATH = 1
+DFX_WORKSPACE_COUNTER_BYTES = 1 << 18
 
 EXPORTS = (
     "dfx_abi_version", "dfx_status_string", "dfx_kv_store_unified", "dfx_kv_store_distinct",

@@ -65,10 +65,11 @@ struct Shape {
     static constexpr int PREFIX_BYTES = (kMaxSeqs + 1) * 4;
     static constexpr int MISC_BYTES = 128;
     // A partial result is stored per 32-row query block b = wave * NB + qb, whatever the shape of
-    // the workgroup that wrote it, in an area of BLOCK_FLOATS floats (the format, which uses a
-    // little over half of it, is described at AttnState::store_partial).
+    // the workgroup that wrote it, in an area of BLOCK_FLOATS floats: 2 * NDB chunks of 64 x 16
+    // bytes of fp16 accumulators, then 64 x 16 bytes of row statistics (the format is described at
+    // AttnState::store_partial).
     static constexpr int BLOCKS = NB * NW;
-    static constexpr int BLOCK_FLOATS = 64 * (NDB * 16 + 2);
+    static constexpr int BLOCK_FLOATS = 256 * (2 * NDB + 1);
     static constexpr int SLOT_FLOATS = BLOCKS * BLOCK_FLOATS;
 };
 
@@ -353,7 +354,7 @@ struct AttnState {
     typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
     static constexpr int kChunks = S::NDB * 2;
     static constexpr int kStatsOff = kChunks * 64 * 16;
-    static_assert(kStatsOff + 64 * 16 <= S::BLOCK_FLOATS * 4, "a block fits its slot");
+    static_assert(kStatsOff + 64 * 16 == S::BLOCK_FLOATS * 4, "a block fills its slot exactly");
 
     // 2^-(exponent of mx) and its inverse (1 for zero); mx >= 0.
     DFX_D static void row_scale(float mx, float& down, float& up) {

@@ -74,7 +74,8 @@ int make_plan(const dfx_attn_params* p, Plan& plan) {
 // workgroup.  The counter area has the same size whatever the launch (room for the largest
 // grid): calls with different workgroup counts may share a workspace, and the counters must
 // never land where an earlier call left partial results.
-int64_t counter_bytes(const Plan&) { return (static_cast<int64_t>(kMaxWorkgroups) + 1) * 4; }
+static_assert((kMaxWorkgroups + 1) * 4 == DFX_WORKSPACE_COUNTER_BYTES, "one counter per workgroup of the largest grid");
+int64_t counter_bytes(const Plan&) { return DFX_WORKSPACE_COUNTER_BYTES; }
 int64_t plan_workspace_bytes(const Plan& plan) {
     return counter_bytes(plan) + 2 * static_cast<int64_t>(plan.n_wg) * plan.slot_floats * 4;
 }
@@ -133,13 +134,20 @@ extern "C" int64_t dfx_paged_attn_workspace_bytes(const dfx_attn_params* p) {
     return plan_workspace_bytes(plan);
 }
 
-extern "C" int dfx_paged_attn(const dfx_attn_params* p, dfx_stream_t stream) {
-    Plan plan;
+namespace {
+
+// Argument checks shared by the entry points (everything but the workspace).  `empty`: the call is
+// valid and there is nothing to launch.
+int check_args(const dfx_attn_params* p, Plan& plan, bool& empty) {
+    empty = false;
     const int rc = make_plan(p, plan);
     if (rc != DFX_OK) return rc;
     // no query rows, no launch: a store asked for with such a call would be skipped silently
     if (p->store_slot_mapping != nullptr && p->num_seqs > 0 && p->max_seqlen_q == 0) return DFX_ERR_INVALID_ARG;
-    if (p->num_seqs == 0 || p->max_seqlen_q == 0) return DFX_OK;
+    if (p->num_seqs == 0 || p->max_seqlen_q == 0) {
+        empty = true;
+        return DFX_OK;
+    }
     if (!p->q || !p->k_new || !p->v_new || !p->out || !p->cu_seqlens_q || !p->cu_seqlens_new)
         return DFX_ERR_INVALID_ARG;
     const bool has_cache = p->k_cache != nullptr;
@@ -167,8 +175,19 @@ extern "C" int dfx_paged_attn(const dfx_attn_params* p, dfx_stream_t stream) {
             return DFX_ERR_INVALID_ARG;
         if (!aligned16(p->k_cache) || !aligned16(p->v_cache)) return DFX_ERR_INVALID_ARG;
     }
+    return DFX_OK;
+}
+
+// Checks and launch; `workspace` replaces p->workspace.
+int run_paged_attn(const dfx_attn_params* p, void* workspace, int64_t workspace_bytes, dfx_stream_t stream) {
+    Plan plan;
+    bool empty;
+    const int rc = check_args(p, plan, empty);
+    if (rc != DFX_OK || empty) return rc;
+    const bool has_cache = p->k_cache != nullptr;
     const int64_t need = plan_workspace_bytes(plan);
-    if (plan.n_wg > 1 && (p->workspace == nullptr || p->workspace_bytes < need || !aligned16(p->workspace)))
+    if (plan.n_wg > 1 && (workspace == nullptr || workspace_bytes < need ||
+                          (reinterpret_cast<uintptr_t>(workspace) & 255u) != 0))
         return DFX_ERR_WORKSPACE;
 
     KArgs ka;
@@ -186,8 +205,8 @@ extern "C" int dfx_paged_attn(const dfx_attn_params* p, dfx_stream_t stream) {
     ka.v_scale = p->v_scale;
     ka.store_slots = has_cache ? p->store_slot_mapping : nullptr;
     ka.store_slots_i64 = p->store_slot_index_type == DFX_INDEX_I64;
-    ka.arrivals = static_cast<int*>(p->workspace);
-    ka.workspace = reinterpret_cast<float*>(static_cast<uint8_t*>(p->workspace) + counter_bytes(plan));
+    ka.arrivals = static_cast<int*>(workspace);
+    ka.workspace = reinterpret_cast<float*>(static_cast<uint8_t*>(workspace) + counter_bytes(plan));
     ka.q_st = p->q_stride_token;
     ka.q_sh = p->q_stride_head;
     ka.kn_st = p->kn_stride_token;
@@ -237,4 +256,11 @@ extern "C" int dfx_paged_attn(const dfx_attn_params* p, dfx_stream_t stream) {
     DFX_ATTN_CASE(128, 2)
 #undef DFX_ATTN_CASE
     return DFX_ERR_UNSUPPORTED;
+}
+
+}  // namespace
+
+extern "C" int dfx_paged_attn(const dfx_attn_params* p, dfx_stream_t stream) {
+    if (p == nullptr) return DFX_ERR_INVALID_ARG;
+    return run_paged_attn(p, p->workspace, p->workspace_bytes, stream);
 }

@@ -15,17 +15,44 @@ import torch
 from . import _lib
 from .kv_cache_kernels import _FP8_DTYPES, _index_type, _scales, _stream
 
-_workspaces = {}
+class _Workspace:
+    __slots__ = ("tensor", "zeroed")
+
+    def __init__(self, tensor):
+        self.tensor = tensor
+        self.zeroed = False  # an executed (not merely captured) fill has cleared the arrival counters
+
+
+_workspaces = {}   # (device index, stream handle | "capture") -> _Workspace
+_retired = []      # outgrown workspaces stay alive: graphs captured earlier still point at them
 
 
 def _workspace(device: torch.device, stream: int, nbytes: int) -> torch.Tensor:
-    key = (device.index, stream)
-    ws = _workspaces.get(key)
-    if ws is None or ws.numel() < nbytes:
-        # zero-filled once: the arrival counters at its start must be 0 before the first launch
-        ws = torch.zeros(max(nbytes, 1), dtype=torch.uint8, device=device)
-        _workspaces[key] = ws
-    return ws
+    """Scratch of ``dfx_paged_attn`` for this device and stream.  Eager calls use one workspace per
+    stream; calls recorded into a graph share one per device (replays run on whatever stream is
+    current then, so the capture stream means nothing), which every eager call keeps allocated and
+    cleared at the size it needs itself: the usual warm-up-then-capture order records nothing extra.
+    A capture that finds no cleared workspace records a fill of the counter area in front of the
+    launch, and keeps doing so in every capture until an eager call has cleared it for real."""
+    capturing = torch.cuda.is_current_stream_capturing()
+    nbytes = max(int(nbytes), _lib.DFX_WORKSPACE_COUNTER_BYTES)
+
+    def get(key):
+        ws = _workspaces.get(key)
+        if ws is None or ws.tensor.numel() < nbytes:
+            if ws is not None:
+                _retired.append(ws.tensor)
+            ws = _Workspace(torch.empty(nbytes, dtype=torch.uint8, device=device))
+            _workspaces[key] = ws
+        if not ws.zeroed:
+            ws.tensor[:_lib.DFX_WORKSPACE_COUNTER_BYTES].zero_()  # a fill kernel, never a memset node
+            ws.zeroed = not capturing
+        return ws
+
+    if capturing:
+        return get((device.index, "capture")).tensor
+    get((device.index, "capture"))
+    return get((device.index, stream)).tensor
 
 
 def paged_attention(q, k, v, k_cache, v_cache, scale, *, block_tables, context_lens, cu_seqlens_q,
@@ -91,10 +118,10 @@ def paged_attention(q, k, v, k_cache, v_cache, scale, *, block_tables, context_l
             f"`N`: {k.shape[0]}, `slot_mapping.numel()`: {store_slot_mapping.numel()}"
         p.store_slot_mapping = store_slot_mapping.data_ptr()
         p.store_slot_index_type = _index_type(store_slot_mapping)
+    stream = _stream()
     need = lib.dfx_paged_attn_workspace_bytes(C.byref(p))
     if need < 0:
         _lib.check(int(need), "dfx_paged_attn_workspace_bytes")
-    stream = _stream()
     ws = _workspace(q.device, stream, int(need))
     p.workspace, p.workspace_bytes = ws.data_ptr(), ws.numel()
     _lib.check(lib.dfx_paged_attn(C.byref(p), stream), "dfx_paged_attn")

@@ -19,7 +19,7 @@
 extern "C" {
 #endif
 
-#define DFX_ABI_VERSION 3
+#define DFX_ABI_VERSION 4
 
 typedef void* dfx_stream_t; /* a hipStream_t; NULL is the default stream */
 
@@ -184,10 +184,11 @@ typedef struct dfx_attn_params {
 
 /* Bytes of scratch dfx_paged_attn needs for these shapes (depends on the sizes
  * and max_workgroups only, never on device data). Negative: dfx_status.
- * The workspace starts with one arrival counter per workgroup, which the kernel
- * expects to be zero and resets before it ends: zero-fill a new workspace once
- * (hipMemsetAsync, or a fill kernel under graph capture).  Calls that share a
- * workspace must not overlap in time. */
+ * The workspace starts with DFX_WORKSPACE_COUNTER_BYTES of arrival counters, which
+ * the kernel expects to be zero and resets before it ends: zero-fill that area of a
+ * new workspace once (hipMemsetAsync, or a fill kernel under graph capture).  Calls
+ * that share a workspace must not overlap in time. */
+#define DFX_WORKSPACE_COUNTER_BYTES (1 << 18)
 int64_t dfx_paged_attn_workspace_bytes(const dfx_attn_params* params);
 
 int dfx_paged_attn(const dfx_attn_params* params, dfx_stream_t stream);

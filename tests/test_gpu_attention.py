@@ -321,6 +321,41 @@ def test_static_decode_in_a_captured_graph(dev):
     assert max_abs_err(got.view(t, wl.num_q_heads, wl.head_dim), oracle_fp32(wl2)) <= ATOL_BF16
 
 
+def test_graphs_captured_as_the_reference_runner_does(dev):
+    """strategy/block_diffusion/engine/model_runner.py:239-262: warm up on the current stream, then
+    capture one graph per batch size, largest first, on the capture context's own side stream.
+    Here the smaller graph is replayed first, and the eager warm-up uses a smaller batch than the
+    first capture (so the capture needs a larger workspace than any eager call has made)."""
+    sizes = (12, 5)
+    wls = {n: make_workload("c3", num_seqs=n, ctx=(300, 1100), seed=50 + n).to(dev) for n in sizes}
+    att = dfx.Attention(28, 128, wls[5].scale, 4)
+    cur = {}
+    dfx.set_fetch_fn_for_attn_metadata(lambda: cur["md"])
+
+    def call(n):
+        wl = wls[n]
+        att.k_cache, att.v_cache = wl.k_cache, wl.v_cache
+        cur["md"] = metadata_for(wl, "static")
+        t = wl.q.shape[0]
+        return att(wl.q.reshape(t, -1), wl.k_new.reshape(t, -1), wl.v_new.reshape(t, -1))
+
+    call(5)                                   # warm-up on the current stream
+    torch.cuda.synchronize()
+    graphs, outs = {}, {}
+    for n in sizes:
+        graphs[n] = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graphs[n]):
+            outs[n] = call(n)
+    for n in reversed(sizes):
+        graphs[n].replay()
+        torch.cuda.synchronize()
+        got = outs[n].clone()
+        want = call(n)
+        torch.cuda.synchronize()
+        assert torch.equal(got, want), f"batch {n}"
+        assert max_abs_err(got.view(-1, 28, 128), oracle_fp32(wls[n])) <= ATOL_BF16
+
+
 @pytest.mark.parametrize("flags", PATHS)
 @pytest.mark.parametrize("name,over", [
     ("c1", {}),

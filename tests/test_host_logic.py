@@ -89,7 +89,8 @@ def test_argument_errors_do_not_launch():
     assert lib.dfx_paged_attn_workspace_bytes(C.byref(p)) == -1       # 30 % 4 != 0
     p.num_q_heads, p.max_workgroups, p.max_seqlen_q = 28, 8, 32
     need = lib.dfx_paged_attn_workspace_bytes(C.byref(p))
-    assert need == 65536 * 4 + 2 * 8 * 256 * (2 * 4 * 4 * 4 + 4) * 4   # counters + slots, NB = 2 (224 rows), hd 128
+    # counters + two slots per workgroup of 8 query blocks (224 rows) of 8 fp16 chunks + statistics, hd 128
+    assert need == _lib.DFX_WORKSPACE_COUNTER_BYTES + 2 * 8 * 8 * (8 + 1) * 64 * 16
     assert lib.dfx_paged_attn(C.byref(p), None) == -1                  # null tensors
 
 

@@ -16,11 +16,13 @@ DFX_KV_BF16, DFX_KV_FP8_E4M3 = 0, 1
 DFX_MASK_FULL, DFX_MASK_BLOCK_CAUSAL = 0, 1
 DFX_INDEX_I32, DFX_INDEX_I64 = 0, 1
 DFX_ATTN_GENERIC_PATH = 1
+DFX_ERR_SCRATCH_LIMIT = -5
+DFX_STATIC_SCRATCH_BYTES = 40 << 20
 DFX_WORKSPACE_COUNTER_BYTES = 1 << 18
 
 EXPORTS = (
     "dfx_abi_version", "dfx_status_string", "dfx_kv_store_unified", "dfx_kv_store_distinct",
-    "dfx_kv_load", "dfx_paged_attn_workspace_bytes", "dfx_paged_attn", "dfx_rope_kv_store",
+    "dfx_kv_load", "dfx_paged_attn_workspace_bytes", "dfx_paged_attn", "dfx_paged_attn_static", "dfx_rope_kv_store",
 )
 
 
@@ -95,6 +97,8 @@ def load() -> C.CDLL:
     lib.dfx_paged_attn_workspace_bytes.argtypes = [C.POINTER(AttnParams)]
     lib.dfx_paged_attn.restype = i32
     lib.dfx_paged_attn.argtypes = [C.POINTER(AttnParams), vp]
+    lib.dfx_paged_attn_static.restype = i32
+    lib.dfx_paged_attn_static.argtypes = [C.POINTER(AttnParams), vp]
     lib.dfx_rope_kv_store.restype = i32
     lib.dfx_rope_kv_store.argtypes = [C.POINTER(RopeParams), vp]
     if lib.dfx_abi_version() != DFX_ABI_VERSION:

@@ -10,6 +10,7 @@ extern "C" const char* dfx_status_string(int status) {
         case DFX_ERR_UNSUPPORTED: return "unsupported shape";
         case DFX_ERR_WORKSPACE: return "workspace missing or too small";
         case DFX_ERR_LAUNCH: return "HIP launch failed";
+        case DFX_ERR_SCRATCH_LIMIT: return "shape exceeds the static scratch limit";
         default: return "unknown status";
     }
 }

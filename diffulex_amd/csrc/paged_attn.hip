@@ -8,9 +8,17 @@
 // core (attn_tile.h): the streaming path (attn_stream.h: direct-to-LDS loads in a 4-stage
 // ring; page sizes that are multiples of 16; bf16 KV, or FP8-E4M3 KV with head_dim 128) and
 // the generic path (attn_generic.h: any page size, any layout of the fresh K/V).
+#include <mutex>
+
 #include "attn_common.h"
 #include "attn_generic.h"
 #include "attn_stream.h"
+
+// Scratch of dfx_paged_attn_static: the arrival counters and partial-result slots that
+// dfx_paged_attn takes from its caller, for callers that cannot allocate device memory.  Every
+// GPU the library runs on holds its own copy until the process ends.  The name is a host-side
+// stand-in for the symbol; its device address comes from hipGetSymbolAddress (static_scratch()).
+static __device__ __align__(256) unsigned char scratch[DFX_STATIC_SCRATCH_BYTES];
 
 namespace dfx {
 namespace {
@@ -259,6 +267,67 @@ int run_paged_attn(const dfx_attn_params* p, void* workspace, int64_t workspace_
 }
 
 }  // namespace
+
+namespace {
+
+__global__ void zero_words_kernel(int* p, int n) {
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x) p[i] = 0;
+}
+
+struct StaticScratch {
+    void* ptr = nullptr;   // device address of this device's copy of `scratch`
+    bool zeroed = false;   // an executed (not merely captured) launch has cleared the counters
+};
+
+// Address of the current device's scratch array, looked up once per device.
+int static_scratch(StaticScratch*& out) {
+    constexpr int kMaxDevices = 64;
+    static StaticScratch table[kMaxDevices];
+    static std::mutex mu;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return DFX_ERR_LAUNCH;
+    std::lock_guard<std::mutex> lock(mu);
+    if (table[dev].ptr == nullptr) {
+        void* ptr = nullptr;
+        if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || ptr == nullptr) return DFX_ERR_LAUNCH;
+        table[dev].ptr = ptr;
+    }
+    out = &table[dev];
+    return DFX_OK;
+}
+
+}  // namespace
+
+extern "C" int dfx_paged_attn_static(const dfx_attn_params* p, dfx_stream_t stream) {
+    Plan plan;
+    bool empty;
+    const int rc = check_args(p, plan, empty);
+    if (rc != DFX_OK || empty) return rc;
+    if (plan_workspace_bytes(plan) > static_cast<int64_t>(DFX_STATIC_SCRATCH_BYTES)) return DFX_ERR_SCRATCH_LIMIT;
+    StaticScratch* sc = nullptr;
+    const int rs = static_scratch(sc);
+    if (rs != DFX_OK) return rs;
+    // The arrival counters must be zero when a launch starts; every launch leaves them zero.  The
+    // first launch on a device clears them with a fill kernel (never a memset: this call may be
+    // recorded into a graph).  A launch that is only captured has not run, so captures keep
+    // recording the fill until an eager launch has executed it.
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(st, &cap) != hipSuccess) return DFX_ERR_LAUNCH;
+    bool fill;
+    {
+        static std::mutex mu;
+        std::lock_guard<std::mutex> lock(mu);
+        fill = !sc->zeroed;
+        if (fill && cap == hipStreamCaptureStatusNone) sc->zeroed = true;
+    }
+    if (fill) {
+        const int n = static_cast<int>(counter_bytes(plan) / 4);
+        hipLaunchKernelGGL(zero_words_kernel, dim3(64), dim3(256), 0, st, static_cast<int*>(sc->ptr), n);
+        if (hipGetLastError() != hipSuccess) return DFX_ERR_LAUNCH;
+    }
+    return run_paged_attn(p, sc->ptr, static_cast<int64_t>(DFX_STATIC_SCRATCH_BYTES), stream);
+}
 
 extern "C" int dfx_paged_attn(const dfx_attn_params* p, dfx_stream_t stream) {
     if (p == nullptr) return DFX_ERR_INVALID_ARG;

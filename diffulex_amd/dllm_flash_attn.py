@@ -58,13 +58,15 @@ def _workspace(device: torch.device, stream: int, nbytes: int) -> torch.Tensor:
 def paged_attention(q, k, v, k_cache, v_cache, scale, *, block_tables, context_lens, cu_seqlens_q,
                     cu_seqlens_new, max_seqlen_q, mask_mode=_lib.DFX_MASK_FULL, diffusion_block_size=32,
                     k_scale=None, v_scale=None, max_workgroups=0, out=None, flags=0,
-                    store_slot_mapping=None) -> torch.Tensor:
+                    store_slot_mapping=None, static_scratch=False) -> torch.Tensor:
     """Marshal tensors into ``dfx_attn_params`` and launch ``dfx_paged_attn`` on the
     current stream.  q: [T, H_q, hd]; k, v: [T_new, H_kv, hd]; caches
     [pages, page, H_kv, hd] or None.  ``store_slot_mapping`` ([T_new] int32/int64): the same
     launch also writes the fresh rows into those cache slots (what
     ``store_kvcache_unified_layout`` does in a launch of its own); the slots must lie outside
-    every attended context."""
+    every attended context.  ``static_scratch``: launch through ``dfx_paged_attn_static``, which
+    keeps its scratch in a static device array of the library instead of a workspace tensor (the C
+    call then allocates nothing; pass ``out`` to keep this wrapper from allocating either)."""
     lib = _lib.load()
     assert q.is_cuda and q.dtype == torch.bfloat16 and k.dtype == torch.bfloat16 and v.dtype == torch.bfloat16
     assert q.dim() == 3 and k.dim() == 3 and v.shape == k.shape
@@ -119,6 +121,9 @@ def paged_attention(q, k, v, k_cache, v_cache, scale, *, block_tables, context_l
         p.store_slot_mapping = store_slot_mapping.data_ptr()
         p.store_slot_index_type = _index_type(store_slot_mapping)
     stream = _stream()
+    if static_scratch:
+        _lib.check(lib.dfx_paged_attn_static(C.byref(p), stream), "dfx_paged_attn_static")
+        return out
     need = lib.dfx_paged_attn_workspace_bytes(C.byref(p))
     if need < 0:
         _lib.check(int(need), "dfx_paged_attn_workspace_bytes")

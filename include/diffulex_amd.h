@@ -28,7 +28,8 @@ typedef enum dfx_status {
     DFX_ERR_INVALID_ARG = -1, /* null pointer, negative size, misaligned pointer or stride */
     DFX_ERR_UNSUPPORTED = -2, /* a shape this build has no kernel for (see each function) */
     DFX_ERR_WORKSPACE = -3,   /* workspace missing or smaller than dfx_paged_attn_workspace_bytes */
-    DFX_ERR_LAUNCH = -4       /* the HIP runtime refused the launch */
+    DFX_ERR_LAUNCH = -4,      /* the HIP runtime refused the launch */
+    DFX_ERR_SCRATCH_LIMIT = -5 /* dfx_paged_attn_static: the shape needs more than DFX_STATIC_SCRATCH_BYTES */
 } dfx_status;
 
 typedef enum dfx_kv_dtype {
@@ -192,6 +193,23 @@ typedef struct dfx_attn_params {
 int64_t dfx_paged_attn_workspace_bytes(const dfx_attn_params* params);
 
 int dfx_paged_attn(const dfx_attn_params* params, dfx_stream_t stream);
+
+/*
+ * dfx_paged_attn without a caller-provided workspace, for callers that cannot allocate device
+ * memory (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).
+ * No counterpart in the reference.
+ *
+ * Same arguments, results and kernels as dfx_paged_attn; params->workspace and
+ * params->workspace_bytes are ignored.  The arrival counters and partial-result slots live in a
+ * static device array of DFX_STATIC_SCRATCH_BYTES inside the library, one copy per GPU, held
+ * until the process ends.  The call allocates and frees nothing.  Shapes for which
+ * dfx_paged_attn_workspace_bytes() exceeds DFX_STATIC_SCRATCH_BYTES are refused with
+ * DFX_ERR_SCRATCH_LIMIT (lower max_workgroups, or use dfx_paged_attn).  All calls on one GPU
+ * share that GPU's array: calls that overlap in time on one GPU (two streams, two threads)
+ * race, as calls of dfx_paged_attn that share a workspace do.
+ */
+#define DFX_STATIC_SCRATCH_BYTES (40u << 20)
+int dfx_paged_attn_static(const dfx_attn_params* params, dfx_stream_t stream);
 
 /*
  * Rotary position embedding of the fresh Q and K rows, optionally fused with the

@@ -92,6 +92,17 @@ def test_argument_errors_do_not_launch():
     # counters + two slots per workgroup of 8 query blocks (224 rows) of 8 fp16 chunks + statistics, hd 128
     assert need == _lib.DFX_WORKSPACE_COUNTER_BYTES + 2 * 8 * 8 * (8 + 1) * 64 * 16
     assert lib.dfx_paged_attn(C.byref(p), None) == -1                  # null tensors
+    assert lib.dfx_paged_attn_static(C.byref(p), None) == -1           # the same checks, nothing launched
+    assert lib.dfx_paged_attn_static(None, None) == -1
+    p.max_workgroups = 4096                                            # 302 MB of slots: beyond the static array
+    assert lib.dfx_paged_attn_workspace_bytes(C.byref(p)) > _lib.DFX_STATIC_SCRATCH_BYTES
+    # (made-up, aligned addresses: the refusal comes before anything touches the device)
+    p.q = p.k_new = p.v_new = p.out = p.cu_seqlens_q = p.cu_seqlens_new = 4096
+    p.q_stride_token, p.q_stride_head, p.o_stride_token, p.o_stride_head = 3584, 128, 3584, 128
+    p.kn_stride_token = p.vn_stride_token = 512
+    p.kn_stride_head = p.vn_stride_head = 128
+    p.scale, p.diffusion_block_size = 0.5, 32
+    assert lib.dfx_paged_attn_static(C.byref(p), None) == _lib.DFX_ERR_SCRATCH_LIMIT
 
 
 def test_device_quantiser_source_matches_oracle_on_host():

@@ -16,6 +16,7 @@ DFX_KV_BF16, DFX_KV_FP8_E4M3 = 0, 1
 DFX_MASK_FULL, DFX_MASK_BLOCK_CAUSAL = 0, 1
 DFX_INDEX_I32, DFX_INDEX_I64 = 0, 1
 DFX_ATTN_GENERIC_PATH = 1
+DFX_ATTN_NO_PIPELINE = 2
 DFX_ERR_SCRATCH_LIMIT = -5
 DFX_STATIC_SCRATCH_BYTES = 40 << 20
 DFX_WORKSPACE_COUNTER_BYTES = 1 << 18

@@ -45,7 +45,17 @@ def _compile(src: Path, obj: Path) -> None:
         sys.stderr.write(err + "\n")
 
 
+def _generate() -> None:
+    """Run the source generators under csrc/ (the hand-scheduled tile step of the streaming kernel)."""
+    import importlib.util
+    spec = importlib.util.spec_from_file_location("gen_pipe_step", CSRC / "gen_pipe_step.py")
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    mod.main()
+
+
 def build(verbose: bool = True) -> Path:
+    _generate()
     obj_dir = PKG_DIR / "build"
     obj_dir.mkdir(exist_ok=True)
     objs = [obj_dir / (Path(s).stem + ".o") for s in SOURCES]

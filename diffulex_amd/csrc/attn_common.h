@@ -11,6 +11,7 @@
 // tokens 32*tb + 16*sl + {4h..4h+3, 8+4h..8+4h+3}.
 #pragma once
 
+#include "attn_pipe_gen.h"
 #include "dfx_common.h"
 #include "fp8_e4m3.h"
 #include "partition.h"
@@ -131,9 +132,12 @@ struct TileInfo {
                      // (diffulex_kernel/python/dllm_flash_attn.py:260-261)
 };
 
-template <int HD, int NB, int NW = kWaves>
+// HIDDEN: the O^T accumulators live in the fixed registers of attn_pipe_gen.h instead of `o`
+// (pipelined kernel); the epilogues reach them one 32-row d block at a time through get_o / set_o.
+template <int HD, int NB, int NW = kWaves, bool HIDDEN = false>
 struct AttnState {
     using S = Shape<HD, NB, NW>;
+    static_assert(!HIDDEN || (HD == 128 && NB == 1), "register map of attn_pipe_gen.h");
 
     const KArgs& a;
     const int tid, lane, wave, col, half;
@@ -148,6 +152,15 @@ struct AttnState {
     DFX_D explicit AttnState(const KArgs& args)
         : a(args), tid(threadIdx.x), lane(threadIdx.x & 63), wave(threadIdx.x >> 6), col(threadIdx.x & 31),
           half((threadIdx.x >> 5) & 1) {}
+
+    DFX_D f32x16 get_o(int db, int qb) const {
+        if constexpr (HIDDEN) return pipe_get_output(db);
+        else return o[db][qb];
+    }
+    DFX_D void set_o(int db, int qb, const f32x16& v) {
+        if constexpr (HIDDEN) pipe_set_output(db, v);
+        else o[db][qb] = v;
+    }
 
     DFX_D void set_sequence(int seq, int kv_head) {
         s = seq;
@@ -179,11 +192,14 @@ struct AttnState {
         for (int qb = 0; qb < NB; ++qb) {
             m_run[qb] = -INFINITY;
             l_run[qb] = 0.0f;
+            if constexpr (!HIDDEN) {
 #pragma unroll
-            for (int db = 0; db < S::NDB; ++db)
+                for (int db = 0; db < S::NDB; ++db)
 #pragma unroll
-                for (int e = 0; e < 16; ++e) o[db][qb][e] = 0.0f;
+                    for (int e = 0; e < 16; ++e) o[db][qb][e] = 0.0f;
+            }
         }
+        if constexpr (HIDDEN) pipe_zero_outputs();
     }
 
     // Q rows of row tile rt into B-operand registers (zeros for rows past G * q_len).
@@ -304,7 +320,8 @@ struct AttnState {
             const float inv = 1.0f / l_tot[qb];
             uint16_t* op = a.out + (q0 + i) * a.o_st + (kvh * a.group + g) * a.o_sh + half * 8;
 #pragma unroll
-            for (int db = 0; db < S::NDB; ++db)
+            for (int db = 0; db < S::NDB; ++db) {
+                const f32x16 ov = get_o(db, qb);
 #pragma unroll
                 for (int pair = 0; pair < 2; ++pair) {
                     uint32_t w[2][2];  // [chunk of the pair][dword of this lane's half of it]
@@ -312,9 +329,9 @@ struct AttnState {
                     for (int c = 0; c < 2; ++c) {
                         const int ii = pair * 2 + c;
                         w[c][0] = __builtin_bit_cast(uint32_t, __builtin_convertvector(
-                            f32x2{o[db][qb][ii * 4 + 0] * inv, o[db][qb][ii * 4 + 1] * inv}, bf16x2));
+                            f32x2{ov[ii * 4 + 0] * inv, ov[ii * 4 + 1] * inv}, bf16x2));
                         w[c][1] = __builtin_bit_cast(uint32_t, __builtin_convertvector(
-                            f32x2{o[db][qb][ii * 4 + 2] * inv, o[db][qb][ii * 4 + 3] * inv}, bf16x2));
+                            f32x2{ov[ii * 4 + 2] * inv, ov[ii * 4 + 3] * inv}, bf16x2));
                     }
                     // afterwards x[0] is the lower-half dword and x[1] the upper-half dword of
                     // chunk `half` of the pair
@@ -323,6 +340,7 @@ struct AttnState {
                     const u32x4 chunk = {x0[0], x1[0], x0[1], x1[1]};
                     if (valid) *reinterpret_cast<u32x4*>(op + db * 32 + pair * 16) = chunk;
                 }
+            }
         }
     }
 
@@ -369,9 +387,11 @@ struct AttnState {
     DFX_D float row_magnitude(int qb) const {
         float mx = 0.0f;
 #pragma unroll
-        for (int db = 0; db < S::NDB; ++db)
+        for (int db = 0; db < S::NDB; ++db) {
+            const f32x16 ov = get_o(db, qb);
 #pragma unroll
-            for (int e = 0; e < 16; ++e) mx = fmaxf(mx, fabsf(o[db][qb][e]));
+            for (int e = 0; e < 16; ++e) mx = fmaxf(mx, fabsf(ov[e]));
+        }
         return wave_xor32_max(mx);
     }
 
@@ -392,11 +412,12 @@ struct AttnState {
 #pragma unroll
             for (int c = 0; c < kChunks; ++c) {
                 const int db = c >> 1, e0 = (c & 1) * 8;
+                const f32x16 ov = get_o(db, qb);
                 u32x4v w;
-                w.x = to_f16x2(o[db][qb][e0 + 0] * down, o[db][qb][e0 + 1] * down);
-                w.y = to_f16x2(o[db][qb][e0 + 2] * down, o[db][qb][e0 + 3] * down);
-                w.z = to_f16x2(o[db][qb][e0 + 4] * down, o[db][qb][e0 + 5] * down);
-                w.w = to_f16x2(o[db][qb][e0 + 6] * down, o[db][qb][e0 + 7] * down);
+                w.x = to_f16x2(ov[e0 + 0] * down, ov[e0 + 1] * down);
+                w.y = to_f16x2(ov[e0 + 2] * down, ov[e0 + 3] * down);
+                w.z = to_f16x2(ov[e0 + 4] * down, ov[e0 + 5] * down);
+                w.w = to_f16x2(ov[e0 + 6] * down, ov[e0 + 7] * down);
                 __builtin_amdgcn_raw_buffer_store_b128(w, rs, (c * 64 + lane) * 16, 0, kDeviceScope);
             }
             const f32x4 st = {m_run[qb], l_tot[qb], up, 0.0f};
@@ -416,13 +437,16 @@ struct AttnState {
             float down, up;
             row_scale(row_magnitude(qb), down, up);
 #pragma unroll
-            for (int db = 0; db < S::NDB; ++db)
+            for (int db = 0; db < S::NDB; ++db) {
+                f32x16 ov = get_o(db, qb);
 #pragma unroll
                 for (int e = 0; e < 16; e += 2) {
-                    const f32x2 v = from_f16x2(to_f16x2(o[db][qb][e] * down, o[db][qb][e + 1] * down));
-                    o[db][qb][e] = v.x * up;
-                    o[db][qb][e + 1] = v.y * up;
+                    const f32x2 v = from_f16x2(to_f16x2(ov[e] * down, ov[e + 1] * down));
+                    ov[e] = v.x * up;
+                    ov[e + 1] = v.y * up;
                 }
+                set_o(db, qb, ov);
+            }
         }
     }
 
@@ -449,19 +473,24 @@ struct AttnState {
             l_run[qb] = la + lb;
             m_run[qb] = mn;
 #pragma unroll
-            for (int c = 0; c < kChunks; ++c) {
-                const int db = c >> 1, e0 = (c & 1) * 8;
-                const u32x4v w = __builtin_amdgcn_raw_buffer_load_b128(rs, (c * 64 + lane) * 16, 0, kDeviceScope);
-                const uint32_t ws[4] = {w.x, w.y, w.z, w.w};
+            for (int db = 0; db < S::NDB; ++db) {
+                f32x16 ov = get_o(db, qb);
 #pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const f32x2 h = from_f16x2(ws[j]);
-                    const float b0 = h.x * up, b1 = h.y * up;  // exact: a power of two
-                    const float oa0 = o[db][qb][e0 + 2 * j] * wa, ob0 = b0 * wb;
-                    const float oa1 = o[db][qb][e0 + 2 * j + 1] * wa, ob1 = b1 * wb;
-                    o[db][qb][e0 + 2 * j] = oa0 + ob0;
-                    o[db][qb][e0 + 2 * j + 1] = oa1 + ob1;
+                for (int hc = 0; hc < 2; ++hc) {
+                    const int c = db * 2 + hc, e0 = hc * 8;
+                    const u32x4v w = __builtin_amdgcn_raw_buffer_load_b128(rs, (c * 64 + lane) * 16, 0, kDeviceScope);
+                    const uint32_t ws[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        const f32x2 h = from_f16x2(ws[j]);
+                        const float b0 = h.x * up, b1 = h.y * up;  // exact: a power of two
+                        const float oa0 = ov[e0 + 2 * j] * wa, ob0 = b0 * wb;
+                        const float oa1 = ov[e0 + 2 * j + 1] * wa, ob1 = b1 * wb;
+                        ov[e0 + 2 * j] = oa0 + ob0;
+                        ov[e0 + 2 * j + 1] = oa1 + ob1;
+                    }
                 }
+                set_o(db, qb, ov);
             }
         }
     }
@@ -490,8 +519,8 @@ struct AttnState {
 // ones, and no two items share such a workgroup).  Must be called by every thread of the
 // workgroup; l_tot are whole-row sums; `flag` is one int of LDS.  Returns whether this workgroup
 // wrote the rows.
-template <int HD, int NB, int NW>
-DFX_D bool finish_cut_item(AttnState<HD, NB, NW>& at, int rt, int64_t item_begin, int n_tiles, const WgSplit& split,
+template <int HD, int NB, int NW, bool HIDDEN>
+DFX_D bool finish_cut_item(AttnState<HD, NB, NW, HIDDEN>& at, int rt, int64_t item_begin, int n_tiles, const WgSplit& split,
                            int my_slot, const float (&l_tot)[NB], int* flag) {
     const KArgs& a = at.a;
     const int me = static_cast<int>(blockIdx.x);

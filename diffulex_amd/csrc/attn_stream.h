@@ -98,9 +98,9 @@ DFX_D void wait_async_loads() {
     asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
 }
 
-template <int HD, int NB, int NW, bool COMPACT = false, int KVB = 2>
-struct StreamAttn : TileMath<HD, NB, NW> {
-    using Base = TileMath<HD, NB, NW>;
+template <int HD, int NB, int NW, bool COMPACT = false, int KVB = 2, bool HIDDEN = false>
+struct StreamAttn : TileMath<HD, NB, NW, HIDDEN> {
+    using Base = TileMath<HD, NB, NW, HIDDEN>;
     using C = StreamCfg<HD, NB, NW, COMPACT, KVB>;
     using L = TileLayout<HD>;
     using Base::a;
@@ -203,6 +203,9 @@ struct StreamAttn : TileMath<HD, NB, NW> {
     // ---- loads -----------------------------------------------------------------------------
     // Start the loads of planned unit `rel` (this wave's band of K and V rows) into its ring stage.
     DFX_D void issue_unit(int rel) const {
+#ifdef DFX_ABLATE_LOADS
+        if (rel >= 4) return;
+#endif
         const BandDesc b = bands[rel * NW + wave];
         const int last = uniform(b.last);
         const bool is_ctx = uniform(b.is_ctx) != 0;
@@ -304,6 +307,36 @@ struct StreamAttn : TileMath<HD, NB, NW> {
         if (wait) touch_queries();
     }
 
+    // Pipelined kernel: adopt the item of unit d; its query rows go into the Q operand registers
+    // and O^T is cleared (attn_pipe_gen.h).  Waits for every outstanding load of the wave.
+    DFX_D void begin_item_hidden(const UnitDesc& d) {
+        static_assert(HIDDEN, "pipelined kernel only");
+        this->s = uniform(d.s);
+        this->kvh = uniform(d.kvh);
+        this->q0 = uniform(d.q0);
+        this->sh.q_len = uniform(d.q_len);
+        const int r = this->row_of(uniform(d.rt), 0);
+        const bool valid = r < a.group * this->sh.q_len;
+        const int g = valid ? r / this->sh.q_len : 0;
+        const int i = valid ? r - g * this->sh.q_len : 0;
+        this->vis_limit[0] = (i / a.dbs + 1) * a.dbs;
+        const uint16_t* qp = a.q + (this->q0 + i) * a.q_st + (this->kvh * a.group + g) * a.q_sh + half * 8;
+        pipe_load_queries(qp, __ballot(valid));
+        this->reset_accumulators();
+    }
+
+    DFX_D TileInfo tile_info_of(int rel) const {
+        const UnitDesc u = units[rel];
+        TileInfo t;
+        t.base = uniform(u.base);
+        t.limit = uniform(u.limit);
+        t.is_ctx = (uniform(u.flags) & kUnitCtx) != 0;
+        t.holes = static_cast<uint32_t>(uniform(u.flags)) >> kUnitHoleShift;  // a bit per band of rows
+        t.c_tile = a.c;
+        t.v_mul = 1.0f;
+        return t;
+    }
+
     // Close the item whose last unit of this workgroup's piece is planned unit `last_rel`.
     // Returns 0 (the run goes on in the next plan), 1 (rows written), 2 (piece stored), 3 (pieces merged).
     DFX_D int finish_run(int last_rel, const WgSplit& split) {
@@ -322,6 +355,9 @@ struct StreamAttn : TileMath<HD, NB, NW> {
 
     // Wait until at most `younger` units' loads of this wave are outstanding (younger <= 2).
     DFX_D static void wait_younger(int younger) {
+#ifdef DFX_ABLATE_LOADS
+        return;
+#endif
         if (younger >= 2) wait_async_loads<2 * C::LOADS_PER_UNIT>();
         else if (younger == 1) wait_async_loads<C::LOADS_PER_UNIT>();
         else wait_async_loads<0>();
@@ -333,26 +369,11 @@ __global__ void __launch_bounds__(64 * NW, COMPACT ? 2 : 1) paged_attn_stream_ke
     extern __shared__ __attribute__((aligned(256))) uint8_t smem[];
     using C = StreamCfg<HD, NB, NW, COMPACT>;
     StreamAttn<HD, NB, NW, COMPACT> at(a, smem);
-#ifdef DFX_TRACE
-    // Development build: thread 0 accumulates phase times (100 MHz clock) in LDS and leaves them
-    // in the unused upper part of the counter area: [0] entry, [1] prefix built, [2] first plan
-    // done, [3] ring filled and queries in, [4] exit, [5] tile loops, [6] tiles, [7..9] time of
-    // epilogues that wrote rows / stored a piece / merged, [10..12] their counts, [13] begin_item.
-    long long* tr = reinterpret_cast<long long*>(smem + C::LDS_BYTES);
-    if (threadIdx.x == 0) {
-        for (int i = 0; i < 16; ++i) tr[i] = 0;
-        tr[0] = wall_clock64();
-    }
-#define DFX_T(i) do { if (threadIdx.x == 0) tr[i] = wall_clock64(); } while (0)
-#else
-#define DFX_T(i) do {} while (0)
-#endif
     // The fused cache store comes first, while next to nothing is live in registers: anywhere
     // later its address arithmetic would push values of the tile loop out of their registers.
     store_fresh_rows<HD, false>(a);
     const UnitSummary summary = build_unit_prefix<C::RT>(a, at.prefix, at.misc);
     at.per_head = summary.per_head;
-    DFX_T(1);
     const int64_t total = static_cast<int64_t>(at.per_head) * a.h_kv;
     if (total == 0) return;
     const int w = blockIdx.x;
@@ -370,9 +391,6 @@ __global__ void __launch_bounds__(64 * NW, COMPACT ? 2 : 1) paged_attn_stream_ke
         __syncthreads();  // every wave is done with the previous plan and its stages
         at.plan_units(chunk, n_units);
         __syncthreads();
-#ifdef DFX_TRACE
-        if (chunk == begin) DFX_T(2);
-#endif
 
         // An item that opens with this plan: its query rows are requested ahead of the ring fill,
         // so that their (cold) latency runs concurrently with that of the first tiles.
@@ -381,9 +399,6 @@ __global__ void __launch_bounds__(64 * NW, COMPACT ? 2 : 1) paged_attn_stream_ke
         int issued = 0;  // ring fill: kStages - 1 units in flight
         for (; issued < C::kStages - 1 && issued < n_units; ++issued) at.issue_unit(issued);
         at.touch_queries();  // unconditional: the compiler must see no path into the tile loop with these loads pending
-#ifdef DFX_TRACE
-        if (chunk == begin) DFX_T(3);
-#endif
 
         int rel = 0;
         while (rel < n_units) {
@@ -391,19 +406,7 @@ __global__ void __launch_bounds__(64 * NW, COMPACT ? 2 : 1) paged_attn_stream_ke
             const UnitDesc d = at.units[rel];
             const int flags = uniform(d.flags);
             const int run_end = min(rel + uniform(d.run), n_units);
-#ifdef DFX_TRACE
-            long long tb = 0;
-            if (threadIdx.x == 0) tb = wall_clock64();
-#endif
             if ((flags & kUnitFirst) && rel != 0) at.begin_item(d);
-#ifdef DFX_TRACE
-            long long ts = 0;
-            if (threadIdx.x == 0) {
-                ts = wall_clock64();
-                tr[13] += ts - tb;
-                tr[6] += run_end - rel;
-            }
-#endif
             for (; rel < run_end; ++rel) {
                 // the unit must have landed: only younger units may still be outstanding
                 at.wait_younger(issued - rel - 1);
@@ -430,29 +433,9 @@ __global__ void __launch_bounds__(64 * NW, COMPACT ? 2 : 1) paged_attn_stream_ke
                     at.outputs_untouched();
                 }
             }
-#ifdef DFX_TRACE
-            long long te = 0;
-            if (threadIdx.x == 0) {
-                te = wall_clock64();
-                tr[5] += te - ts;
-            }
-            const int kind = at.finish_run(rel - 1, split);
-            if (threadIdx.x == 0 && kind > 0) {
-                tr[6 + kind] += wall_clock64() - te;
-                tr[9 + kind] += 1;
-            }
-#else
             at.finish_run(rel - 1, split);
-#endif
         }
     }
-#ifdef DFX_TRACE
-    if (threadIdx.x == 0) {
-        tr[4] = wall_clock64();
-        long long* out = reinterpret_cast<long long*>(a.arrivals + 16384) + blockIdx.x * 16;
-        for (int i = 0; i < 16; ++i) out[i] = tr[i];
-    }
-#endif
 }
 
 // FP8-E4M3 context cache (fresh K/V stay bf16).  The ring stages hold the codes as stored; in
@@ -526,6 +509,142 @@ __global__ void __launch_bounds__(64 * NW, 1) paged_attn_stream_fp8_kernel(const
                 } else {
                     at.outputs_untouched();
                 }
+            }
+            at.finish_run(rel - 1, split);
+        }
+    }
+}
+
+// The bf16 streaming kernel with the software-pipelined tile step of attn_pipe_gen.h (head_dim
+// 128, 4-stage ring).  One step of its loop computes S^T of unit r + 1 and the softmax and O^T of
+// unit r, so the ring holds the K tile of the next unit and the V tile of the current one.
+//
+// amdgpu_num_vgpr(32): the compiler allocates v0..v31 and a0..a31 only; the registers above hold
+// the matrix state of the generated blocks, which the compiler never sees.
+template <int NW>
+__global__ void __launch_bounds__(64 * NW, 1) __attribute__((amdgpu_num_vgpr(32)))
+paged_attn_pipe_kernel(const KArgs a) {
+    extern __shared__ __attribute__((aligned(256))) uint8_t smem[];
+    constexpr int HD = 128;
+    using C = StreamCfg<HD, 1, NW, false>;
+    using SA = StreamAttn<HD, 1, NW, false, 2, true>;
+    SA at(a, smem);
+    pipe_reserve();
+    store_fresh_rows<HD, false>(a);
+    const UnitSummary summary = build_unit_prefix<C::RT>(a, at.prefix, at.misc);
+    at.per_head = summary.per_head;
+    const int64_t total = static_cast<int64_t>(at.per_head) * a.h_kv;
+    if (total == 0) return;
+    const int w = blockIdx.x;
+    const int n_active = a.fixed_wg ? a.n_wg
+                                    : effective_workgroups(total, static_cast<int64_t>(summary.items) * a.h_kv,
+                                                           summary.max_tiles, a.n_wg);
+    const WgSplit split = make_wg_split(total, n_active);
+    at.begin = w < n_active ? split.first(w) : 0;
+    at.end = w < n_active ? split.first(w + 1) : 0;
+    if (at.begin >= at.end) return;
+    const int64_t begin = at.begin, end = at.end;
+    const bool busy = at.wave < a.busy_waves;  // waves whose 32 rows exist in no item of this launch only fetch
+    constexpr int kHoleRows = C::ROWS_PER_WAVE;
+    static_assert(kHoleRows == 8 || kHoleRows == 16, "mask blocks of attn_pipe_gen.h");
+
+    for (int64_t chunk = begin; chunk < end; chunk += C::kPlanUnits) {
+        const int n_units = static_cast<int>(min(static_cast<int64_t>(C::kPlanUnits), end - chunk));
+        __syncthreads();  // every wave is done with the previous plan and its stages
+        at.plan_units(chunk, n_units);
+        __syncthreads();
+
+        int issued = 0;  // ring fill: kStages - 1 units in flight
+        for (; issued < C::kStages - 1 && issued < n_units; ++issued) at.issue_unit(issued);
+
+        auto tile_of = [&](int r) { return smem + C::STAGES_OFF + (r % C::kStages) * C::STAGE_BYTES; };
+        // Unit r must have landed: only younger units may still be outstanding.  Behind the barrier
+        // every wave has finished the units before `done` (their K and their V tile), and unit x
+        // may overwrite the stage of unit x - kStages while x - kStages < done: `can_issue` says
+        // whether the wave has a unit to fetch now.
+        auto admit = [&](int r, int done) {
+            at.wait_younger(issued - r - 1);
+            __builtin_amdgcn_s_barrier();
+            return issued < n_units && issued < done + C::kStages;
+        };
+        // A tile load keeps the issuing wave standing for some 180 cycles.  The two waves of a SIMD
+        // issue theirs at different points of a step -- the lower half of the workgroup in front of
+        // it, the upper half between its two halves -- so that one of them always has matrix work.
+        const bool loads_first = at.wave < NW / 2;
+        // Mask of the score set that holds unit r, if that tile needs one; updates the lane maximum.
+        auto mask = [&](int r, bool set_a, float& mx_lane) {
+            const TileInfo t = at.tile_info_of(r);
+            const bool bc = !t.is_ctx && a.mask_mode == DFX_MASK_BLOCK_CAUSAL;
+            if (!(t.base + C::TN > t.limit || t.holes != 0 || bc)) return;
+            int lim = t.limit;
+            if (bc) lim = min(lim, at.vis_limit[0]);
+            const int thr = lim - t.base - 4 * at.half;
+            const uint32_t holes = static_cast<uint32_t>(t.holes);
+            if (set_a) {
+                if constexpr (kHoleRows == 8) pipe_mask_a_8(thr, holes, mx_lane);
+                else pipe_mask_a_16(thr, holes, mx_lane);
+            } else {
+                if constexpr (kHoleRows == 8) pipe_mask_b_8(thr, holes, mx_lane);
+                else pipe_mask_b_16(thr, holes, mx_lane);
+            }
+        };
+
+        int rel = 0;
+        while (rel < n_units) {
+            // a run of units of one item: all of this workgroup's piece of it, or up to the end of the plan
+            const UnitDesc d = at.units[rel];
+            const int run_end = min(rel + uniform(d.run), n_units);
+            if (uniform(d.flags) & kUnitFirst) at.begin_item_hidden(d);
+
+            // S^T of the run's first tile (into score set A), with nothing to overlap it with
+            if (admit(rel, rel)) at.issue_unit(issued++);
+            float mx_lane = 0.0f;  // the lane's maximum over the score set that is consumed next
+            if (busy) {
+                pipe_first_scores(at.lds_address(tile_of(rel)) + at.k_lane, mx_lane);
+                mask(rel, true, mx_lane);
+            }
+            // step r: softmax and O^T of unit r, S^T of unit r + 1; the two score sets swap roles
+            auto step = [&](int r, bool cur_is_a) {
+                const bool has_next = r + 1 < run_end;
+                const bool fetch = has_next && admit(r + 1, r);
+                if (fetch && (loads_first || !busy)) at.issue_unit(issued);
+                if (busy) {
+                    // raise the running maximum (and rescale O^T and the row sum) if this tile exceeds
+                    // it by more than the threshold
+                    const float m_tile = wave_xor32_max(mx_lane) * a.c;
+                    float& m_run = at.m_run[0];
+                    if (__any(m_tile > m_run + kRescaleThreshold)) {
+                        const float m_new = fmaxf(m_run, m_tile);
+                        const float alpha = (m_new == -INFINITY) ? 1.0f : fast_exp2(m_run - m_new);
+                        at.l_run[0] *= alpha;
+                        pipe_rescale_outputs(alpha);
+                        m_run = m_new;
+                    }
+                    const float neg_m = (m_run == -INFINITY) ? 0.0f : -m_run;
+                    const uint32_t v_cur = at.lds_address(tile_of(r) + C::MAT_BYTES) + at.v_lane;
+                    if (has_next) {
+                        const uint32_t k_next = at.lds_address(tile_of(r + 1)) + at.k_lane;
+                        if (cur_is_a) pipe_step_ab_x(k_next, v_cur, a.c, neg_m, at.l_run[0]);
+                        else pipe_step_ba_x(k_next, v_cur, a.c, neg_m, at.l_run[0]);
+                    } else {
+                        if (cur_is_a) pipe_last_a_x(v_cur, a.c, neg_m, at.l_run[0]);
+                        else pipe_last_b_x(v_cur, a.c, neg_m, at.l_run[0]);
+                    }
+                    if (fetch && !loads_first) at.issue_unit(issued);
+                    if (has_next) {
+                        if (cur_is_a) pipe_step_ab_y(a.c, neg_m, at.l_run[0], mx_lane);
+                        else pipe_step_ba_y(a.c, neg_m, at.l_run[0], mx_lane);
+                        mask(r + 1, !cur_is_a, mx_lane);
+                    } else {
+                        if (cur_is_a) pipe_last_a_y(a.c, neg_m, at.l_run[0]);
+                        else pipe_last_b_y(a.c, neg_m, at.l_run[0]);
+                    }
+                }
+                if (fetch) ++issued;
+            };
+            while (rel < run_end) {
+                step(rel++, true);
+                if (rel < run_end) step(rel++, false);
             }
             at.finish_run(rel - 1, split);
         }

@@ -88,9 +88,9 @@ DFX_D void mfma_outputs_ready(f32x16& x0, f32x16& x1) {
     asm volatile("s_nop 15\n\ts_nop 1" : "+a"(x0), "+a"(x1));
 }
 
-template <int HD, int NB, int NW>
-struct TileMath : AttnState<HD, NB, NW> {
-    using Base = AttnState<HD, NB, NW>;
+template <int HD, int NB, int NW, bool HIDDEN = false>
+struct TileMath : AttnState<HD, NB, NW, HIDDEN> {
+    using Base = AttnState<HD, NB, NW, HIDDEN>;
     using S = Shape<HD, NB, NW>;
     using L = TileLayout<HD>;
     using Base::col;
@@ -174,6 +174,10 @@ struct TileMath : AttnState<HD, NB, NW> {
 
     // Wait states before vector instructions read the O^T accumulators (rescale, epilogue).
     DFX_D void outputs_ready() {
+        if constexpr (HIDDEN) {
+            pipe_outputs_ready();
+            return;
+        }
 #pragma unroll
         for (int qb = 0; qb < NB; ++qb) {
             if constexpr (S::NDB == 4) mfma_outputs_ready(o[0][qb], o[1][qb], o[2][qb], o[3][qb]);

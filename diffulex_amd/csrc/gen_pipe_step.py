@@ -1,0 +1,434 @@
+#!/usr/bin/env python3
+"""Generates attn_pipe_gen.h: the software-pipelined tile step of the streaming paged-attention
+kernel as hand-scheduled gfx950 assembly on registers the compiler never touches.
+
+    python diffulex_amd/csrc/gen_pipe_step.py        (diffulex_amd/build.py runs it before compiling)
+
+Why.  The matrix unit and the vector ALU of a SIMD only work at the same time if one wave's
+instruction stream alternates between them: a 32x32x16 matrix instruction occupies its pipeline
+for 8 passes, in whose shadow the wave can issue four or five independent vector instructions.
+One step therefore computes S^T = K Q^T of the NEXT tile and O^T += V^T P^T of the CURRENT tile,
+with the softmax of the current tile (exp2, row sum, bf16 rounding) and the row maximum of the
+next one cut into pieces between the matrix instructions.  Left to the compiler, loop-carried
+matrix state around inline assembly is copied between registers (or spilled) at control-flow
+merges.  The kernel that uses these blocks is therefore compiled with amdgpu_num_vgpr(32): the
+compiler allocates v0..v31 and a0..a31 only, and the matrix state lives in the registers above,
+which appear in no operand list -- only in the clobber list of pipe_reserve(), so that the
+kernel's register count covers them.
+
+Register map (head_dim 128; one 32-row query block per wave; 128 + 128 registers per lane):
+    a[32:95]   O^T accumulators, 32-row d block db in a[32 + 16 db : 47 + 16 db]
+    a[96:127]  Q operand, contraction slab s in a[96 + 4 s : 99 + 4 s]
+    v[48:79]   score set A: tokens 0..31 in v[48:63], tokens 32..63 in v[64:79]
+    v[80:111]  score set B
+    v[112:127] operand ring: four 4-register buffers (K operands in phase X, V^T in phase Y)
+    v[32:42]   temporaries: exp2 pair, K operand address, 8 V^T operand addresses
+    v[0:31], a[0:31]  the compiler's
+The two score sets swap roles every step (steps AB and BA), so nothing is ever moved.  P (the
+bf16 pairs, the B operand of the second product) overwrites the current score set as it is
+consumed: pair j of the 16 (token block j / 8) goes to register j of the set, whose score
+(element j of token block 0) an earlier or the same pair has read by then.
+
+Hazards handled here by construction (the compiler does not see inside the blocks):
+  * vector-ALU result -> matrix instruction operand: 2 wait states (an s_nop 1 is emitted when the
+    producer is closer than that);
+  * transcendental result -> any reader: at least one instruction in between;
+  * matrix result -> vector-ALU reader: the readers (row maximum of the next tile) come at least
+    four matrix instructions later, or behind 18 wait states; every block that reads the O^T
+    accumulators with the vector ALU starts with those wait states;
+  * LDS operands: exact s_waitcnt lgkmcnt(n) on the in-order LDS return queue; a block starts
+    with lgkmcnt(0) so that only its own reads are in the queue.
+"""
+from __future__ import annotations
+
+import os
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ABLATE = set(filter(None, os.environ.get("DFX_PIPE_ABLATE", "").split(",")))  # development: drop instruction classes
+
+HD = 128
+ROWB = HD * 2
+NSLAB = HD // 16            # 8
+NDB = HD // 32              # 4
+COMPILER_REGS = 32          # v0..v31 and a0..a31 are the compiler's (amdgpu_num_vgpr(32))
+O_BASE, Q_BASE = 32, 96
+TMP, NTMP = 32, 11
+SA, SB, RING = 48, 80, 112
+T_EXP = [TMP + 0, TMP + 1]  # exp2 arguments / results of the pair in flight
+T_ADDR = TMP + 2            # K operand address of the slab being read (phase X); scratch elsewhere
+T_VADDR = TMP + 3           # 8 V^T operand addresses (phase Y)
+NEG_INF = "0xff800000"
+MFMA_TO_VALU = ["s_nop 15", "s_nop 1"]  # 18 wait states: the longest the ISA asks for
+
+
+def vr(base, n=1):
+    return f"v{base}" if n == 1 else f"v[{base}:{base + n - 1}]"
+
+
+def ar(base, n=1):
+    return f"a{base}" if n == 1 else f"a[{base}:{base + n - 1}]"
+
+
+def swizzle(row):
+    return ((row & 3) << 2) | ((row >> 2) & 3)
+
+
+def join(ins):
+    return "\\n\\t".join(ins)
+
+
+class Block:
+    """Instruction list with LDS queue tracking and the vector-ALU -> matrix operand hazard."""
+
+    def __init__(self):
+        self.ins = []
+        self.lds_queue = []         # tags of outstanding LDS reads, oldest first
+        self.recent_valu_defs = []  # register sets written by the last two instructions
+
+    def _push(self, text, defs=()):
+        self.ins.append(text)
+        self.recent_valu_defs = (self.recent_valu_defs + [set(defs)])[-2:]
+
+    def valu(self, text, defs):
+        if "valu" in ABLATE and ("v_exp" in text or "v_fma" in text or "v_add_f32" in text or "v_cvt" in text or "v_max" in text):
+            return
+        self._push(text, defs)
+
+    def other(self, text):
+        self._push(text)
+
+    def lds_read(self, text, tag):
+        if "lds" in ABLATE:
+            return
+        self._push(text)
+        self.lds_queue.append(tag)
+
+    def wait_lds(self, tag):
+        """Wait until the read `tag` has returned (reads return in order)."""
+        if tag not in self.lds_queue:
+            return
+        younger = len(self.lds_queue) - 1 - self.lds_queue.index(tag)
+        self._push(f"s_waitcnt lgkmcnt({younger})")
+        self.lds_queue = self.lds_queue[len(self.lds_queue) - younger:]
+
+    def mfma(self, dst, a, b, c, reads):
+        """reads: registers (numbers) of vector operands a/b/c written by the vector ALU."""
+        if "mfma" in ABLATE:
+            return
+        if any(set(reads) & d for d in self.recent_valu_defs):
+            self._push("s_nop 1")
+        self._push(f"v_mfma_f32_32x32x16_bf16 {dst}, {a}, {b}, {c}")
+
+    def text(self):
+        return join(self.ins)
+
+
+def pair_instrs(cur, pr):
+    """The 7 vector instructions of element pair pr (0..15) of score set `cur`: two exp2 arguments,
+    two exp2, two row-sum additions, one bf16 pair.  Operands: %[c] scale (SGPR), %[nm] minus the
+    running maximum, %[l] the row sum."""
+    tb, i = pr >> 3, pr & 7
+    s0, s1 = cur + 16 * tb + 2 * i, cur + 16 * tb + 2 * i + 1
+    t0, t1 = T_EXP
+    p = cur + pr
+    return [
+        (f"v_fma_f32 {vr(t0)}, {vr(s0)}, %[c], %[nm]", {t0}),
+        (f"v_fma_f32 {vr(t1)}, {vr(s1)}, %[c], %[nm]", {t1}),
+        (f"v_exp_f32 {vr(t0)}, {vr(t0)}", {t0}),
+        (f"v_exp_f32 {vr(t1)}, {vr(t1)}", {t1}),
+        (f"v_add_f32 %[l], %[l], {vr(t0)}", set()),
+        (f"v_add_f32 %[l], %[l], {vr(t1)}", set()),
+        (f"v_cvt_pk_bf16_f32 {vr(p)}, {vr(t0)}, {vr(t1)}", {p}),
+    ]
+
+
+def vaddr_instrs():
+    """V^T operand addresses vx[z] = %[v0] ^ const_z."""
+    out = []
+    for z in range(2 * NDB):
+        const = (((z >> 1) * 4) ^ swizzle((z & 1) * 8)) * 16
+        if z == 0:
+            out.append((f"v_mov_b32 {vr(T_VADDR)}, %[v0]", {T_VADDR}))
+        else:
+            out.append((f"v_xor_b32 {vr(T_VADDR + z)}, {const:#x}, %[v0]", {T_VADDR + z}))
+    return out
+
+
+def max_instrs(nxt):
+    """Maximum of the lane's 32 scores of set `nxt` into %[mx] (one lane: half a query row)."""
+    out = [(f"v_max3_f32 %[mx], {vr(nxt)}, {vr(nxt + 1)}, {vr(nxt + 2)}", set())]
+    regs = list(range(nxt + 3, nxt + 32))
+    while regs:
+        if len(regs) >= 2:
+            out.append((f"v_max3_f32 %[mx], %[mx], {vr(regs[0])}, {vr(regs[1])}", set()))
+            regs = regs[2:]
+        else:
+            out.append((f"v_max_f32 %[mx], %[mx], {vr(regs[0])}", set()))
+            regs = regs[1:]
+    return out
+
+
+def emit_valu(b, stream, n):
+    for _ in range(n):
+        if stream:
+            text, defs = stream.pop(0)
+            b.valu(text, defs)
+
+
+def phase_x(b, nxt, stream, quotas):
+    """S^T of the next tile into set `nxt`: 16 matrix instructions (slab-major, token block minor),
+    K operands read three ahead through the ring, `quotas[i]` vector instructions behind the i-th.
+    (LDS instructions take their address when they issue, in program order: the address register
+    may be rewritten for the next slab right behind the read.)"""
+    n = 2 * NSLAB
+
+    def read(i):
+        slab, tb = i >> 1, i & 1
+        if tb == 0 and slab > 0:
+            b.valu(f"v_xor_b32 {vr(T_ADDR)}, {slab * 32:#x}, %[k0]", {T_ADDR})
+        addr = "%[k0]" if slab == 0 else vr(T_ADDR)
+        b.lds_read(f"ds_read_b128 {vr(RING + 4 * (i % 4), 4)}, {addr} offset:{tb * 32 * ROWB}", ("k", i))
+
+    for i in range(3):
+        read(i)
+    for i in range(n):
+        if i + 3 < n:
+            read(i + 3)
+        b.wait_lds(("k", i))
+        slab, tb = i >> 1, i & 1
+        dst = vr(nxt + 16 * tb, 16)
+        b.mfma(dst, vr(RING + 4 * (i % 4), 4), ar(Q_BASE + 4 * slab, 4), "0" if slab == 0 else dst, reads=())
+        emit_valu(b, stream, quotas[i])
+
+
+def phase_y(b, cur, stream, quotas):
+    """O^T += V^T P^T of the current tile: 16 matrix instructions ordered (token block, 16-token
+    slab, d block), V^T operands (two transposing 8-byte reads each) two instructions ahead."""
+    n = 4 * NDB
+
+    def read(j):
+        tb, sl, db = j // (2 * NDB), (j // NDB) & 1, j % NDB
+        for ii in range(2):
+            off = (tb * 32 + sl * 16 + ii * 8) * ROWB
+            b.lds_read(f"ds_read_b64_tr_b16 {vr(RING + 4 * (j % 4) + 2 * ii, 2)}, {vr(T_VADDR + 2 * db + ii)} offset:{off}",
+                       ("v", j, ii))
+
+    read(0)
+    read(1)
+    for j in range(n):
+        if j + 2 < n:
+            read(j + 2)
+        b.wait_lds(("v", j, 1))
+        tb, sl, db = j // (2 * NDB), (j // NDB) & 1, j % NDB
+        acc = ar(O_BASE + 16 * db, 16)
+        p = cur + 8 * tb + 4 * sl
+        b.mfma(acc, vr(RING + 4 * (j % 4), 4), vr(p, 4), acc, reads=range(p, p + 4))
+        emit_valu(b, stream, quotas[j])
+
+
+def spread(total, slots):
+    """`total` instructions over `slots` matrix instructions, as evenly as integers allow."""
+    return [((i + 1) * total) // slots - (i * total) // slots for i in range(slots)]
+
+
+def step_blocks(cur, nxt, has_next):
+    """The two halves of a step.  X: S^T of the next tile with pairs 0..8 of the current set and the
+    V^T addresses in its shadow (no next tile: the vector instructions alone).  Y: O^T += V^T P^T with
+    pairs 9..13 behind its first 8 matrix instructions (pairs 8..11 feed the 9th, pairs 12..15 the
+    13th), pairs 14, 15 and the row maximum of the next set behind the rest.  The halves are separate
+    blocks so that a wave can issue its tile loads between them."""
+    pairs = [pair_instrs(cur, pr) for pr in range(16)]
+    flat = lambda ps: [ins for p in ps for ins in p]
+    sx = flat(pairs[:9]) + vaddr_instrs()
+    y1 = flat(pairs[9:14])
+    y2a = flat(pairs[14:16])
+    bx = Block()
+    bx.other("s_waitcnt lgkmcnt(0)")
+    by = Block()
+    by.other("s_waitcnt lgkmcnt(0)")
+    if has_next:
+        phase_x(bx, nxt, sx, spread(len(sx), 2 * NSLAB))
+        y2 = y2a + max_instrs(nxt)
+        qa = spread(len(y2a) + 4, 4)
+        sy = y1 + y2
+        phase_y(by, cur, sy, spread(len(y1), 8) + qa + spread(len(y2) - sum(qa), 4))
+    else:
+        emit_valu(bx, sx, len(sx))
+        sy = y1 + y2a
+        phase_y(by, cur, sy, spread(len(y1), 8) + spread(len(y2a), 4) + [0, 0, 0, 0])
+    assert not sx and not sy and not bx.lds_queue and not by.lds_queue
+    return bx.text(), by.text()
+
+
+def first_scores_block(nxt):
+    """S^T of a run's first tile into set `nxt` and its lane maximum, with nothing to overlap."""
+    b = Block()
+    b.other("s_waitcnt lgkmcnt(0)")
+    phase_x(b, nxt, [], [0] * (2 * NSLAB))
+    for t in MFMA_TO_VALU:
+        b.other(t)
+    for text, defs in max_instrs(nxt):
+        b.valu(text, defs)
+    return b.text()
+
+
+def mask_block(s, hole_rows):
+    """Masks score set `s`: element (tb, e) of the lane is token tb * 32 + (e / 4) * 8 + e % 4 of the
+    tile (plus 4 for the upper half of the wave, which %[thr] accounts for) and is set to -inf if
+    that token number is >= %[thr] or if bit (token / hole_rows) of %[holes] is set; then the lane
+    maximum of the masked set into %[mx].  The set's matrix results are ready (caller)."""
+    t, ninf = T_ADDR, T_EXP[0]
+    ins = [f"v_mov_b32 {vr(ninf)}, {NEG_INF}"]  # (a literal and vcc in one instruction exceed the constant bus)
+    for g in range(8):  # groups of 4 elements = 8 tokens
+        tb, q = g >> 2, g & 3
+        bit = (g * 8) // hole_rows
+        ins += [f"s_bitcmp1_b32 %[holes], {bit}", "s_cselect_b64 vcc, -1, 0",
+                f"v_cndmask_b32 {vr(t)}, %[thr], -1, vcc"]
+        for j in range(4):
+            reg = s + 16 * tb + 4 * q + j
+            ins += [f"v_cmp_lt_i32 vcc, {g * 8 + j}, {vr(t)}",
+                    f"v_cndmask_b32 {vr(reg)}, {vr(ninf)}, {vr(reg)}, vcc"]
+    ins += [text for text, _ in max_instrs(s)]
+    return join(ins)
+
+
+def asm_fn(name, args, body, outs=(), ins=(), clobbers=(), comment=None):
+    head = "".join(f"// {line}\n" for line in (comment or "").split("\n") if line)
+    ops = f"\n                 : {', '.join(outs)}\n                 : {', '.join(ins)}"
+    clob = ", ".join(f'"{c}"' for c in clobbers)
+    if clob:
+        ops += f"\n                 : {clob}"
+    return f'''{head}DFX_D void {name}({args}) {{
+    asm volatile("{body}"{ops});
+}}
+
+'''
+
+
+def step_fns(name, cur, nxt, has_next, comment=None):
+    x, y = step_blocks(cur, nxt, has_next)
+    fx = asm_fn(name + "_x", ("uint32_t k_next, " if has_next else "") + "float c, float neg_m, float& l_run", x,
+                ['[l] "+v"(l_run)'], (['[k0] "v"(k_next)'] if has_next else []) + ['[c] "s"(c)', '[nm] "v"(neg_m)'],
+                ["memory"], comment)
+    # (phase X has written the V^T operand addresses from v_cur: it takes it as well)
+    fx = fx.replace('[c] "s"(c)', '[v0] "v"(v_cur), [c] "s"(c)').replace("float c, float neg_m", "uint32_t v_cur, float c, float neg_m", 1)
+    fy = asm_fn(name + "_y", "float c, float neg_m, float& l_run" + (", float& mx" if has_next else ""), y,
+                ['[l] "+v"(l_run)'] + (['[mx] "=&v"(mx)'] if has_next else []), ['[c] "s"(c)', '[nm] "v"(neg_m)'], ["memory"])
+    return fx + fy
+
+
+def generate():
+    reserved = [f"v{i}" for i in range(COMPILER_REGS, 128)] + [f"a{i}" for i in range(COMPILER_REGS, 128)]
+    parts = ['''// GENERATED by gen_pipe_step.py -- do not edit.  The generator's header describes the register
+// map, the schedule and the hazards the blocks take care of themselves.
+//
+// These blocks keep their state (score sets, O^T accumulators, Q operand) in v32..v127 and
+// a32..a127 without naming those registers in any operand list.  They may only be used in a kernel
+// compiled with __attribute__((amdgpu_num_vgpr(32))), whose compiler-allocated registers end at
+// v31 / a31, and which calls pipe_reserve() once.
+#pragma once
+
+#include "dfx_common.h"
+
+namespace dfx {
+
+''']
+    parts.append(asm_fn("pipe_reserve", "", "", clobbers=reserved,
+                        comment="Makes the kernel's register count cover the registers of the blocks below (no instruction)."))
+    parts.append(asm_fn("pipe_zero_outputs", "", join(f"v_accvgpr_write_b32 {ar(O_BASE + i)}, 0" for i in range(16 * NDB)),
+                        comment="O^T = 0."))
+    # rescale: four at a time so that each read has three instructions behind it before its use
+    resc = list(MFMA_TO_VALU)
+    for g in range(0, 16 * NDB, 4):
+        resc += [f"v_accvgpr_read_b32 {vr(TMP + i - g)}, {ar(O_BASE + i)}" for i in range(g, g + 4)]
+        resc += [f"v_mul_f32 {vr(TMP + i - g)}, {vr(TMP + i - g)}, %[alpha]" for i in range(g, g + 4)]
+        resc += [f"v_accvgpr_write_b32 {ar(O_BASE + i)}, {vr(TMP + i - g)}" for i in range(g, g + 4)]
+    parts.append(asm_fn("pipe_rescale_outputs", "float alpha", join(resc), ins=['[alpha] "v"(alpha)'],
+                        comment="O^T *= alpha (per lane: one query row per lane column), behind the wait states for the matrix results."))
+    # queries: 8 x 16-byte loads of the lane's row half into score set A (dead when an item begins),
+    # zeroed for lanes without a row, then into the Q operand registers
+    ql = [f"global_load_dwordx4 {vr(SA + 4 * s, 4)}, %[p], off offset:{s * 32}" for s in range(NSLAB)]
+    ql.append("s_waitcnt vmcnt(0)")
+    ql += [f"v_cndmask_b32 {vr(SA + i)}, 0, {vr(SA + i)}, %[valid]" for i in range(4 * NSLAB)]
+    ql += [f"v_accvgpr_write_b32 {ar(Q_BASE + i)}, {vr(SA + i)}" for i in range(4 * NSLAB)]
+    parts.append(asm_fn("pipe_load_queries", "const void* row, uint64_t valid", join(ql),
+                        ins=['[p] "v"(row)', '[valid] "s"(valid)'], clobbers=["memory"],
+                        comment="Q operand: the lane's half (64 bytes of every 128: slab s at byte 32 s) of its query row at `row`,\n"
+                                "zeros for lanes whose bit in `valid` is clear (their `row` must still be readable).  Waits for\n"
+                                "every outstanding vector memory operation of the wave (vmcnt(0))."))
+    for d in range(NDB):
+        outs = [f'"=v"(x[{e}])' for e in range(16)]
+        body = join(f"v_accvgpr_read_b32 %{e}, {ar(O_BASE + 16 * d + e)}" for e in range(16))
+        parts.append(f'''DFX_D f32x16 pipe_get_output_{d}() {{
+    float x[16];
+    asm volatile("{body}"
+                 : {", ".join(outs)});
+    f32x16 v;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) v[e] = x[e];
+    return v;
+}}
+
+''')
+        ins = [f'"v"(v[{e}])' for e in range(16)]
+        body = join(f"v_accvgpr_write_b32 {ar(O_BASE + 16 * d + e)}, %{e}" for e in range(16))
+        parts.append(f'''DFX_D void pipe_set_output_{d}(const f32x16& v) {{
+    asm volatile("{body}"
+                 :
+                 : {", ".join(ins)});
+}}
+
+''')
+    parts.append('''// d block db of the O^T accumulators (db a compile-time constant after unrolling).  The caller
+// has waited for the matrix results (pipe_outputs_ready()).
+DFX_D f32x16 pipe_get_output(int db) {
+    switch (db) {
+        case 0: return pipe_get_output_0();
+        case 1: return pipe_get_output_1();
+        case 2: return pipe_get_output_2();
+        default: return pipe_get_output_3();
+    }
+}
+DFX_D void pipe_set_output(int db, const f32x16& v) {
+    switch (db) {
+        case 0: pipe_set_output_0(v); break;
+        case 1: pipe_set_output_1(v); break;
+        case 2: pipe_set_output_2(v); break;
+        default: pipe_set_output_3(v); break;
+    }
+}
+
+DFX_D void pipe_outputs_ready() { asm volatile("s_nop 15\\n\\ts_nop 1" ::: "memory"); }
+
+''')
+    parts.append(asm_fn("pipe_first_scores", "uint32_t k_next, float& mx", first_scores_block(SA),
+                        ['[mx] "=&v"(mx)'], ['[k0] "v"(k_next)'], ["memory"],
+                        "S^T of a run's first tile (LDS address k_next: tile + the lane's K operand offset) into score\nset A, and the lane's maximum."))
+    for hole_rows in (8, 16):
+        for nm, s in (("a", SA), ("b", SB)):
+            parts.append(asm_fn(f"pipe_mask_{nm}_{hole_rows}", "int thr, uint32_t holes, float& mx", mask_block(s, hole_rows),
+                                ['[mx] "=&v"(mx)'], ['[thr] "v"(thr)', '[holes] "s"(holes)'], ["vcc", "scc"],
+                                f"Mask of score set {nm.upper()} (tokens >= thr of the tile, and the {hole_rows}-token bands whose bit in `holes` is set,\n"
+                                "become -inf) and the lane's maximum of the masked set."))
+    parts.append(step_fns("pipe_step_ab", SA, SB, True,
+                          "One step, in two halves (_x then _y): softmax and O^T += V^T P^T of the current score set (A; v_cur:\n"
+                          "LDS address of the V tile + the lane's V^T operand offset), S^T of the next tile into the other set\n"
+                          "and its lane maximum."))
+    parts.append(step_fns("pipe_step_ba", SB, SA, True))
+    parts.append(step_fns("pipe_last_a", SA, SB, False, "Last step of a run: no next tile."))
+    parts.append(step_fns("pipe_last_b", SB, SA, False))
+    parts.append("}  // namespace dfx\n")
+    return "".join(parts)
+
+
+def main():
+    out = os.path.join(HERE, "attn_pipe_gen.h")
+    text = generate()
+    if not os.path.exists(out) or open(out).read() != text:
+        with open(out, "w") as f:
+            f.write(text)
+    return out
+
+
+if __name__ == "__main__":
+    print(main())

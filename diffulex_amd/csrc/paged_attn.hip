@@ -30,6 +30,7 @@ struct Plan {
     bool fp8;
     bool stream;   // streaming tile path (else generic)
     bool compact;  // streaming path, two workgroups per compute unit
+    bool pipelined;  // streaming path, bf16 KV, 4-stage ring: software-pipelined tile step
     int64_t slot_floats;
 };
 
@@ -65,6 +66,7 @@ int make_plan(const dfx_attn_params* p, Plan& plan) {
                   p->kn_stride_token == p->vn_stride_token && p->kn_stride_head == p->vn_stride_head &&
                   (!plan.fp8 || p->head_dim == 128);
     plan.compact = plan.stream && !plan.fp8 && plan.nb == 1 && p->num_seqs <= kCompactMaxSeqs;
+    plan.pipelined = plan.stream && !plan.fp8 && !plan.compact && plan.hd == 128 && !(p->flags & DFX_ATTN_NO_PIPELINE);
     if (p->max_workgroups > 0) {
         plan.n_wg = p->max_workgroups;
     } else {
@@ -107,18 +109,18 @@ int launch(const KArgs& ka, const Plan& plan, hipStream_t st) {
             lds = StreamCfg<HD, 1, 4, true>::LDS_BYTES;
         } else {
             main_k = paged_attn_stream_kernel<HD, 1, NW, false>;
+            if constexpr (HD == 128) {
+                if (plan.pipelined) main_k = paged_attn_pipe_kernel<NW>;
+            }
             lds = StreamCfg<HD, 1, NW, false>::LDS_BYTES;
-#ifdef DFX_TRACE
-            lds += 128;  // the phase timers of the development build
-#endif
         }
         threads = 64 * NW;
     } else {
         main_k = paged_attn_generic_kernel<HD, NB, PATH == 1>;
         lds = GenericCfg<HD, NB>::LDS_BYTES;
     }
-    static bool configured[2] = {false, false};  // raising the dynamic LDS limit is idempotent
-    bool& done = configured[plan.compact ? 1 : 0];
+    static bool configured[3] = {false, false, false};  // raising the dynamic LDS limit is idempotent
+    bool& done = configured[plan.compact ? 1 : (plan.pipelined ? 2 : 0)];
     if (!done) {
         if (hipFuncSetAttribute(reinterpret_cast<const void*>(main_k), hipFuncAttributeMaxDynamicSharedMemorySize,
                                 lds) != hipSuccess)

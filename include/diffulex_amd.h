@@ -46,6 +46,7 @@ typedef enum dfx_index_type { DFX_INDEX_I32 = 0, DFX_INDEX_I64 = 1 } dfx_index_t
 
 /* dfx_attn_params.flags */
 #define DFX_ATTN_GENERIC_PATH 1 /* use the generic tile path even where the streaming path applies */
+#define DFX_ATTN_NO_PIPELINE 2  /* streaming path: the plain tile loop instead of the software-pipelined one */
 
 /* ABI version of the loaded library (== DFX_ABI_VERSION it was built with). */
 int dfx_abi_version(void);

@@ -10,20 +10,22 @@ from pathlib import Path
 
 LIB_PATH = Path(__file__).resolve().parent / "libdiffulex_amd.so"
 
-DFX_ABI_VERSION = 4
+DFX_ABI_VERSION = 5
 DFX_OK = 0
 DFX_KV_BF16, DFX_KV_FP8_E4M3 = 0, 1
 DFX_MASK_FULL, DFX_MASK_BLOCK_CAUSAL = 0, 1
 DFX_INDEX_I32, DFX_INDEX_I64 = 0, 1
 DFX_ATTN_GENERIC_PATH = 1
 DFX_ATTN_NO_PIPELINE = 2
+DFX_ATTN_PAIRING = 4
 DFX_ERR_SCRATCH_LIMIT = -5
 DFX_STATIC_SCRATCH_BYTES = 40 << 20
 DFX_WORKSPACE_COUNTER_BYTES = 1 << 18
 
 EXPORTS = (
     "dfx_abi_version", "dfx_status_string", "dfx_kv_store_unified", "dfx_kv_store_distinct",
-    "dfx_kv_load", "dfx_paged_attn_workspace_bytes", "dfx_paged_attn", "dfx_paged_attn_static", "dfx_rope_kv_store",
+    "dfx_kv_load", "dfx_paged_attn_workspace_bytes", "dfx_paged_attn", "dfx_paged_attn_static", "dfx_paged_attn_plan_bytes", "dfx_paged_attn_plan", "dfx_stream_capture_id",
+    "dfx_rope_kv_store",
 )
 
 
@@ -47,6 +49,7 @@ class AttnParams(C.Structure):
         ("diffusion_block_size", C.c_int32), ("kv_dtype", C.c_int32), ("mask_mode", C.c_int32),
         ("max_workgroups", C.c_int32), ("flags", C.c_int32), ("scale", C.c_float),
         ("store_slot_mapping", C.c_void_p), ("store_slot_index_type", C.c_int32),
+        ("plan", C.c_void_p), ("plan_bytes", C.c_int64),
     ]
 
 
@@ -98,6 +101,12 @@ def load() -> C.CDLL:
     lib.dfx_paged_attn_workspace_bytes.argtypes = [C.POINTER(AttnParams)]
     lib.dfx_paged_attn.restype = i32
     lib.dfx_paged_attn.argtypes = [C.POINTER(AttnParams), vp]
+    lib.dfx_paged_attn_plan_bytes.restype = i64
+    lib.dfx_paged_attn_plan_bytes.argtypes = [C.POINTER(AttnParams), i64]
+    lib.dfx_stream_capture_id.restype = i64
+    lib.dfx_stream_capture_id.argtypes = [vp]
+    lib.dfx_paged_attn_plan.restype = i32
+    lib.dfx_paged_attn_plan.argtypes = [C.POINTER(AttnParams), vp, i64, vp]
     lib.dfx_paged_attn_static.restype = i32
     lib.dfx_paged_attn_static.argtypes = [C.POINTER(AttnParams), vp]
     lib.dfx_rope_kv_store.restype = i32

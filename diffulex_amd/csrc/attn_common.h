@@ -45,6 +45,8 @@ struct KArgs {
     int* arrivals;     // one arrival counter per workgroup, zero between launches
     const void* store_slots;  // fused KV-cache store: slot per fresh row, or null
     int store_slots_i64;
+    const uint8_t* plan;      // launch plan built by the plan kernels, or null
+    uint32_t plan_signature;  // of this launch's configuration: a plan made for another one is ignored
     int64_t q_st, q_sh, kn_st, kn_sh, vn_st, vn_sh, o_st, o_sh;
     int64_t c_sp, c_st, c_sh;  // cache strides in elements: page, token, head
     int64_t bt_stride, n_pages;
@@ -521,7 +523,7 @@ struct AttnState {
 // wrote the rows.
 template <int HD, int NB, int NW, bool HIDDEN>
 DFX_D bool finish_cut_item(AttnState<HD, NB, NW, HIDDEN>& at, int rt, int64_t item_begin, int n_tiles, const WgSplit& split,
-                           int my_slot, const float (&l_tot)[NB], int* flag) {
+                           int partner, const float (&l_tot)[NB], int* flag, int64_t piece_begin = 0) {
     const KArgs& a = at.a;
     const int me = static_cast<int>(blockIdx.x);
     const int64_t item_last = item_begin + n_tiles - 1;
@@ -530,15 +532,24 @@ DFX_D bool finish_cut_item(AttnState<HD, NB, NW, HIDDEN>& at, int rt, int64_t it
     const int64_t total = split.q * split.n_wg + split.r;
     int wa, wb;
     owners_of_units(split, me, item_begin, item_last, wa, wb);
-    const int p = sparse ? n_tiles : wb - wa + 1;
-    auto owner_of_piece = [&](int j) { return sparse ? wg_of_unit(item_last - j, total, split.n_wg) : wb - j; };
+    // Pairing partition (partner >= 0): two pieces, the item's first tiles (piece 0, processed by the
+    // partner of the item's owner at the very start of its work) and the rest (piece 1, the owner's);
+    // both are the first thing their workgroup does, hence its first partial-result slot.
+    const bool paired = partner >= 0;
+    const bool my_piece_is_first = piece_begin == item_begin;
+    const int p = paired ? 2 : (sparse ? n_tiles : wb - wa + 1);
+    auto owner_of_piece = [&](int j) {
+        if (paired) return (j == 0) == my_piece_is_first ? me : partner;
+        return sparse ? wg_of_unit(item_last - j, total, split.n_wg) : wb - j;
+    };
     auto slot_of_piece = [&](int j) {
         const int w = owner_of_piece(j);
+        if (paired) return 2 * w;
         const int64_t ws = split.first(w);
         return partial_slot(w, ws > item_begin ? ws : item_begin, ws);
     };
-    int j = sparse ? static_cast<int>(item_last - split.first(me)) : wb - me;  // the first piece of the subtree carried
-    (void)my_slot;  // == slot_of_piece(j)
+    // the first piece of the subtree carried
+    int j = paired ? (my_piece_is_first ? 0 : 1) : (sparse ? static_cast<int>(item_last - split.first(me)) : wb - me);
 #pragma unroll
     for (int qb = 0; qb < NB; ++qb) at.l_run[qb] = l_tot[qb];
 

@@ -206,7 +206,7 @@ struct GenericAttn : TileMath<HD, NB, kWaves> {
         float l_tot[NB];
         this->row_sums(l_tot);
         if (complete) this->store_output(rt, l_tot);
-        else finish_cut_item(*this, rt, item_begin, item_tiles, split, slot, l_tot, misc + kMaxWaves + 1);
+        else finish_cut_item(*this, rt, item_begin, item_tiles, split, -1, l_tot, misc + kMaxWaves + 1);
     }
 };
 

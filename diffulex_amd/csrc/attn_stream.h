@@ -32,7 +32,8 @@ namespace dfx {
 struct UnitDesc {
     int32_t s, kvh, rt, q0;
     int32_t q_len, base, limit, flags;
-    int32_t slot, run;   // run: units from this one to the end of this workgroup's piece of the item
+    int32_t partner, run;  // partner: pairing partition, the workgroup with the other piece of this item (else -1);
+                           // run: units from this one to the end of this workgroup's piece of the item
     int32_t item_rel;    // first unit of the item, relative to the workgroup's first unit
     int32_t n_tiles;     // KV tiles of the item
 };
@@ -42,6 +43,43 @@ struct BandDesc {
     int32_t last;  // last valid row of the band; later rows re-read it
     int32_t is_ctx;
 };
+// ---- the launch plan (plan.h builds it; layout of the buffer described there) ----------------------
+constexpr uint32_t kPlanMagic = 0x44465850u;  // "DFXP"
+
+struct PlanHeader {
+    uint32_t magic;      // kPlanMagic once both kernels have run; 0: unusable
+    uint32_t signature;  // of the launch configuration the plan was made for
+    int32_t n_active;    // workgroups that take part
+    int32_t mode;        // 0: equal linear ranges, 1: pairing partition
+    int32_t per_head;    // units per KV head
+    int32_t total_units;
+    int32_t capacity;    // unit descriptors the buffer has room for
+    int32_t critical;    // pairing: the critical length M (tiles), for diagnostics
+    int32_t pad[8];
+};
+static_assert(sizeof(PlanHeader) == 64, "header is one 64-byte line");
+
+struct WgWork {
+    int64_t a0, a1, b0, b1;  // linear unit ranges [a0, a1) then [b0, b1), each inside one item under pairing
+    int32_t partner;         // pairing: the workgroup holding the other piece of the shared item, or -1
+    int32_t ubase;           // index of the workgroup's first unit descriptor
+    int32_t pad[2];
+};
+static_assert(sizeof(WgWork) == 48, "three 16-byte words");
+
+struct PlanLayout {
+    int64_t prefix_off, work_off, units_off, bands_off, bytes;
+};
+DFX_HD PlanLayout plan_layout(int num_seqs, int n_wg, int64_t capacity, int waves) {
+    PlanLayout l;
+    l.prefix_off = sizeof(PlanHeader);
+    l.work_off = (l.prefix_off + (static_cast<int64_t>(num_seqs) + 1) * 4 + 63) / 64 * 64;
+    l.units_off = (l.work_off + static_cast<int64_t>(n_wg) * sizeof(WgWork) + 63) / 64 * 64;
+    l.bands_off = l.units_off + capacity * static_cast<int64_t>(sizeof(UnitDesc));
+    l.bytes = l.bands_off + capacity * waves * static_cast<int64_t>(sizeof(BandDesc));
+    return l;
+}
+
 enum : int32_t { kUnitCtx = 1, kUnitFirst = 2, kUnitLast = 4, kUnitComplete = 8, kUnitHoleShift = 8 };
 
 // COMPACT: a configuration small enough (2 stages, short plan, at most kCompactMaxSeqs sequences)
@@ -119,6 +157,7 @@ struct StreamAttn : TileMath<HD, NB, NW, HIDDEN> {
     BandDesc* bands;
     uint32_t stages_lds;  // LDS byte address of stage 0
     int64_t begin, end;
+    int64_t rel_base;  // what UnitDesc::item_rel is relative to: the first unit of the workgroup's work
     int per_head;
     float k_mul, v_mul;  // the current item's FP8 scales
 
@@ -132,7 +171,11 @@ struct StreamAttn : TileMath<HD, NB, NW, HIDDEN> {
     // ---- planning --------------------------------------------------------------------------
     // Describe units [first, first + count) in the plan table (entry i is unit first + i); one
     // lane per (unit, wave).
-    DFX_D void plan_units(int64_t first, int count) const {
+    // [begin, end) is the range of the linear unit space the workgroup is working on (all of its
+    // units, or one of its two ranges under the pairing partition, whose `partner` then holds the
+    // other piece of a cut item).
+    DFX_D void plan_units(int64_t first, int count, int partner = -1, int seg = 0) const {
+        (void)seg;
         for (int idx = tid; idx < count * NW; idx += C::THREADS) {
             const int64_t pos = first + idx / NW;
             const int w = idx % NW;
@@ -169,9 +212,9 @@ struct StreamAttn : TileMath<HD, NB, NW, HIDDEN> {
                 d.flags = (is_ctx ? kUnitCtx : 0) | (tile == tile0 ? kUnitFirst : 0) |
                           (tile == tile1 - 1 ? kUnitLast : 0) |
                           (tile0 == 0 && tile1 == item_tiles ? kUnitComplete : 0);
-                d.slot = partial_slot(static_cast<int>(blockIdx.x), pos - (tile - tile0), begin);
+                d.partner = partner;
                 d.run = tile1 - tile;
-                d.item_rel = static_cast<int>(pos - tile - begin);
+                d.item_rel = static_cast<int>(pos - tile - rel_base);
                 d.n_tiles = item_tiles;
                 units[slot_in_ring] = d;
             }
@@ -349,8 +392,81 @@ struct StreamAttn : TileMath<HD, NB, NW, HIDDEN> {
             this->store_output(uniform(e.rt), l_tot);
             return 1;
         }
-        return finish_cut_item(*this, uniform(e.rt), begin + uniform(e.item_rel), uniform(e.n_tiles), split,
-                               uniform(e.slot), l_tot, misc + kMaxWaves + 1) ? 3 : 2;
+        return finish_cut_item(*this, uniform(e.rt), rel_base + uniform(e.item_rel), uniform(e.n_tiles), split,
+                               uniform(e.partner), l_tot, misc + kMaxWaves + 1, rel_base) ? 3 : 2;
+    }
+
+    // ---- the workgroup's work -----------------------------------------------------------------
+    // Calls body(n_units) for every chunk of the workgroup's units, with the chunk's descriptors in
+    // the LDS tables and begin / end set to the range of the unit space the chunk belongs to.  The
+    // descriptors come from the plan buffer if the launch has a valid one; otherwise the workgroup
+    // works out its equal share of the unit space and its descriptors itself.
+    WgSplit split;
+    template <typename Body>
+    DFX_D void for_each_chunk(Body&& body) {
+        const PlanHeader* hdr = reinterpret_cast<const PlanHeader*>(a.plan);
+        const bool planned = hdr != nullptr && uniform(static_cast<int>(hdr->magic)) == static_cast<int>(kPlanMagic) &&
+                             uniform(static_cast<int>(hdr->signature)) == static_cast<int>(a.plan_signature);
+        WgWork w;
+        w.a0 = w.a1 = w.b0 = w.b1 = 0;
+        w.partner = -1;
+        w.ubase = 0;
+        int64_t total;
+        int n_active;
+        const UnitDesc* g_units = nullptr;
+        const BandDesc* g_bands = nullptr;
+        if (planned) {
+            per_head = uniform(hdr->per_head);
+            total = uniform(hdr->total_units);
+            n_active = uniform(hdr->n_active);
+            if (total == 0) return;
+            const PlanLayout lay = plan_layout(a.num_seqs, a.n_wg, uniform(hdr->capacity), NW);
+            const WgWork* gw = reinterpret_cast<const WgWork*>(a.plan + lay.work_off) + blockIdx.x;
+            w.a0 = gw->a0;
+            w.a1 = gw->a1;
+            w.b0 = gw->b0;
+            w.b1 = gw->b1;
+            w.partner = gw->partner;
+            w.ubase = gw->ubase;
+            g_units = reinterpret_cast<const UnitDesc*>(a.plan + lay.units_off);
+            g_bands = reinterpret_cast<const BandDesc*>(a.plan + lay.bands_off);
+        } else {
+            const UnitSummary summary = build_unit_prefix<C::RT>(a, prefix, misc);
+            per_head = summary.per_head;
+            total = static_cast<int64_t>(per_head) * a.h_kv;
+            if (total == 0) return;
+            n_active = a.fixed_wg ? a.n_wg
+                                  : effective_workgroups(total, static_cast<int64_t>(summary.items) * a.h_kv,
+                                                         summary.max_tiles, a.n_wg);
+        }
+        split = make_wg_split(total, n_active);
+        if (!planned && static_cast<int>(blockIdx.x) < n_active) {
+            w.a0 = split.first(blockIdx.x);
+            w.a1 = split.first(blockIdx.x + 1);
+        }
+        rel_base = w.a0;
+        // With a plan the descriptors of both ranges follow each other in its unit list: one list here
+        // too, so that tiles of the second range are already on their way while the first is finished.
+        const int64_t n_total = (w.a1 - w.a0) + (planned ? w.b1 - w.b0 : 0);
+        begin = w.a0;
+        end = planned ? w.a0 + n_total : w.a1;  // (with a plan only the length matters from here on)
+        for (int64_t done = 0; done < n_total; done += C::kPlanUnits) {
+            const int n_units = static_cast<int>(min(static_cast<int64_t>(C::kPlanUnits), n_total - done));
+            __syncthreads();  // every wave is done with the previous descriptors and their stages
+            if (planned) {
+                // descriptors are multiples of 16 bytes: copied as such
+                const u32x4* su = reinterpret_cast<const u32x4*>(g_units + w.ubase + done);
+                u32x4* du = reinterpret_cast<u32x4*>(units);
+                for (int i = tid; i < n_units * 3; i += C::THREADS) du[i] = su[i];
+                const u32x4* sb = reinterpret_cast<const u32x4*>(g_bands + (w.ubase + done) * NW);
+                u32x4* db = reinterpret_cast<u32x4*>(bands);
+                for (int i = tid; i < n_units * NW; i += C::THREADS) db[i] = sb[i];
+            } else {
+                plan_units(begin + done, n_units);
+            }
+            __syncthreads();
+            body(n_units);
+        }
     }
 
     // Wait until at most `younger` units' loads of this wave are outstanding (younger <= 2).
@@ -372,26 +488,8 @@ __global__ void __launch_bounds__(64 * NW, COMPACT ? 2 : 1) paged_attn_stream_ke
     // The fused cache store comes first, while next to nothing is live in registers: anywhere
     // later its address arithmetic would push values of the tile loop out of their registers.
     store_fresh_rows<HD, false>(a);
-    const UnitSummary summary = build_unit_prefix<C::RT>(a, at.prefix, at.misc);
-    at.per_head = summary.per_head;
-    const int64_t total = static_cast<int64_t>(at.per_head) * a.h_kv;
-    if (total == 0) return;
-    const int w = blockIdx.x;
-    const int n_active = a.fixed_wg ? a.n_wg
-                                    : effective_workgroups(total, static_cast<int64_t>(summary.items) * a.h_kv,
-                                                           summary.max_tiles, a.n_wg);
-    const WgSplit split = make_wg_split(total, n_active);
-    at.begin = w < n_active ? split.first(w) : 0;
-    at.end = w < n_active ? split.first(w + 1) : 0;
-    if (at.begin >= at.end) return;
-    const int64_t begin = at.begin, end = at.end;
-
-    for (int64_t chunk = begin; chunk < end; chunk += C::kPlanUnits) {
-        const int n_units = static_cast<int>(min(static_cast<int64_t>(C::kPlanUnits), end - chunk));
-        __syncthreads();  // every wave is done with the previous plan and its stages
-        at.plan_units(chunk, n_units);
-        __syncthreads();
-
+    at.for_each_chunk([&](int n_units) {
+        const WgSplit& split = at.split;
         // An item that opens with this plan: its query rows are requested ahead of the ring fill,
         // so that their (cold) latency runs concurrently with that of the first tiles.
         const bool opens = (uniform(at.units[0].flags) & kUnitFirst) != 0;
@@ -435,7 +533,7 @@ __global__ void __launch_bounds__(64 * NW, COMPACT ? 2 : 1) paged_attn_stream_ke
             }
             at.finish_run(rel - 1, split);
         }
-    }
+    });
 }
 
 // FP8-E4M3 context cache (fresh K/V stay bf16).  The ring stages hold the codes as stored; in
@@ -449,26 +547,8 @@ __global__ void __launch_bounds__(64 * NW, 1) paged_attn_stream_fp8_kernel(const
     using C = StreamCfg<HD, 1, NW, false, 1>;
     StreamAttn<HD, 1, NW, false, 1> at(a, smem);
     store_fresh_rows<HD, true>(a);  // first, as in the bf16 kernel
-    const UnitSummary summary = build_unit_prefix<C::RT>(a, at.prefix, at.misc);
-    at.per_head = summary.per_head;
-    const int64_t total = static_cast<int64_t>(at.per_head) * a.h_kv;
-    if (total == 0) return;
-    const int w = blockIdx.x;
-    const int n_active = a.fixed_wg ? a.n_wg
-                                    : effective_workgroups(total, static_cast<int64_t>(summary.items) * a.h_kv,
-                                                           summary.max_tiles, a.n_wg);
-    const WgSplit split = make_wg_split(total, n_active);
-    at.begin = w < n_active ? split.first(w) : 0;
-    at.end = w < n_active ? split.first(w + 1) : 0;
-    if (at.begin >= at.end) return;
-    const int64_t begin = at.begin, end = at.end;
-
-    for (int64_t chunk = begin; chunk < end; chunk += C::kPlanUnits) {
-        const int n_units = static_cast<int>(min(static_cast<int64_t>(C::kPlanUnits), end - chunk));
-        __syncthreads();  // every wave is done with the previous plan, its stages and bf16 tiles
-        at.plan_units(chunk, n_units);
-        __syncthreads();
-
+    at.for_each_chunk([&](int n_units) {
+        const WgSplit& split = at.split;
         const bool opens = (uniform(at.units[0].flags) & kUnitFirst) != 0;
         if (opens) at.begin_item(at.units[0], false);  // query rows ahead of the ring fill, as in the bf16 kernel
         int issued = 0;
@@ -512,7 +592,7 @@ __global__ void __launch_bounds__(64 * NW, 1) paged_attn_stream_fp8_kernel(const
             }
             at.finish_run(rel - 1, split);
         }
-    }
+    });
 }
 
 // The bf16 streaming kernel with the software-pipelined tile step of attn_pipe_gen.h (head_dim
@@ -531,29 +611,11 @@ paged_attn_pipe_kernel(const KArgs a) {
     SA at(a, smem);
     pipe_reserve();
     store_fresh_rows<HD, false>(a);
-    const UnitSummary summary = build_unit_prefix<C::RT>(a, at.prefix, at.misc);
-    at.per_head = summary.per_head;
-    const int64_t total = static_cast<int64_t>(at.per_head) * a.h_kv;
-    if (total == 0) return;
-    const int w = blockIdx.x;
-    const int n_active = a.fixed_wg ? a.n_wg
-                                    : effective_workgroups(total, static_cast<int64_t>(summary.items) * a.h_kv,
-                                                           summary.max_tiles, a.n_wg);
-    const WgSplit split = make_wg_split(total, n_active);
-    at.begin = w < n_active ? split.first(w) : 0;
-    at.end = w < n_active ? split.first(w + 1) : 0;
-    if (at.begin >= at.end) return;
-    const int64_t begin = at.begin, end = at.end;
     const bool busy = at.wave < a.busy_waves;  // waves whose 32 rows exist in no item of this launch only fetch
     constexpr int kHoleRows = C::ROWS_PER_WAVE;
     static_assert(kHoleRows == 8 || kHoleRows == 16, "mask blocks of attn_pipe_gen.h");
-
-    for (int64_t chunk = begin; chunk < end; chunk += C::kPlanUnits) {
-        const int n_units = static_cast<int>(min(static_cast<int64_t>(C::kPlanUnits), end - chunk));
-        __syncthreads();  // every wave is done with the previous plan and its stages
-        at.plan_units(chunk, n_units);
-        __syncthreads();
-
+    at.for_each_chunk([&](int n_units) {
+        const WgSplit& split = at.split;
         int issued = 0;  // ring fill: kStages - 1 units in flight
         for (; issued < C::kStages - 1 && issued < n_units; ++issued) at.issue_unit(issued);
 
@@ -567,10 +629,12 @@ paged_attn_pipe_kernel(const KArgs a) {
             __builtin_amdgcn_s_barrier();
             return issued < n_units && issued < done + C::kStages;
         };
-        // A tile load keeps the issuing wave standing for some 180 cycles.  The two waves of a SIMD
-        // issue theirs at different points of a step -- the lower half of the workgroup in front of
-        // it, the upper half between its two halves -- so that one of them always has matrix work.
-        const bool loads_first = at.wave < NW / 2;
+        // The two waves of a SIMD run half a step apart.  Everything that is not matrix work -- the
+        // issue of the tile loads (which keeps a wave standing for hundreds of cycles while memory
+        // is busy), the plan entries, the decision about the running maximum -- is done by the lower
+        // half of the workgroup behind its matrix work, at the end of a step, and by the upper half
+        // in front of it: while one wave of a SIMD does that, the other has the matrix unit.
+        const bool compute_first = at.wave < NW / 2;
         // Mask of the score set that holds unit r, if that tile needs one; updates the lane maximum.
         auto mask = [&](int r, bool set_a, float& mx_lane) {
             const TileInfo t = at.tile_info_of(r);
@@ -599,45 +663,58 @@ paged_attn_pipe_kernel(const KArgs a) {
             // S^T of the run's first tile (into score set A), with nothing to overlap it with
             if (admit(rel, rel)) at.issue_unit(issued++);
             float mx_lane = 0.0f;  // the lane's maximum over the score set that is consumed next
+            float neg_m = 0.0f;    // minus the running maximum the exponentials of the next step refer to
+            // Raise the running maximum (and rescale O^T and the row sum) if the tile about to be
+            // consumed exceeds it by more than the threshold.
+            auto prepare = [&] {
+                const float m_tile = wave_xor32_max(mx_lane) * a.c;
+                float& m_run = at.m_run[0];
+                if (__any(m_tile > m_run + kRescaleThreshold)) {
+                    const float m_new = fmaxf(m_run, m_tile);
+                    const float alpha = (m_new == -INFINITY) ? 1.0f : fast_exp2(m_run - m_new);
+                    at.l_run[0] *= alpha;
+                    pipe_rescale_outputs(alpha);
+                    m_run = m_new;
+                }
+                neg_m = (m_run == -INFINITY) ? 0.0f : -m_run;
+            };
             if (busy) {
                 pipe_first_scores(at.lds_address(tile_of(rel)) + at.k_lane, mx_lane);
                 mask(rel, true, mx_lane);
+                if (compute_first) prepare();
             }
             // step r: softmax and O^T of unit r, S^T of unit r + 1; the two score sets swap roles
             auto step = [&](int r, bool cur_is_a) {
                 const bool has_next = r + 1 < run_end;
                 const bool fetch = has_next && admit(r + 1, r);
-                if (fetch && (loads_first || !busy)) at.issue_unit(issued);
+                if (!compute_first || !busy) {
+                    if (fetch) at.issue_unit(issued);
+                    if (busy) prepare();
+                }
                 if (busy) {
-                    // raise the running maximum (and rescale O^T and the row sum) if this tile exceeds
-                    // it by more than the threshold
-                    const float m_tile = wave_xor32_max(mx_lane) * a.c;
-                    float& m_run = at.m_run[0];
-                    if (__any(m_tile > m_run + kRescaleThreshold)) {
-                        const float m_new = fmaxf(m_run, m_tile);
-                        const float alpha = (m_new == -INFINITY) ? 1.0f : fast_exp2(m_run - m_new);
-                        at.l_run[0] *= alpha;
-                        pipe_rescale_outputs(alpha);
-                        m_run = m_new;
-                    }
-                    const float neg_m = (m_run == -INFINITY) ? 0.0f : -m_run;
                     const uint32_t v_cur = at.lds_address(tile_of(r) + C::MAT_BYTES) + at.v_lane;
                     if (has_next) {
                         const uint32_t k_next = at.lds_address(tile_of(r + 1)) + at.k_lane;
-                        if (cur_is_a) pipe_step_ab_x(k_next, v_cur, a.c, neg_m, at.l_run[0]);
-                        else pipe_step_ba_x(k_next, v_cur, a.c, neg_m, at.l_run[0]);
-                    } else {
-                        if (cur_is_a) pipe_last_a_x(v_cur, a.c, neg_m, at.l_run[0]);
-                        else pipe_last_b_x(v_cur, a.c, neg_m, at.l_run[0]);
-                    }
-                    if (fetch && !loads_first) at.issue_unit(issued);
-                    if (has_next) {
-                        if (cur_is_a) pipe_step_ab_y(a.c, neg_m, at.l_run[0], mx_lane);
-                        else pipe_step_ba_y(a.c, neg_m, at.l_run[0], mx_lane);
+                        if (cur_is_a) {
+                            pipe_step_ab_x(k_next, v_cur, a.c, neg_m, at.l_run[0]);
+                            pipe_step_ab_y(a.c, neg_m, at.l_run[0], mx_lane);
+                        } else {
+                            pipe_step_ba_x(k_next, v_cur, a.c, neg_m, at.l_run[0]);
+                            pipe_step_ba_y(a.c, neg_m, at.l_run[0], mx_lane);
+                        }
                         mask(r + 1, !cur_is_a, mx_lane);
                     } else {
-                        if (cur_is_a) pipe_last_a_y(a.c, neg_m, at.l_run[0]);
-                        else pipe_last_b_y(a.c, neg_m, at.l_run[0]);
+                        if (cur_is_a) {
+                            pipe_last_a_x(v_cur, a.c, neg_m, at.l_run[0]);
+                            pipe_last_a_y(a.c, neg_m, at.l_run[0]);
+                        } else {
+                            pipe_last_b_x(v_cur, a.c, neg_m, at.l_run[0]);
+                            pipe_last_b_y(a.c, neg_m, at.l_run[0]);
+                        }
+                    }
+                    if (compute_first) {
+                        if (fetch) at.issue_unit(issued);
+                        if (has_next) prepare();
                     }
                 }
                 if (fetch) ++issued;
@@ -648,7 +725,7 @@ paged_attn_pipe_kernel(const KArgs a) {
             }
             at.finish_run(rel - 1, split);
         }
-    }
+    });
 }
 
 }  // namespace dfx

@@ -8,11 +8,13 @@
 // core (attn_tile.h): the streaming path (attn_stream.h: direct-to-LDS loads in a 4-stage
 // ring; page sizes that are multiples of 16; bf16 KV, or FP8-E4M3 KV with head_dim 128) and
 // the generic path (attn_generic.h: any page size, any layout of the fresh K/V).
+#include <atomic>
 #include <mutex>
 
 #include "attn_common.h"
 #include "attn_generic.h"
 #include "attn_stream.h"
+#include "plan.h"
 
 // Scratch of dfx_paged_attn_static: the arrival counters and partial-result slots that
 // dfx_paged_attn takes from its caller, for callers that cannot allocate device memory.  Every
@@ -66,7 +68,10 @@ int make_plan(const dfx_attn_params* p, Plan& plan) {
                   p->kn_stride_token == p->vn_stride_token && p->kn_stride_head == p->vn_stride_head &&
                   (!plan.fp8 || p->head_dim == 128);
     plan.compact = plan.stream && !plan.fp8 && plan.nb == 1 && p->num_seqs <= kCompactMaxSeqs;
-    plan.pipelined = plan.stream && !plan.fp8 && !plan.compact && plan.hd == 128 && !(p->flags & DFX_ATTN_NO_PIPELINE);
+    // (8 waves only: with 4 waves a wave has twice the tile loads to address, and the 32 registers
+    // the pipelined kernel leaves the compiler no longer hold that without spilling in the loop)
+    plan.pipelined = plan.stream && !plan.fp8 && !plan.compact && plan.hd == 128 && plan.nb == 2 &&
+                     !(p->flags & DFX_ATTN_NO_PIPELINE);
     if (p->max_workgroups > 0) {
         plan.n_wg = p->max_workgroups;
     } else {
@@ -90,43 +95,78 @@ int64_t plan_workspace_bytes(const Plan& plan) {
     return counter_bytes(plan) + 2 * static_cast<int64_t>(plan.n_wg) * plan.slot_floats * 4;
 }
 
-// PATH: 0 generic bf16, 1 generic FP8, 2 streaming bf16, 3 streaming FP8
+// Raising a kernel's dynamic LDS limit is idempotent but not free: done once per device and kernel.
+bool ensure_lds_limit(const void* kernel, int slot, int lds) {
+    static std::atomic<uint32_t> configured[64];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return false;
+    const uint32_t bit = 1u << slot;
+    if (configured[dev].load(std::memory_order_acquire) & bit) return true;
+    if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess) return false;
+    configured[dev].fetch_or(bit, std::memory_order_release);
+    return true;
+}
+
+// PATH: 0 generic bf16, 1 generic FP8, 2 streaming bf16, 3 streaming FP8.
+// pa == nullptr: the attention launch.  Otherwise the two plan kernels for that launch (streaming
+// paths only).
 template <int HD, int NB, int PATH>
-int launch(const KArgs& ka, const Plan& plan, hipStream_t st) {
+int launch(const KArgs& ka, const Plan& plan, hipStream_t st, const PlanArgs* pa) {
     void (*main_k)(const KArgs);
-    int lds, threads = kThreads;
+    void (*plan_k)(const KArgs, const PlanArgs) = nullptr;
+    void (*fill_k)(const KArgs, const PlanArgs) = nullptr;
+    int lds, threads = kThreads, fill_lds = 0, slot;
+    constexpr int NW = 4 * NB;  // streaming paths: one 32-row query block per wave
+    constexpr int kSlotBase = (HD == 128 ? 0 : 8) + (NB == 1 ? 0 : 4);
     if constexpr (PATH == 3) {
-        constexpr int NW = 4 * NB;
         main_k = paged_attn_stream_fp8_kernel<HD, NW>;
-        lds = StreamCfg<HD, 1, NW, false, 1>::LDS_BYTES;
+        using C = StreamCfg<HD, 1, NW, false, 1>;
+        lds = C::LDS_BYTES;
+        plan_k = paged_attn_plan_kernel<C::RT>;
+        fill_k = paged_attn_plan_fill_kernel<HD, 1, NW, false, 1>;
+        fill_lds = C::STAGES_OFF;
         threads = 64 * NW;
+        slot = kSlotBase + 3;
     } else if constexpr (PATH == 2) {
-        // the streaming path gives every wave one 32-row query block: 4 waves for up to 128 rows,
-        // 8 waves (two per SIMD, so one wave's softmax overlaps the other's matrix work) for 256
-        constexpr int NW = 4 * NB;
+        // 4 waves for up to 128 rows (then two workgroups per compute unit where the batch allows),
+        // 8 waves (two per SIMD) for up to 256
         if (NB == 1 && plan.compact) {
+            using C = StreamCfg<HD, 1, 4, true>;
             main_k = paged_attn_stream_kernel<HD, 1, 4, true>;
-            lds = StreamCfg<HD, 1, 4, true>::LDS_BYTES;
+            lds = C::LDS_BYTES;
+            plan_k = paged_attn_plan_kernel<C::RT>;
+            fill_k = paged_attn_plan_fill_kernel<HD, 1, 4, true, 2>;
+            fill_lds = C::STAGES_OFF;
+            slot = kSlotBase + 1;
         } else {
+            using C = StreamCfg<HD, 1, NW, false>;
             main_k = paged_attn_stream_kernel<HD, 1, NW, false>;
-            if constexpr (HD == 128) {
-                if (plan.pipelined) main_k = paged_attn_pipe_kernel<NW>;
+            slot = kSlotBase + 0;
+            if constexpr (HD == 128 && NW == 8) {
+                if (plan.pipelined) {
+                    main_k = paged_attn_pipe_kernel<NW>;
+                    slot = kSlotBase + 2;
+                }
             }
-            lds = StreamCfg<HD, 1, NW, false>::LDS_BYTES;
+            lds = C::LDS_BYTES;
+            plan_k = paged_attn_plan_kernel<C::RT>;
+            fill_k = paged_attn_plan_fill_kernel<HD, 1, NW, false, 2>;
+            fill_lds = C::STAGES_OFF;
         }
         threads = 64 * NW;
     } else {
         main_k = paged_attn_generic_kernel<HD, NB, PATH == 1>;
         lds = GenericCfg<HD, NB>::LDS_BYTES;
+        slot = 16 + kSlotBase / 4 * 2 + PATH;
     }
-    static bool configured[3] = {false, false, false};  // raising the dynamic LDS limit is idempotent
-    bool& done = configured[plan.compact ? 1 : (plan.pipelined ? 2 : 0)];
-    if (!done) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void*>(main_k), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                lds) != hipSuccess)
-            return DFX_ERR_LAUNCH;
-        done = true;
+    if (pa != nullptr) {
+        if (plan_k == nullptr) return DFX_ERR_UNSUPPORTED;
+        constexpr int kPlanLds = (2 * (kMaxSeqs + 1) + 2 * kMaxPairItems + 64) * 4;
+        hipLaunchKernelGGL(plan_k, dim3(1), dim3(512), kPlanLds, st, ka, *pa);
+        hipLaunchKernelGGL(fill_k, dim3(plan.n_wg), dim3(threads), fill_lds, st, ka, *pa);
+        return hipGetLastError() == hipSuccess ? DFX_OK : DFX_ERR_LAUNCH;
     }
+    if (!ensure_lds_limit(reinterpret_cast<const void*>(main_k), slot, lds)) return DFX_ERR_LAUNCH;
     hipLaunchKernelGGL(main_k, dim3(plan.n_wg), dim3(threads), lds, st, ka);
     if (hipGetLastError() != hipSuccess) return DFX_ERR_LAUNCH;
     return DFX_OK;
@@ -189,16 +229,57 @@ int check_args(const dfx_attn_params* p, Plan& plan, bool& empty) {
 }
 
 // Checks and launch; `workspace` replaces p->workspace.
-int run_paged_attn(const dfx_attn_params* p, void* workspace, int64_t workspace_bytes, dfx_stream_t stream) {
+// The launch configuration a plan depends on (everything but the tensors' base pointers, the
+// scale and the store): a plan made for another configuration is ignored by the kernels.
+uint32_t plan_signature(const dfx_attn_params* p, const Plan& plan) {
+    uint64_t h = 1469598103934665603ull;
+    auto mix = [&](uint64_t v) {
+        for (int i = 0; i < 8; ++i) {
+            h ^= (v >> (8 * i)) & 0xffu;
+            h *= 1099511628211ull;
+        }
+    };
+    mix(plan.hd); mix(plan.nb); mix(plan.n_wg); mix(plan.fp8); mix(plan.stream); mix(plan.compact);
+    mix(p->num_seqs); mix(p->num_q_heads); mix(p->num_kv_heads); mix(p->page_size); mix(p->max_pages_per_seq);
+    mix(p->max_seqlen_q); mix(p->diffusion_block_size); mix(p->mask_mode); mix(p->max_workgroups);
+    mix(p->kn_stride_token); mix(p->kn_stride_head); mix(p->cache_stride_page); mix(p->cache_stride_token);
+    mix(p->cache_stride_head); mix(p->block_table_stride); mix(p->n_pages); mix(p->k_cache != nullptr);
+    mix(reinterpret_cast<uintptr_t>(p->block_tables)); mix(reinterpret_cast<uintptr_t>(p->context_lens));
+    mix(reinterpret_cast<uintptr_t>(p->cu_seqlens_q)); mix(reinterpret_cast<uintptr_t>(p->cu_seqlens_new));
+    const uint32_t sig = static_cast<uint32_t>(h ^ (h >> 32));
+    return sig == 0 ? 1u : sig;
+}
+
+int plan_waves(const Plan& plan) { return plan.compact ? 4 : 4 * plan.nb; }
+
+// Checks and launch; `workspace` replaces p->workspace.  plan_out != nullptr: instead of the
+// attention launch, build its plan into plan_out (plan_bytes of room).
+int run_paged_attn(const dfx_attn_params* p, void* workspace, int64_t workspace_bytes, dfx_stream_t stream,
+                   void* plan_out = nullptr, int64_t plan_bytes = 0) {
     Plan plan;
     bool empty;
     const int rc = check_args(p, plan, empty);
     if (rc != DFX_OK || empty) return rc;
     const bool has_cache = p->k_cache != nullptr;
     const int64_t need = plan_workspace_bytes(plan);
-    if (plan.n_wg > 1 && (workspace == nullptr || workspace_bytes < need ||
-                          (reinterpret_cast<uintptr_t>(workspace) & 255u) != 0))
+    if (plan_out == nullptr && plan.n_wg > 1 &&
+        (workspace == nullptr || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 255u) != 0))
         return DFX_ERR_WORKSPACE;
+    PlanArgs pa;
+    if (plan_out != nullptr) {
+        if (!plan.stream) return DFX_ERR_UNSUPPORTED;
+        if ((reinterpret_cast<uintptr_t>(plan_out) & 255u) != 0) return DFX_ERR_INVALID_ARG;
+        const PlanLayout fixed = plan_layout(p->num_seqs, plan.n_wg, 0, plan_waves(plan));
+        const int64_t per_unit = static_cast<int64_t>(sizeof(UnitDesc)) + plan_waves(plan) * static_cast<int64_t>(sizeof(BandDesc));
+        if (plan_bytes < fixed.bytes) return DFX_ERR_WORKSPACE;
+        pa.buf = static_cast<uint8_t*>(plan_out);
+        pa.capacity = (plan_bytes - fixed.bytes) / per_unit;
+        if (pa.capacity > 0x7fffffff) pa.capacity = 0x7fffffff;
+        pa.n_wg = plan.n_wg;
+        pa.waves = plan_waves(plan);
+        pa.signature = plan_signature(p, plan);
+        pa.allow_pairing = (p->flags & DFX_ATTN_PAIRING) ? 1 : 0;
+    }
 
     KArgs ka;
     ka.q = static_cast<const uint16_t*>(p->q);
@@ -249,16 +330,24 @@ int run_paged_attn(const dfx_attn_params* p, void* workspace, int64_t workspace_
         ka.busy_waves = static_cast<int>(rows >= 32 * kMaxWaves ? kMaxWaves : (rows + 31) / 32);
     }
     ka.c = p->scale * kLog2e;
+    ka.plan = nullptr;
+    ka.plan_signature = plan_signature(p, plan);
+    if (plan_out == nullptr && plan.stream && p->plan != nullptr) {
+        const PlanLayout fixed = plan_layout(p->num_seqs, plan.n_wg, 0, plan_waves(plan));
+        if (p->plan_bytes < fixed.bytes || (reinterpret_cast<uintptr_t>(p->plan) & 255u) != 0) return DFX_ERR_INVALID_ARG;
+        ka.plan = static_cast<const uint8_t*>(p->plan);
+    }
 
     hipStream_t st = static_cast<hipStream_t>(stream);
+    const PlanArgs* pap = plan_out != nullptr ? &pa : nullptr;
 #define DFX_ATTN_CASE(HD_, NB_)                                               \
     if (plan.hd == HD_ && plan.nb == NB_) {                                   \
         if (plan.stream && plan.fp8) {                                        \
-            if constexpr (HD_ == 128) return launch<HD_, NB_, 3>(ka, plan, st); \
+            if constexpr (HD_ == 128) return launch<HD_, NB_, 3>(ka, plan, st, pap); \
         }                                                                     \
-        if (plan.stream) return launch<HD_, NB_, 2>(ka, plan, st);       \
-        if (plan.fp8) return launch<HD_, NB_, 1>(ka, plan, st);          \
-        return launch<HD_, NB_, 0>(ka, plan, st);                        \
+        if (plan.stream) return launch<HD_, NB_, 2>(ka, plan, st, pap);       \
+        if (plan.fp8) return launch<HD_, NB_, 1>(ka, plan, st, pap);          \
+        return launch<HD_, NB_, 0>(ka, plan, st, pap);                        \
     }
     DFX_ATTN_CASE(64, 1)
     DFX_ATTN_CASE(64, 2)
@@ -329,6 +418,27 @@ extern "C" int dfx_paged_attn_static(const dfx_attn_params* p, dfx_stream_t stre
         if (hipGetLastError() != hipSuccess) return DFX_ERR_LAUNCH;
     }
     return run_paged_attn(p, sc->ptr, static_cast<int64_t>(DFX_STATIC_SCRATCH_BYTES), stream);
+}
+
+extern "C" int64_t dfx_stream_capture_id(dfx_stream_t stream) {
+    hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+    unsigned long long id = 0;
+    if (hipStreamGetCaptureInfo(static_cast<hipStream_t>(stream), &status, &id) != hipSuccess) return -1;
+    return status == hipStreamCaptureStatusActive ? static_cast<int64_t>(id) + 1 : 0;
+}
+
+extern "C" int64_t dfx_paged_attn_plan_bytes(const dfx_attn_params* p, int64_t max_units) {
+    Plan plan;
+    const int rc = make_plan(p, plan);
+    if (rc != DFX_OK) return rc;
+    if (!plan.stream) return DFX_ERR_UNSUPPORTED;
+    if (max_units < 0) return DFX_ERR_INVALID_ARG;
+    return plan_layout(p->num_seqs, plan.n_wg, max_units, plan_waves(plan)).bytes;
+}
+
+extern "C" int dfx_paged_attn_plan(const dfx_attn_params* p, void* plan_buf, int64_t plan_bytes, dfx_stream_t stream) {
+    if (p == nullptr || plan_buf == nullptr) return DFX_ERR_INVALID_ARG;
+    return run_paged_attn(p, nullptr, 0, stream, plan_buf, plan_bytes);
 }
 
 extern "C" int dfx_paged_attn(const dfx_attn_params* p, dfx_stream_t stream) {

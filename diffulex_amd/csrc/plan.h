@@ -1,0 +1,291 @@
+// The launch plan of the streaming paged-attention kernels, built once per decoding step and read
+// by the attention launch of every layer (the lengths, block tables and strides are the same for
+// all of them; only the q / k / v / cache base pointers change).
+//
+// Layout of the plan buffer:
+//   PlanHeader                                  64 bytes
+//   int32 prefix[num_seqs + 1]                  exclusive prefix of the sequences' units (per KV head)
+//   WgWork work[n_wg]                           what every workgroup does (partition.h: linear ranges
+//                                               of the unit space, or the pairing partition)
+//   UnitDesc units[capacity]                    one per unit, in each workgroup's processing order
+//   BandDesc bands[capacity * NW]               one per unit and wave
+// Two kernels fill it: paged_attn_plan_kernel (one workgroup: prefix, partition) and
+// paged_attn_plan_fill_kernel (one workgroup per attention workgroup: the descriptors).  A plan
+// whose header does not carry the magic number, or whose unit capacity was too small for the
+// batch, is ignored by the attention kernels, which then plan for themselves.
+#pragma once
+
+#include "attn_stream.h"
+
+namespace dfx {
+
+struct PlanArgs {
+    uint8_t* buf;
+    int64_t capacity;   // unit descriptors
+    int n_wg;           // workgroups of the attention launch
+    int waves;          // waves per attention workgroup
+    uint32_t signature;
+    int allow_pairing;
+};
+
+// Linear position of item y (0 <= y < items of the sequence) inside the sequence's units, and its tiles.
+DFX_HD void item_of_sequence(const SeqShape& sh, int rt, int& offset, int& tiles) {
+    tiles = tiles_of_row_tile(sh, rt);
+    if (sh.rph == 0) {
+        offset = rt * sh.n_tiles;
+    } else {
+        const int g = rt / sh.rph, k = rt - g * sh.rph;
+        offset = g * units_before_row_tile(sh, sh.rph) + units_before_row_tile(sh, k);
+    }
+}
+
+// Descending bitonic sort of n (a power of two) keys in LDS by all threads of the workgroup.
+DFX_D void bitonic_sort_desc(uint32_t* keys, int n) {
+    for (int k = 2; k <= n; k <<= 1)
+        for (int j = k >> 1; j > 0; j >>= 1) {
+            for (int i = threadIdx.x; i < n; i += blockDim.x) {
+                const int ixj = i ^ j;
+                if (ixj > i) {
+                    const uint32_t x = keys[i], y = keys[ixj];
+                    const bool up = (i & k) == 0;  // this pair sorts descending
+                    if (up ? x < y : x > y) {
+                        keys[i] = y;
+                        keys[ixj] = x;
+                    }
+                }
+            }
+            __syncthreads();
+        }
+}
+
+// Phase one, one workgroup of 512 threads: the unit prefix, the partition and every workgroup's work.
+template <int RT>
+__global__ void __launch_bounds__(512) paged_attn_plan_kernel(const KArgs a, const PlanArgs pa) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    int* prefix = reinterpret_cast<int*>(smem);                         // [kMaxSeqs + 1]
+    int* iprefix = prefix + kMaxSeqs + 1;                               // [kMaxSeqs + 1] items before a sequence
+    uint32_t* keys = reinterpret_cast<uint32_t*>(iprefix + kMaxSeqs + 1);  // [kMaxPairItems]
+    int* ubase = reinterpret_cast<int*>(keys + kMaxPairItems);          // [kMaxPairItems]
+    int* misc = ubase + kMaxPairItems;                                  // [64]
+    PlanHeader* hdr = reinterpret_cast<PlanHeader*>(pa.buf);
+    const PlanLayout lay = plan_layout(a.num_seqs, pa.n_wg, pa.capacity, pa.waves);
+    int* g_prefix = reinterpret_cast<int*>(pa.buf + lay.prefix_off);
+    WgWork* work = reinterpret_cast<WgWork*>(pa.buf + lay.work_off);
+    const int tid = threadIdx.x;
+
+    const UnitSummary summary = build_unit_prefix<RT>(a, prefix, misc);
+    const int per_head = summary.per_head;
+    const int64_t total = static_cast<int64_t>(per_head) * a.h_kv;
+    const int64_t n_items = static_cast<int64_t>(summary.items) * a.h_kv;
+    const int n_active = total == 0 ? 0
+                         : a.fixed_wg ? a.n_wg
+                                      : effective_workgroups(total, n_items, summary.max_tiles, a.n_wg);
+    for (int s = tid; s <= a.num_seqs; s += blockDim.x) g_prefix[s] = prefix[s];
+
+    // items before each sequence (row tiles of sequences that have units)
+    {
+        int carry = 0;
+        for (int base = 0; base < a.num_seqs; base += blockDim.x) {
+            const int sq = base + tid;
+            int r = 0;
+            if (sq < a.num_seqs) {
+                const SeqShape shp = load_seq_shape(a, sq, RT);
+                r = shp.units > 0 ? shp.n_row_tiles : 0;
+            }
+            int tot;
+            const int incl = block_inclusive_scan(r, misc, tot);
+            if (sq < a.num_seqs) iprefix[sq + 1] = carry + incl;
+            carry += tot;
+        }
+        if (tid == 0) iprefix[0] = 0;
+        __syncthreads();
+    }
+    const int items_per_head = summary.items;
+
+    // item x (KV head minor: the heads of one (sequence, row tile) are neighbours, and stay
+    // neighbours in the sorted list, being equally long) -> its first unit and its tiles
+    auto locate_item = [&](int x, int64_t& begin, int& tiles) {
+        const int y = x / a.h_kv, kvh = x - y * a.h_kv;
+        (void)items_per_head;
+        int lo = 0, hi = a.num_seqs;  // the sequence with iprefix[s] <= y < iprefix[s + 1]
+        while (lo < hi) {
+            const int mid = (lo + hi) >> 1;
+            if (iprefix[mid + 1] <= y) lo = mid + 1;
+            else hi = mid;
+        }
+        const SeqShape shp = load_seq_shape(a, lo, RT);
+        int off;
+        item_of_sequence(shp, y - iprefix[lo], off, tiles);
+        begin = static_cast<int64_t>(kvh) * per_head + prefix[lo] + off;
+    };
+
+    // ---- pairing partition, if it applies --------------------------------------------------------
+    const int m = n_active;
+    bool pairing = pa.allow_pairing && total > 0 && n_items <= m && m <= kMaxPairItems && total >= m;
+    int critical = 0;
+    if (pairing) {  // (uniform: every thread takes the same branch)
+        int n_sort = 1;
+        while (n_sort < m) n_sort <<= 1;
+        for (int x = tid; x < n_sort; x += blockDim.x) {
+            uint32_t key = 0;  // empty entry: sorts last
+            if (x < n_items) {
+                int64_t begin;
+                int tiles;
+                locate_item(x, begin, tiles);
+                key = (static_cast<uint32_t>(tiles) << 10) | static_cast<uint32_t>(kMaxPairItems - 1 - x);
+                if (tiles >= (1 << 21)) key = 0xffffffffu;  // (cannot be keyed: forces the fallback below)
+            }
+            keys[x] = key;
+        }
+        __syncthreads();
+        bitonic_sort_desc(keys, n_sort);
+        // the launch's critical length: the worst pair (k-th longest with k-th shortest)
+        int worst = 0;
+        for (int k = tid; 2 * k < m; k += blockDim.x) {
+            const int l = static_cast<int>(keys[k] >> 10), s = static_cast<int>(keys[m - 1 - k] >> 10);
+            const int c = (2 * k == m - 1) ? l : pair_critical_length(l, s);
+            worst = max(worst, c);
+        }
+#pragma unroll
+        for (int d = 32; d >= 1; d >>= 1) worst = max(worst, __shfl_xor(worst, d));
+        if ((tid & 63) == 0) misc[32 + (tid >> 6)] = worst;
+        __syncthreads();
+        for (int w = 0; w < static_cast<int>(blockDim.x >> 6); ++w) critical = max(critical, misc[32 + w]);
+        __syncthreads();
+        const int even = static_cast<int>((total + m - 1) / m);
+        pairing = critical <= even + kPairSlack && keys[0] != 0xffffffffu;
+    }
+
+    if (pairing) {
+        // unit counts per workgroup, then their exclusive prefix
+        int carry = 0;
+        for (int base = 0; base < m; base += blockDim.x) {
+            const int k = base + tid;
+            int count = 0;
+            if (k < m) {
+                const int kp = m - 1 - k;
+                const int mine = static_cast<int>(keys[k] >> 10), other = static_cast<int>(keys[kp] >> 10);
+                if (k < kp) count = mine - pair_donation(mine, other, critical);
+                else if (k > kp) count = mine + pair_donation(other, mine, critical);
+                else count = mine;
+            }
+            int tot;
+            const int incl = block_inclusive_scan(count, misc, tot);
+            if (k < m) ubase[k] = carry + incl - count;
+            carry += tot;
+        }
+        __syncthreads();
+        // Which workgroup gets which entry of the sorted list.  The KV heads of one sequence are
+        // equally long, hence neighbours in the list, and read the same token rows of the cache at
+        // the same time: they go to workgroups whose numbers differ by a multiple of m / h_kv (of 8,
+        // the number of XCDs, at the usual sizes), i.e. onto the same XCD, behind the same L2 and TLB
+        // -- where the equal ranges of the linear unit space put them too.
+        const int heads = (a.h_kv > 0 && m % a.h_kv == 0) ? a.h_kv : 1;
+        auto workgroup_of = [&](int entry) { return (entry % heads) * (m / heads) + entry / heads; };
+        for (int k = tid; k < pa.n_wg; k += blockDim.x) {
+            WgWork w;
+            w.a0 = w.a1 = w.b0 = w.b1 = 0;
+            w.partner = -1;
+            w.ubase = 0;
+            w.pad[0] = w.pad[1] = 0;
+            if (k >= m) {
+                work[k] = w;
+                continue;
+            }
+            {
+                const int kp = m - 1 - k;
+                const int mine = static_cast<int>(keys[k] >> 10), other = static_cast<int>(keys[kp] >> 10);
+                int64_t my_begin = 0, other_begin = 0;
+                int t;
+                if (mine > 0) locate_item(kMaxPairItems - 1 - static_cast<int>(keys[k] & 1023u), my_begin, t);
+                if (other > 0) locate_item(kMaxPairItems - 1 - static_cast<int>(keys[kp] & 1023u), other_begin, t);
+                if (k < kp) {  // the long item's owner keeps its end
+                    const int d = pair_donation(mine, other, critical);
+                    w.a0 = my_begin + d;
+                    w.a1 = my_begin + mine;
+                    if (d > 0) w.partner = workgroup_of(kp);
+                } else if (k > kp) {  // the partner: donated tiles first, then its own item
+                    const int d = pair_donation(other, mine, critical);
+                    w.a0 = other_begin;
+                    w.a1 = other_begin + d;
+                    w.b0 = my_begin;
+                    w.b1 = my_begin + mine;
+                    if (d > 0) w.partner = workgroup_of(kp);
+                } else {
+                    w.a0 = my_begin;
+                    w.a1 = my_begin + mine;
+                }
+                w.ubase = ubase[k];
+            }
+            work[workgroup_of(k)] = w;
+        }
+    } else {
+        const WgSplit split = make_wg_split(total > 0 ? total : 1, n_active > 0 ? n_active : 1);
+        for (int k = tid; k < pa.n_wg; k += blockDim.x) {
+            WgWork w;
+            w.a0 = w.a1 = w.b0 = w.b1 = 0;
+            w.partner = -1;
+            w.ubase = 0;
+            w.pad[0] = w.pad[1] = 0;
+            if (k < n_active && total > 0) {
+                w.a0 = split.first(k);
+                w.a1 = split.first(k + 1);
+                w.ubase = static_cast<int32_t>(w.a0);
+            }
+            work[k] = w;
+        }
+    }
+    if (tid == 0) {
+        PlanHeader h;
+        h.magic = total <= pa.capacity ? kPlanMagic : 0u;  // too small a buffer: the kernels plan for themselves
+        h.signature = pa.signature;
+        h.n_active = n_active;
+        h.mode = pairing ? 1 : 0;
+        h.per_head = per_head;
+        h.total_units = static_cast<int32_t>(total);
+        h.capacity = static_cast<int32_t>(pa.capacity);
+        h.critical = critical;
+        for (int i = 0; i < 8; ++i) h.pad[i] = 0;
+        *hdr = h;
+    }
+}
+
+// Phase two, one workgroup per attention workgroup: the unit and band descriptors of its work.
+template <int HD, int NB, int NW, bool COMPACT, int KVB>
+__global__ void __launch_bounds__(64 * NW) paged_attn_plan_fill_kernel(const KArgs a, const PlanArgs pa) {
+    extern __shared__ __attribute__((aligned(256))) uint8_t smem[];
+    using C = StreamCfg<HD, NB, NW, COMPACT, KVB>;
+    StreamAttn<HD, NB, NW, COMPACT, KVB> at(a, smem);
+    const PlanHeader* hdr = reinterpret_cast<const PlanHeader*>(pa.buf);
+    if (hdr->magic != kPlanMagic) return;
+    const PlanLayout lay = plan_layout(a.num_seqs, pa.n_wg, pa.capacity, NW);
+    const int* g_prefix = reinterpret_cast<const int*>(pa.buf + lay.prefix_off);
+    const WgWork w = reinterpret_cast<const WgWork*>(pa.buf + lay.work_off)[blockIdx.x];
+    UnitDesc* g_units = reinterpret_cast<UnitDesc*>(pa.buf + lay.units_off);
+    BandDesc* g_bands = reinterpret_cast<BandDesc*>(pa.buf + lay.bands_off);
+    for (int s = threadIdx.x; s <= a.num_seqs; s += blockDim.x) at.prefix[s] = g_prefix[s];
+    at.per_head = hdr->per_head;
+    __syncthreads();
+    int64_t done = w.ubase;
+    at.rel_base = w.a0;
+    for (int seg = 0; seg < 2; ++seg) {
+        at.begin = seg == 0 ? w.a0 : w.b0;
+        at.end = seg == 0 ? w.a1 : w.b1;
+        for (int64_t chunk = at.begin; chunk < at.end; chunk += C::kPlanUnits) {
+            const int n = static_cast<int>(min(static_cast<int64_t>(C::kPlanUnits), at.end - chunk));
+            at.plan_units(chunk, n, seg == 0 ? w.partner : -1, seg);
+            __syncthreads();
+            // descriptors are multiples of 16 bytes: copy as such
+            const u32x4* su = reinterpret_cast<const u32x4*>(at.units);
+            u32x4* du = reinterpret_cast<u32x4*>(g_units + done);
+            for (int i = threadIdx.x; i < n * 3; i += blockDim.x) du[i] = su[i];
+            const u32x4* sb = reinterpret_cast<const u32x4*>(at.bands);
+            u32x4* db = reinterpret_cast<u32x4*>(g_bands + done * NW);
+            for (int i = threadIdx.x; i < n * NW; i += blockDim.x) db[i] = sb[i];
+            done += n;
+            __syncthreads();
+        }
+    }
+}
+
+}  // namespace dfx

@@ -58,7 +58,7 @@ def _workspace(device: torch.device, stream: int, nbytes: int) -> torch.Tensor:
 def paged_attention(q, k, v, k_cache, v_cache, scale, *, block_tables, context_lens, cu_seqlens_q,
                     cu_seqlens_new, max_seqlen_q, mask_mode=_lib.DFX_MASK_FULL, diffusion_block_size=32,
                     k_scale=None, v_scale=None, max_workgroups=0, out=None, flags=0,
-                    store_slot_mapping=None, static_scratch=False) -> torch.Tensor:
+                    store_slot_mapping=None, static_scratch=False, plan_cache=None) -> torch.Tensor:
     """Marshal tensors into ``dfx_attn_params`` and launch ``dfx_paged_attn`` on the
     current stream.  q: [T, H_q, hd]; k, v: [T_new, H_kv, hd]; caches
     [pages, page, H_kv, hd] or None.  ``store_slot_mapping`` ([T_new] int32/int64): the same
@@ -66,7 +66,12 @@ def paged_attention(q, k, v, k_cache, v_cache, scale, *, block_tables, context_l
     ``store_kvcache_unified_layout`` does in a launch of its own); the slots must lie outside
     every attended context.  ``static_scratch``: launch through ``dfx_paged_attn_static``, which
     keeps its scratch in a static device array of the library instead of a workspace tensor (the C
-    call then allocates nothing; pass ``out`` to keep this wrapper from allocating either)."""
+    call then allocates nothing; pass ``out`` to keep this wrapper from allocating either).
+    ``plan_cache`` (a dict): the launch plan (``dfx_paged_attn_plan``: partition of the batch over
+    the workgroups, page address of every tile) is built on the first call and reused by later
+    calls with the same dict -- the attention layers of one decoding step, whose lengths and block
+    tables are the same.  In-place updates of those tensors and graph captures are noticed (they
+    change the cache key); a caller that rewrites them behind PyTorch's back drops the dict."""
     lib = _lib.load()
     assert q.is_cuda and q.dtype == torch.bfloat16 and k.dtype == torch.bfloat16 and v.dtype == torch.bfloat16
     assert q.dim() == 3 and k.dim() == 3 and v.shape == k.shape
@@ -121,6 +126,20 @@ def paged_attention(q, k, v, k_cache, v_cache, scale, *, block_tables, context_l
         p.store_slot_mapping = store_slot_mapping.data_ptr()
         p.store_slot_index_type = _index_type(store_slot_mapping)
     stream = _stream()
+    if plan_cache is not None and has_cache:
+        # A plan is only as good as the lengths and tables it was made from: the key carries the
+        # tensors' version counters (any in-place update makes a new key) and the graph capture the
+        # call is recorded into (a plan built outside that capture is not part of its graph).
+        meta = (block_tables, context_lens, cu_seqlens_q, cu_seqlens_new)
+        key = (H_q, H_kv, hd, int(p.kv_dtype), int(mask_mode), int(diffusion_block_size), int(max_seqlen_q), int(flags),
+               int(max_workgroups), k.stride(0), k.stride(1), k_cache.stride()[:3], num_seqs,
+               tuple((t.data_ptr(), t._version) for t in meta), int(lib.dfx_stream_capture_id(stream)))
+        plan = plan_cache.get(key, False)
+        if plan is False:
+            plan = _build_plan(lib, p, q.device, stream, H_q // H_kv, k.shape[0])
+            plan_cache[key] = plan
+        if plan is not None:
+            p.plan, p.plan_bytes = plan.data_ptr(), plan.numel()
     if static_scratch:
         _lib.check(lib.dfx_paged_attn_static(C.byref(p), stream), "dfx_paged_attn_static")
         return out
@@ -131,6 +150,35 @@ def paged_attention(q, k, v, k_cache, v_cache, scale, *, block_tables, context_l
     p.workspace, p.workspace_bytes = ws.data_ptr(), ws.numel()
     _lib.check(lib.dfx_paged_attn(C.byref(p), stream), "dfx_paged_attn")
     return out
+
+
+def _build_plan(lib, p, device, stream, group, t_new):
+    """Launch ``dfx_paged_attn_plan`` for the configuration in ``p``; None where no plan applies
+    (generic tile path).  The unit capacity is an upper bound from the shapes alone: no device data
+    is read."""
+    row_tiles = -(-group * int(p.max_seqlen_q) // 128)
+    tiles = int(p.num_seqs) * (-(-int(p.max_pages_per_seq) * int(p.page_size) // 64) + 1) + t_new // 64
+    nbytes = lib.dfx_paged_attn_plan_bytes(C.byref(p), int(p.num_kv_heads) * row_tiles * tiles)
+    if nbytes < 0:
+        return None
+    plan = torch.empty(int(nbytes), dtype=torch.uint8, device=device)
+    _lib.check(lib.dfx_paged_attn_plan(C.byref(p), plan.data_ptr(), plan.numel(), stream), "dfx_paged_attn_plan")
+    return plan
+
+
+def _plan_cache_of(attn_metadata):
+    """The per-step plan cache, kept on the metadata object: the reference's runners build a new
+    metadata object for every step (strategy/*/attention/metadata.py setters), so the plan is
+    rebuilt exactly when lengths and block tables change.  Objects that cannot take the attribute
+    simply get no plan."""
+    cache = getattr(attn_metadata, "dfx_plan_cache", None)
+    if cache is None:
+        cache = {}
+        try:
+            attn_metadata.dfx_plan_cache = cache
+        except (AttributeError, TypeError):
+            return None
+    return cache
 
 
 def _max_seqlen_q(attn_metadata, cu_seqlens_q) -> int:
@@ -192,4 +240,5 @@ def dllm_flash_attn_decode(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, k_
         context_lens=attn_metadata.context_lens, cu_seqlens_q=attn_metadata.cu_seqlens_q,
         cu_seqlens_new=cu_new, max_seqlen_q=_max_seqlen_q(attn_metadata, attn_metadata.cu_seqlens_q),
         mask_mode=mask, diffusion_block_size=attn_metadata.diffusion_block_size,
-        k_scale=k_scale, v_scale=v_scale, store_slot_mapping=store_slot_mapping)
+        k_scale=k_scale, v_scale=v_scale, store_slot_mapping=store_slot_mapping,
+        plan_cache=_plan_cache_of(attn_metadata))

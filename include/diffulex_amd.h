@@ -19,7 +19,7 @@
 extern "C" {
 #endif
 
-#define DFX_ABI_VERSION 4
+#define DFX_ABI_VERSION 5
 
 typedef void* dfx_stream_t; /* a hipStream_t; NULL is the default stream */
 
@@ -47,6 +47,7 @@ typedef enum dfx_index_type { DFX_INDEX_I32 = 0, DFX_INDEX_I64 = 1 } dfx_index_t
 /* dfx_attn_params.flags */
 #define DFX_ATTN_GENERIC_PATH 1 /* use the generic tile path even where the streaming path applies */
 #define DFX_ATTN_NO_PIPELINE 2  /* streaming path: the plain tile loop instead of the software-pipelined one */
+#define DFX_ATTN_PAIRING 4      /* dfx_paged_attn_plan: the pairing partition where it applies (see there) */
 
 /* ABI version of the loaded library (== DFX_ABI_VERSION it was built with). */
 int dfx_abi_version(void);
@@ -182,6 +183,11 @@ typedef struct dfx_attn_params {
      * through k_cache / v_cache although the pointers are declared const. */
     const void* store_slot_mapping;
     int32_t store_slot_index_type; /* dfx_index_type */
+    /* Launch plan built by dfx_paged_attn_plan for this configuration (NULL: the kernel plans for
+     * itself, as it also does if the plan was made for another configuration or its buffer was too
+     * small for the batch). */
+    const void* plan;
+    int64_t plan_bytes;
 } dfx_attn_params;
 
 /* Bytes of scratch dfx_paged_attn needs for these shapes (depends on the sizes
@@ -194,6 +200,39 @@ typedef struct dfx_attn_params {
 int64_t dfx_paged_attn_workspace_bytes(const dfx_attn_params* params);
 
 int dfx_paged_attn(const dfx_attn_params* params, dfx_stream_t stream);
+
+/*
+ * The launch plan of dfx_paged_attn, built once per decoding step and shared by the attention
+ * launches of all layers.
+ * Replaces: nothing on the device.  The reference builds its per-step attention metadata on the
+ *           host (diffulex/strategy/d2f/engine/model_runner.py:244-261, :283-289) and every one of
+ *           its kernel launches re-derives its work from it; here the partition of the batch over
+ *           the workgroups, every tile's page address and the pieces of items shared between
+ *           workgroups are worked out once, on the device, and the launches read them.
+ *
+ * A plan depends on the lengths (context_lens, cu_seqlens_q, cu_seqlens_new), the block tables, the
+ * shapes, max_workgroups, flags and the strides of the caches and of k_new -- not on the base
+ * pointers of q, k_new, v_new, out and the caches, nor on scale: the per-layer views of one cache
+ * allocation share a plan.  It is built on `stream` with no host synchronisation (safe to record
+ * into a graph).  DFX_ATTN_PAIRING in flags asks for the pairing partition where there are at most
+ * as many (sequence, KV head, row tile) items as workgroups: every item gets a home workgroup and
+ * only the excess of long items moves, which needs a third of the partial results that equal ranges
+ * of the unit space need, at about the same speed.
+ *
+ * dfx_paged_attn_plan_bytes: bytes of plan buffer for up to max_units units (one unit = one
+ * 64-token KV tile of one KV head of one row tile of one sequence; an upper bound is
+ * num_kv_heads * row_tiles * (num_seqs * ceil(max_context / 64) + T_new / 64 + num_seqs)).  A buffer
+ * too small for the batch at hand is detected on the device and the plan ignored.  Streaming-path
+ * shapes only (page_size a multiple of 16, k_new and v_new laid out alike; FP8 with head_dim 128):
+ * DFX_ERR_UNSUPPORTED otherwise.  The buffer must be 256-byte aligned.
+ */
+int64_t dfx_paged_attn_plan_bytes(const dfx_attn_params* params, int64_t max_units);
+/* 0 if `stream` is not being captured into a graph, otherwise a positive number that identifies
+ * the capture (-1: the runtime could not tell).  For callers that cache plans: a plan built
+ * outside a capture, or inside another one, is not part of the graph being recorded and must be
+ * built again inside it.  No counterpart in the reference. */
+int64_t dfx_stream_capture_id(dfx_stream_t stream);
+int dfx_paged_attn_plan(const dfx_attn_params* params, void* plan, int64_t plan_bytes, dfx_stream_t stream);
 
 /*
  * dfx_paged_attn without a caller-provided workspace, for callers that cannot allocate device

@@ -576,3 +576,97 @@ def test_non_finite_inputs_stay_inside_their_sequence(dev, flags):
                 assert not torch.isfinite(got[rows].float()).all()
             else:
                 assert torch.equal(got[rows], clean[mw][rows])
+
+
+# ---- launch plans (dfx_paged_attn_plan) ---------------------------------------------------------------
+PLAN_CASES = [
+    ("c3", {}),                                              # 256 items on 256 workgroups: pairing applies
+    ("c3", dict(num_seqs=5, ctx=(200, 700))),                # fewer items than workgroups
+    ("c3", dict(num_seqs=9, ctx=[64, 3000, 100, 2500, 700, 650, 1, 0, 4096])),
+    ("c3", dict(num_seqs=70, ctx=(100, 900))),               # more items than workgroups: equal ranges
+    ("c4", dict(num_seqs=3, ctx=(100, 500))),                # compact kernel, block-causal
+    ("c5", dict(num_seqs=4, ctx=(200, 900))),                # FP8 streaming kernel
+    ("c1", {}),                                              # head_dim 64
+]
+
+
+def _read_plan(plan, num_seqs, n_wg):
+    """Header and per-workgroup work of a plan buffer (layout: csrc/plan.h)."""
+    raw = plan.cpu().numpy()
+    hdr = raw[:64].view(np.int32)
+    work_off = (64 + (num_seqs + 1) * 4 + 63) // 64 * 64
+    work = raw[work_off:work_off + n_wg * 48].reshape(n_wg, 48)
+    ranges = work[:, :32].copy().view(np.int64).reshape(n_wg, 4)
+    partner = work[:, 32:36].copy().view(np.int32).reshape(n_wg)
+    return dict(magic=int(hdr[0]) & 0xffffffff, n_active=int(hdr[2]), mode=int(hdr[3]), per_head=int(hdr[4]),
+                total=int(hdr[5]), critical=int(hdr[7])), ranges, partner
+
+
+@pytest.mark.parametrize("name,over", PLAN_CASES)
+@pytest.mark.parametrize("max_wg", [0, 7])
+def test_planned_launch_with_equal_ranges_gives_the_same_bits(dev, name, over, max_wg):
+    """By default the plan describes the partition the kernels work out for themselves: reading it
+    must not change a bit."""
+    wl = make_workload(name, device=dev, **over)
+    want = _run(wl, max_wg)
+    cache = {}
+    for _ in range(2):   # the second call reuses the plan
+        got = _run(wl, max_wg, plan_cache=cache)
+        assert torch.equal(got, want)
+    assert len(cache) == 1 and next(iter(cache.values())) is not None
+
+
+@pytest.mark.parametrize("name,over", PLAN_CASES)
+def test_planned_launch_with_the_pairing_partition(dev, name, over):
+    wl = make_workload(name, device=dev, **over)
+    cache = {}
+    got = _run(wl, plan_cache=cache, flags=_lib.DFX_ATTN_PAIRING)
+    tol = ATOL_FP8 if wl.kv_fp8 else ATOL_BF16
+    if wl.num_seqs <= 16:
+        assert max_abs_err(got, oracle_fp32(wl)) <= tol
+    assert max_abs_err(got, _run(wl)) <= 1e-2
+    again = _run(wl, plan_cache=cache, flags=_lib.DFX_ATTN_PAIRING)
+    assert torch.equal(again, got)
+
+
+def test_pairing_plan_covers_every_unit_once_at_c3(dev):
+    """The plan of the headline workload: pairing partition, every unit of the linear unit space in
+    exactly one workgroup's ranges, donated pieces in front of the partner's own item."""
+    wl = make_workload("c3", device=dev)
+    cache = {}
+    got = _run(wl, plan_cache=cache, flags=_lib.DFX_ATTN_PAIRING)
+    torch.cuda.synchronize()
+    n_wg = torch.cuda.get_device_properties(dev).multi_processor_count
+    hdr, ranges, partner = _read_plan(next(iter(cache.values())), wl.num_seqs, n_wg)
+    assert hdr["magic"] == 0x44465850 and hdr["mode"] == 1 and hdr["n_active"] == n_wg
+    tiles = sum((int(c) + 63) // 64 + 1 for c in wl.context_lens.tolist())
+    assert hdr["per_head"] == tiles and hdr["total"] == tiles * wl.num_kv_heads
+    spans = sorted((int(a), int(b)) for r in ranges for a, b in ((r[0], r[1]), (r[2], r[3])) if b > a)
+    assert spans[0][0] == 0 and spans[-1][1] == hdr["total"]
+    assert all(x[1] == y[0] for x, y in zip(spans, spans[1:]))
+    loads = [(r[1] - r[0]) + (r[3] - r[2]) for r in ranges]
+    assert max(loads) <= hdr["critical"] and hdr["critical"] <= -(-hdr["total"] // n_wg) + 6
+    cut = [w for w in range(n_wg) if partner[w] >= 0]
+    assert all(partner[partner[w]] == w for w in cut) and 0 < len(cut) < n_wg
+    cu = wl.cu_seqlens_q.tolist()
+    for s, want in zip([0, 63], oracle_fp32(wl, seqs=[0, 63])):
+        assert max_abs_err(got[cu[s]:cu[s + 1]], want) <= ATOL_BF16
+
+
+def test_plan_made_for_another_configuration_is_ignored(dev):
+    """A stale or foreign plan must never be followed: the kernels compare its signature with their
+    own launch and plan for themselves."""
+    wl = make_workload("c3", device=dev, num_seqs=6, ctx=(300, 900))
+    other = make_workload("c3", device=dev, num_seqs=6, ctx=(1000, 1500), seed=9)
+    cache = {}
+    _run(other, plan_cache=cache)
+    plan = next(iter(cache.values()))
+    want = _run(wl)
+    # hand the foreign plan to a launch with other metadata tensors (different signature)
+    p_cache = {}
+    out = _run(wl, plan_cache=p_cache)
+    key = next(iter(p_cache))
+    p_cache[key] = plan
+    got2 = _run(wl, plan_cache=p_cache)
+    assert max_abs_err(got2, want) <= 1e-2 and torch.equal(got2, want)
+    assert max_abs_err(out, want) <= 1e-2

@@ -76,3 +76,49 @@ def test_tile_loop_has_no_spills_and_no_compiler_waits(isa, kernel, max_waits):
         after_barrier = loop[max(i for i, l in enumerate(loop) if l.startswith("s_barrier")):]
         assert not [l for l in after_barrier if "vmcnt" in l]
     assert ops["global_load_lds_dwordx4"] in (2, 4, 8)   # a wave's share of the 64 * head_dim * elt * 2 bytes of a tile
+
+
+PIPE_KERNELS = ["_ZN3dfx22paged_attn_pipe_kernelILi8E"]
+
+
+@pytest.mark.parametrize("kernel", PIPE_KERNELS)
+def test_pipelined_kernel_leaves_the_generated_blocks_registers_alone(isa, kernel):
+    """The generated blocks of csrc/attn_pipe_gen.h keep their state in v32..v127 / a32..a127 across
+    compiler-generated code, which is only sound while the compiler allocates nothing there
+    (amdgpu_num_vgpr(32) on the kernel).  Checked on the generated code: outside the assembly
+    blocks no register above v31 / a31 is named, and the tile loop has no scratch access."""
+    m = re.search(r"^(%s\w*):" % re.escape(kernel), isa, re.M)
+    assert m, kernel
+    body = isa[m.start():isa.index("s_endpgm", m.start())].split("\n")
+    in_asm, top_v, top_a, blocks = False, 0, 0, 0
+    for line in body:
+        t = line.strip()
+        if t.startswith(";;#ASMSTART"):
+            in_asm, blocks = True, blocks + 1
+            continue
+        if t.startswith(";;#ASMEND"):
+            in_asm = False
+            continue
+        if in_asm or not t or t.startswith((";", ".")):
+            continue
+        for mm in re.finditer(r"\b([va])(\d+)\b", t):
+            if mm.group(1) == "v":
+                top_v = max(top_v, int(mm.group(2)))
+            else:
+                top_a = max(top_a, int(mm.group(2)))
+        for mm in re.finditer(r"\b([va])\[(\d+):(\d+)\]", t):
+            if mm.group(1) == "v":
+                top_v = max(top_v, int(mm.group(3)))
+            else:
+                top_a = max(top_a, int(mm.group(3)))
+    assert blocks > 20
+    assert top_v <= 31 and top_a <= 31, (top_v, top_a)
+    # the kernel's register count covers the blocks' registers
+    i = isa.index(".amdhsa_kernel " + m.group(1))
+    assert int(re.search(r"\.amdhsa_next_free_vgpr (\d+)", isa[i:i + 3000]).group(1)) == 256
+    assert int(re.search(r"\.amdhsa_accum_offset (\d+)", isa[i:i + 3000]).group(1)) == 128
+    loop = _tile_loop(isa, kernel)
+    ops = collections.Counter(l.split()[0] for l in loop)
+    # first tile of a run 16, two steps 32 each, two last steps 16 each
+    assert ops["v_mfma_f32_32x32x16_bf16"] == 112
+    assert not [l for l in loop if l.startswith("scratch_")], "a register of the tile loop lives in scratch"

@@ -45,6 +45,7 @@ struct KArgs {
     int* arrivals;     // one arrival counter per workgroup, zero between launches
     const void* store_slots;  // fused KV-cache store: slot per fresh row, or null
     int store_slots_i64;
+    int64_t n_new;            // rows of k_new / v_new (and of the slot mapping)
     const uint8_t* plan;      // launch plan built by the plan kernels, or null
     uint32_t plan_signature;  // of this launch's configuration: a plan made for another one is ignored
     int64_t q_st, q_sh, kn_st, kn_sh, vn_st, vn_sh, o_st, o_sh;
@@ -117,7 +118,9 @@ DFX_D int block_inclusive_scan(int v, int* scratch, int& block_total) {
 DFX_D SeqShape load_seq_shape(const KArgs& a, int s, int rows_per_tile) {
     const int ctx = (a.context_lens != nullptr && a.k_cache != nullptr) ? a.context_lens[s] : 0;
     const int q_len = a.cu_q[s + 1] - a.cu_q[s];
-    const int new_len = a.cu_new[s + 1] - a.cu_new[s];
+    // fresh rows are clamped to the rows k_new / v_new have (padded batches carry offsets beyond them)
+    const int64_t n0 = min(static_cast<int64_t>(a.cu_new[s]), a.n_new), n1 = min(static_cast<int64_t>(a.cu_new[s + 1]), a.n_new);
+    const int new_len = static_cast<int>(n1 - n0);
     return make_seq_shape(ctx, q_len, new_len, a.group, rows_per_tile, a.mask_mode == DFX_MASK_BLOCK_CAUSAL, a.dbs);
 }
 
@@ -319,7 +322,9 @@ struct AttnState {
             const bool valid = r < a.group * sh.q_len;
             const int g = valid ? r / sh.q_len : 0;
             const int i = valid ? r - g * sh.q_len : 0;
-            const float inv = 1.0f / l_tot[qb];
+            // a row none of whose keys is visible (every page of its context a hole, no fresh rows)
+            // has a zero sum: it gets zeros, not 0 * inf
+            const float inv = l_tot[qb] > 0.0f ? 1.0f / l_tot[qb] : 0.0f;
             uint16_t* op = a.out + (q0 + i) * a.o_st + (kvh * a.group + g) * a.o_sh + half * 8;
 #pragma unroll
             for (int db = 0; db < S::NDB; ++db) {
@@ -598,7 +603,9 @@ DFX_D void store_fresh_rows(const KArgs& a) {
     constexpr int kChunksPerHead = HD / 8;
     constexpr int kBatch = 4;  // chunks a thread has in flight: all loads of a batch are issued before its stores
     const int chunks_per_token = a.h_kv * kChunksPerHead;
-    const int64_t total = static_cast<int64_t>(a.cu_new[a.num_seqs]) * chunks_per_token;
+    // (never beyond the rows k_new / v_new and the slot mapping have, whatever the offsets say)
+    const int64_t n_rows = min(static_cast<int64_t>(a.cu_new[a.num_seqs]), a.n_new);
+    const int64_t total = n_rows * chunks_per_token;
     const int64_t n_slots = a.n_pages * a.page_size;
     const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
     uint8_t* kc = const_cast<uint8_t*>(a.k_cache);

@@ -246,9 +246,6 @@ struct StreamAttn : TileMath<HD, NB, NW, HIDDEN> {
     // ---- loads -----------------------------------------------------------------------------
     // Start the loads of planned unit `rel` (this wave's band of K and V rows) into its ring stage.
     DFX_D void issue_unit(int rel) const {
-#ifdef DFX_ABLATE_LOADS
-        if (rel >= 4) return;
-#endif
         const BandDesc b = bands[rel * NW + wave];
         const int last = uniform(b.last);
         const bool is_ctx = uniform(b.is_ctx) != 0;
@@ -471,9 +468,6 @@ struct StreamAttn : TileMath<HD, NB, NW, HIDDEN> {
 
     // Wait until at most `younger` units' loads of this wave are outstanding (younger <= 2).
     DFX_D static void wait_younger(int younger) {
-#ifdef DFX_ABLATE_LOADS
-        return;
-#endif
         if (younger >= 2) wait_async_loads<2 * C::LOADS_PER_UNIT>();
         else if (younger == 1) wait_async_loads<C::LOADS_PER_UNIT>();
         else wait_async_loads<0>();

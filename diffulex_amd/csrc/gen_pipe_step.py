@@ -44,7 +44,6 @@ from __future__ import annotations
 import os
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-ABLATE = set(filter(None, os.environ.get("DFX_PIPE_ABLATE", "").split(",")))  # development: drop instruction classes
 
 HD = 128
 ROWB = HD * 2
@@ -90,16 +89,12 @@ class Block:
         self.recent_valu_defs = (self.recent_valu_defs + [set(defs)])[-2:]
 
     def valu(self, text, defs):
-        if "valu" in ABLATE and ("v_exp" in text or "v_fma" in text or "v_add_f32" in text or "v_cvt" in text or "v_max" in text):
-            return
         self._push(text, defs)
 
     def other(self, text):
         self._push(text)
 
     def lds_read(self, text, tag):
-        if "lds" in ABLATE:
-            return
         self._push(text)
         self.lds_queue.append(tag)
 
@@ -113,8 +108,6 @@ class Block:
 
     def mfma(self, dst, a, b, c, reads):
         """reads: registers (numbers) of vector operands a/b/c written by the vector ALU."""
-        if "mfma" in ABLATE:
-            return
         if any(set(reads) & d for d in self.recent_valu_defs):
             self._push("s_nop 1")
         self._push(f"v_mfma_f32_32x32x16_bf16 {dst}, {a}, {b}, {c}")

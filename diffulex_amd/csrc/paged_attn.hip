@@ -205,8 +205,9 @@ int check_args(const dfx_attn_params* p, Plan& plan, bool& empty) {
     if (has_cache && (!p->block_tables || p->page_size <= 0 || p->max_pages_per_seq < 0 || p->n_pages < 0))
         return DFX_ERR_INVALID_ARG;
     if (plan.fp8 && (!p->k_scale || !p->v_scale)) return DFX_ERR_INVALID_ARG;
+    if (p->num_new_tokens < 0) return DFX_ERR_INVALID_ARG;
     if (p->store_slot_mapping != nullptr) {
-        if (!has_cache) return DFX_ERR_INVALID_ARG;
+        if (!has_cache || p->num_new_tokens <= 0) return DFX_ERR_INVALID_ARG;  // the store needs the row count
         if (p->store_slot_index_type != DFX_INDEX_I32 && p->store_slot_index_type != DFX_INDEX_I64)
             return DFX_ERR_INVALID_ARG;
     }
@@ -241,7 +242,7 @@ uint32_t plan_signature(const dfx_attn_params* p, const Plan& plan) {
     };
     mix(plan.hd); mix(plan.nb); mix(plan.n_wg); mix(plan.fp8); mix(plan.stream); mix(plan.compact);
     mix(p->num_seqs); mix(p->num_q_heads); mix(p->num_kv_heads); mix(p->page_size); mix(p->max_pages_per_seq);
-    mix(p->max_seqlen_q); mix(p->diffusion_block_size); mix(p->mask_mode); mix(p->max_workgroups);
+    mix(p->max_seqlen_q); mix(p->num_new_tokens); mix(p->diffusion_block_size); mix(p->mask_mode); mix(p->max_workgroups);
     mix(p->kn_stride_token); mix(p->kn_stride_head); mix(p->cache_stride_page); mix(p->cache_stride_token);
     mix(p->cache_stride_head); mix(p->block_table_stride); mix(p->n_pages); mix(p->k_cache != nullptr);
     mix(reinterpret_cast<uintptr_t>(p->block_tables)); mix(reinterpret_cast<uintptr_t>(p->context_lens));
@@ -330,6 +331,7 @@ int run_paged_attn(const dfx_attn_params* p, void* workspace, int64_t workspace_
         ka.busy_waves = static_cast<int>(rows >= 32 * kMaxWaves ? kMaxWaves : (rows + 31) / 32);
     }
     ka.c = p->scale * kLog2e;
+    ka.n_new = p->num_new_tokens > 0 ? p->num_new_tokens : INT64_MAX;
     ka.plan = nullptr;
     ka.plan_signature = plan_signature(p, plan);
     if (plan_out == nullptr && plan.stream && p->plan != nullptr) {

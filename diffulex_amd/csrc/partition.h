@@ -167,14 +167,8 @@ DFX_HD void owners_of_units(const WgSplit& sp, int me, int64_t first_unit, int64
 // only cut if its long item exceeds the launch's critical length M, the smallest value every pair
 // can meet; cost constants below are in tiles (measured: a stored piece costs its workgroup about
 // 1.5 tiles' time, a merged one 3, a second item's query rows and output 1.5).
-#ifndef DFX_PAIR_COST_MERGE
-#define DFX_PAIR_COST_MERGE 3
-#endif
-#ifndef DFX_PAIR_COST_DONEE
-#define DFX_PAIR_COST_DONEE 3
-#endif
-constexpr int kPairCostMerge = DFX_PAIR_COST_MERGE;   // on the side that keeps the item's end
-constexpr int kPairCostDonee = DFX_PAIR_COST_DONEE;   // on the side that takes the donated tiles: store + second item
+constexpr int kPairCostMerge = 3;   // on the side that keeps the item's end
+constexpr int kPairCostDonee = 3;   // on the side that takes the donated tiles: store + second item
 constexpr int kPairSlack = 6;       // accept the pairing while M <= ceil(total / n_wg) + this
 constexpr int kMaxPairItems = 1024;
 
@@ -191,14 +185,6 @@ DFX_HD int pair_donation(int l, int s, int M) {
     if (d > l - 1) d = l - 1;             // the owner keeps at least the item's last tile
     return d < 1 ? 1 : d;
 }
-
-// What one workgroup does under the pairing partition: linear unit ranges [a0, a1) then [b0, b1)
-// (either may be empty), each inside one item; `partner` is the workgroup holding the other piece
-// of the item it shares (or -1).
-struct PairWork {
-    int64_t a0, a1, b0, b1;
-    int32_t partner;
-};
 
 // A workgroup writes at most two partial results: slot 2w for a piece that starts at the
 // first unit of its range, slot 2w+1 for a piece that starts later (it then necessarily

@@ -113,6 +113,7 @@ def paged_attention(q, k, v, k_cache, v_cache, scale, *, block_tables, context_l
     p.vn_stride_token, p.vn_stride_head = v.stride(0), v.stride(1)
     p.o_stride_token, p.o_stride_head = out.stride(0), out.stride(1)
     p.num_seqs, p.num_q_heads, p.num_kv_heads, p.head_dim = num_seqs, H_q, H_kv, hd
+    p.num_new_tokens = k.shape[0]
     p.max_seqlen_q = int(max_seqlen_q)
     p.diffusion_block_size = int(diffusion_block_size)
     p.mask_mode = int(mask_mode)

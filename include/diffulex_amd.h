@@ -19,7 +19,7 @@
 extern "C" {
 #endif
 
-#define DFX_ABI_VERSION 5
+#define DFX_ABI_VERSION 6
 
 typedef void* dfx_stream_t; /* a hipStream_t; NULL is the default stream */
 
@@ -143,7 +143,10 @@ typedef struct dfx_attn_params {
     const void* v_new;
     const void* k_cache;         /* [n_pages, page_size, num_kv_heads, head_dim]; NULL: no cached context */
     const void* v_cache;
-    void* out;                   /* [T_q, num_q_heads, head_dim] bf16 */
+    void* out;                   /* [T_q, num_q_heads, head_dim] bf16.  Rows of a sequence that has no key at all
+                                    (no context, no fresh rows) are left unwritten, as the reference leaves
+                                    them (dllm_flash_attn.py:343-345); a row whose keys are all on skipped
+                                    pages gets zeros. */
     const int32_t* block_tables; /* [num_seqs, block_table_stride]; a page whose entry is < 0 (or >= n_pages) is
                                     skipped: its tokens take no part, as in the reference (dllm_flash_attn.py:260-261) */
     const int32_t* context_lens; /* [num_seqs]; NULL means 0 everywhere */
@@ -188,6 +191,11 @@ typedef struct dfx_attn_params {
      * small for the batch). */
     const void* plan;
     int64_t plan_bytes;
+    /* Rows of k_new / v_new (and entries of store_slot_mapping).  Fresh rows the offsets in
+     * cu_seqlens_new point beyond it are neither attended nor stored (padded batches, e.g. the
+     * reference's graph-capture metadata, carry such offsets).  0: unknown, the offsets are trusted;
+     * required (> 0) with store_slot_mapping. */
+    int64_t num_new_tokens;
 } dfx_attn_params;
 
 /* Bytes of scratch dfx_paged_attn needs for these shapes (depends on the sizes

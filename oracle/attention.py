@@ -107,6 +107,10 @@ def paged_attention_fp32(q, k_new, v_new, k_cache, v_cache, block_tables, contex
             vv = torch.cat([vc.float(), v_new[n0:n1].float()], 0)
         else:
             kk, vv = k_new[n0:n1].float(), v_new[n0:n1].float()
+        if kk.shape[0] == 0:
+            # No key at all (every page of the context skipped, no fresh rows): the softmax is over
+            # an empty set.  The reference's kernel divides 0 by 0 there; this build defines zeros.
+            continue
         allowed = visible_mask(q1 - q0, ctx, n1 - n0, mask_mode, dbs)
         qq = q[q0:q1].float()
         for h in range(h_q):

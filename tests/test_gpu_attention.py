@@ -420,6 +420,72 @@ def test_pages_with_negative_table_entries_are_skipped(dev, name, over, flags):
         assert max_abs_err(got, want) <= tol
 
 
+@pytest.mark.parametrize("flags", PATHS)
+@pytest.mark.parametrize("name,over", [
+    ("c3", dict(num_seqs=4, ctx=[300, 513, 64, 700], page=32)),
+    ("c5", dict(num_seqs=3, ctx=[300, 513, 200])),
+    ("c4", dict(num_seqs=3, ctx=[100, 300, 95], page=48)),
+])
+def test_rows_with_no_visible_key_get_zeros(dev, name, over, flags):
+    """A sequence all of whose context pages are skipped and that brings no fresh rows has nothing
+    to attend to: its rows are zeros (finite), the other sequences are unaffected."""
+    wl = make_workload(name, seed=67, **over)
+    bt = wl.block_tables.clone()
+    bt[1, :] = -1
+    wl.block_tables = bt
+    cu_q = wl.cu_seqlens_q.tolist()
+    lens_new = [cu_q[i + 1] - cu_q[i] for i in range(wl.num_seqs)]
+    lens_new[1] = 0                                    # sequence 1: no fresh rows either
+    cu_new = torch.tensor([0] + np.cumsum(lens_new).tolist(), dtype=torch.int32)
+    keep = torch.cat([torch.arange(cu_q[i], cu_q[i + 1]) for i in range(wl.num_seqs) if i != 1])
+    wl.k_new, wl.v_new = wl.k_new[keep].contiguous(), wl.v_new[keep].contiguous()
+    want = oracle_fp32(wl, cu_seqlens_new=cu_new)
+    assert float(want[cu_q[1]:cu_q[2]].abs().max()) == 0.0
+    g = wl.to(dev)
+    tol = ATOL_FP8 if name == "c5" else ATOL_BF16
+    for max_wg in (0, 3):
+        got = _run(g, max_wg, flags=flags, cu_seqlens_new=cu_new.to(dev))
+        assert torch.isfinite(got.float()).all()
+        assert float(got[cu_q[1]:cu_q[2]].float().abs().max()) == 0.0
+        assert max_abs_err(got, want) <= tol
+
+
+@pytest.mark.parametrize("flags", PATHS)
+@pytest.mark.parametrize("name,over", [
+    ("c3", dict(num_seqs=5, ctx=(200, 700))),
+    ("c5", dict(num_seqs=4, ctx=(200, 900))),
+    ("c4", dict(num_seqs=3, ctx=(100, 500))),
+])
+def test_fresh_rows_are_bounded_by_the_rows_passed(dev, name, over, flags):
+    """Offsets in cu_seqlens_new that point beyond the rows of k_new / v_new (padded batches) are
+    cut to the rows there are, for the attention and for the fused store: the result equals the one
+    with the offsets clamped, and the cache rows of the missing tokens stay as they were."""
+    wl = make_workload(name, seed=71, **over).to(dev)
+    cu = wl.cu_seqlens_q
+    t_all = int(cu[-1])
+    t_have = int(cu[-2]) + (t_all - int(cu[-2])) // 2          # the last sequence lost half its fresh rows
+    k_new, v_new = wl.k_new[:t_have].contiguous(), wl.v_new[:t_have].contiguous()
+    slots = wl.slot_mapping[:t_have].contiguous()
+    cu_clamped = torch.clamp(cu, max=t_have)
+    common = dict(block_tables=wl.block_tables, context_lens=wl.context_lens, cu_seqlens_q=cu,
+                  max_seqlen_q=wl.q_len, mask_mode=wl.mask_mode, diffusion_block_size=wl.diffusion_block_size,
+                  k_scale=wl.k_scale, v_scale=wl.v_scale, flags=flags)
+    for max_wg in (0, 3):
+        kc_a, vc_a = wl.k_cache.clone(), wl.v_cache.clone()
+        want = dfx.paged_attention(wl.q, k_new, v_new, kc_a, vc_a, wl.scale, cu_seqlens_new=cu_clamped,
+                                   store_slot_mapping=slots, max_workgroups=max_wg, **common)
+        kc_b, vc_b = wl.k_cache.clone(), wl.v_cache.clone()
+        got = dfx.paged_attention(wl.q, k_new, v_new, kc_b, vc_b, wl.scale, cu_seqlens_new=cu,
+                                  store_slot_mapping=slots, max_workgroups=max_wg, **common)
+        torch.cuda.synchronize()
+        assert torch.equal(got, want)
+        assert torch.equal(kc_b.view(torch.uint8), kc_a.view(torch.uint8))
+        assert torch.equal(vc_b.view(torch.uint8), vc_a.view(torch.uint8))
+    c = wl.to("cpu")
+    ref = oracle_fp32(c, k_new=c.k_new[:t_have], v_new=c.v_new[:t_have], cu_seqlens_new=cu_clamped.cpu())
+    assert max_abs_err(got, ref) <= (ATOL_FP8 if name == "c5" else ATOL_BF16)
+
+
 @pytest.mark.parametrize("name,over,tol", [
     # more sequences than the two-workgroups-per-CU variant plans for (1023): the one-per-CU variants
     ("c3", dict(num_seqs=1500, ctx=(0, 150), h_q=8, h_kv=2), ATOL_BF16),

@@ -103,6 +103,11 @@ def test_argument_errors_do_not_launch():
     p.kn_stride_head = p.vn_stride_head = 128
     p.scale, p.diffusion_block_size = 0.5, 32
     assert lib.dfx_paged_attn_static(C.byref(p), None) == _lib.DFX_ERR_SCRATCH_LIMIT
+    # the fused store needs a cache and the number of fresh rows; a negative row count is refused
+    p.store_slot_mapping, p.num_new_tokens = 4096, 64
+    assert lib.dfx_paged_attn_static(C.byref(p), None) == -1          # no cache
+    p.store_slot_mapping, p.num_new_tokens = None, -1
+    assert lib.dfx_paged_attn_static(C.byref(p), None) == -1
 
 
 def test_device_quantiser_source_matches_oracle_on_host():

@@ -25,7 +25,7 @@ DFX_WORKSPACE_COUNTER_BYTES = 1 << 18
 EXPORTS = (
     "dfx_abi_version", "dfx_status_string", "dfx_kv_store_unified", "dfx_kv_store_distinct",
     "dfx_kv_load", "dfx_paged_attn_workspace_bytes", "dfx_paged_attn", "dfx_paged_attn_static", "dfx_paged_attn_plan_bytes", "dfx_paged_attn_plan", "dfx_stream_capture_id",
-    "dfx_rope_kv_store",
+    "dfx_rope_kv_store", "dfx_build_decode_metadata",
 )
 
 
@@ -66,6 +66,24 @@ class RopeParams(C.Structure):
         ("slot_mapping", C.c_void_p), ("slot_index_type", C.c_int32), ("n_slots", C.c_int64),
         ("k_scale", C.c_void_p), ("v_scale", C.c_void_p),
     ]
+
+
+class MetadataParams(C.Structure):
+    """Mirror of ``dfx_metadata_params``."""
+    _fields_ = [
+        ("strategy", C.c_int32), ("num_seqs", C.c_int32), ("page_size", C.c_int32), ("diffusion_block_size", C.c_int32),
+        ("num_tokens", C.c_void_p), ("prompt_len", C.c_void_p), ("block_state", C.c_void_p),
+        ("block_state_stride", C.c_int64), ("num_diffusion_blocks", C.c_void_p),
+        ("block_tables", C.c_void_p), ("block_table_stride", C.c_int64), ("num_pages", C.c_void_p),
+        ("positions", C.c_void_p), ("slot_mapping", C.c_void_p), ("token_capacity", C.c_int64),
+        ("cu_seqlens_q", C.c_void_p), ("cu_seqlens_k", C.c_void_p), ("context_lens", C.c_void_p),
+        ("seq_lens", C.c_void_p), ("padded_seqs", C.c_int32), ("reserved", C.c_int32),
+        ("padded_tokens", C.c_int64), ("summary", C.c_void_p),
+    ]
+
+
+DFX_BLOCK_IN_CACHE, DFX_BLOCK_TO_CACHE, DFX_BLOCK_ACTIVE = 0, 1, 2
+DFX_META_BLOCK_DIFFUSION, DFX_META_D2F = 0, 1
 
 
 class DfxError(RuntimeError):
@@ -111,6 +129,8 @@ def load() -> C.CDLL:
     lib.dfx_paged_attn_static.argtypes = [C.POINTER(AttnParams), vp]
     lib.dfx_rope_kv_store.restype = i32
     lib.dfx_rope_kv_store.argtypes = [C.POINTER(RopeParams), vp]
+    lib.dfx_build_decode_metadata.restype = i32
+    lib.dfx_build_decode_metadata.argtypes = [C.POINTER(MetadataParams), vp]
     if lib.dfx_abi_version() != DFX_ABI_VERSION:
         raise ImportError(f"{LIB_PATH} has ABI {lib.dfx_abi_version()}, expected {DFX_ABI_VERSION}: rebuild it")
     _lib = lib

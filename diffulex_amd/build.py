@@ -24,7 +24,7 @@ HIP_FLAGS = [
     f"--offload-arch={ARCH}", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function", "-Wno-inline-asm",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
 ]
-SOURCES = ["capi.cpp", "kv_cache.hip", "paged_attn.hip", "rotary.hip"]
+SOURCES = ["capi.cpp", "kv_cache.hip", "metadata.hip", "paged_attn.hip", "rotary.hip"]
 
 
 def _hipcc() -> str:

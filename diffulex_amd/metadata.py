@@ -56,6 +56,92 @@ class PagedAttnMetaData(AttnMetaDataBase):
                 self.total_lens = self.diffusion_block_size + self.context_lens
 
 
+def build_decode_metadata(strategy: str, *, block_tables: torch.Tensor, block_state: torch.Tensor,
+                          page_size: int, diffusion_block_size: int, num_tokens: Optional[torch.Tensor] = None,
+                          num_pages: Optional[torch.Tensor] = None, prompt_len: Optional[torch.Tensor] = None,
+                          num_diffusion_blocks: Optional[torch.Tensor] = None, token_capacity: int,
+                          padded_seqs: int = 0, padded_tokens: int = 0, out: Optional[dict] = None,
+                          kv_cache_layout: str = "unified", sync_summary: bool = False) -> "PagedAttnMetaData":
+    """The metadata of one decode step from per-sequence state kept on the device
+    (``dfx_build_decode_metadata``): what ``prepare_decode`` of the reference's runners computes
+    in Python loops and copies over (block_diffusion/engine/model_runner.py:114-173,
+    d2f/engine/model_runner.py:137-262).
+
+    ``strategy``: "block_diffusion" (``num_tokens`` [B] int32, ``block_state`` [B] uint8 = state of
+    the last diffusion block, ``num_pages`` [B] int32) or "d2f" (``prompt_len`` [B],
+    ``num_diffusion_blocks`` [B], ``block_state`` [B, max_blocks] uint8, ``num_tokens`` optional).
+    ``out``: a dict of preallocated output tensors (``positions``, ``slot_mapping``,
+    ``cu_seqlens_q``, ``cu_seqlens_k``, ``context_lens``, ``seq_lens``, ``summary``), e.g. the
+    buffers a graph was captured on, padded to ``padded_seqs`` / ``padded_tokens``; by default new
+    tensors are made.  Nothing is read back unless ``sync_summary`` is set: ``max_seqlen_q`` is then
+    the true maximum, otherwise an upper bound from the shapes (enough for the attention operators).
+    Returns the metadata object with ``positions`` and ``summary`` attached as attributes."""
+    import ctypes as C
+    from . import _lib
+    from .kv_cache_kernels import _stream
+    lib = _lib.load()
+    dev = block_tables.device
+    B = block_tables.shape[0]
+    rows = max(B, padded_seqs)
+    cap = max(int(token_capacity), int(padded_tokens))
+    i32 = dict(dtype=torch.int32, device=dev)
+    o = dict(out) if out is not None else {}
+    o.setdefault("positions", torch.empty(cap, dtype=torch.int64, device=dev))
+    o.setdefault("slot_mapping", torch.empty(cap, **i32))
+    o.setdefault("cu_seqlens_q", torch.empty(rows + 1, **i32))
+    o.setdefault("cu_seqlens_k", torch.empty(rows + 1, **i32))
+    o.setdefault("context_lens", torch.empty(rows, **i32))
+    o.setdefault("seq_lens", torch.empty(rows, **i32))
+    o.setdefault("summary", torch.empty(8, **i32))
+    assert block_tables.dtype == torch.int32 and block_tables.stride(-1) == 1
+    assert block_state.dtype == torch.uint8 and block_state.stride(-1) == 1
+    p = _lib.MetadataParams()
+    p.strategy = {"block_diffusion": _lib.DFX_META_BLOCK_DIFFUSION, "d2f": _lib.DFX_META_D2F}[strategy]
+    p.num_seqs, p.page_size, p.diffusion_block_size = B, int(page_size), int(diffusion_block_size)
+    for name, t in (("num_tokens", num_tokens), ("prompt_len", prompt_len), ("num_pages", num_pages),
+                    ("num_diffusion_blocks", num_diffusion_blocks)):
+        if t is not None:
+            assert t.dtype == torch.int32 and t.is_contiguous() and t.numel() == B and t.device == dev
+            setattr(p, name, t.data_ptr())
+    p.block_state = block_state.data_ptr()
+    p.block_state_stride = block_state.stride(0) if block_state.dim() == 2 else 1
+    p.block_tables, p.block_table_stride = block_tables.data_ptr(), block_tables.stride(0)
+    for name in ("positions", "slot_mapping", "cu_seqlens_q", "cu_seqlens_k", "context_lens", "seq_lens", "summary"):
+        assert o[name].is_contiguous() and o[name].device == dev
+        setattr(p, name, o[name].data_ptr())
+    assert o["positions"].dtype == torch.int64 and o["positions"].numel() >= cap and o["slot_mapping"].numel() >= cap
+    assert o["cu_seqlens_q"].numel() >= rows + 1 and o["cu_seqlens_k"].numel() >= rows + 1
+    assert o["context_lens"].numel() >= rows and o["seq_lens"].numel() >= rows and o["summary"].numel() >= 8
+    p.token_capacity, p.padded_seqs, p.padded_tokens = cap, int(padded_seqs), int(padded_tokens)
+    _lib.check(lib.dfx_build_decode_metadata(C.byref(p), _stream()), "dfx_build_decode_metadata")
+    d2f = strategy == "d2f"
+    n_tokens = cap
+    max_q = max_k = 0
+    need_store = True
+    if sync_summary:
+        host = o["summary"].tolist()
+        if host[5]:
+            raise ValueError(f"token_capacity {cap} is too small for {max(host[0], host[1])} tokens")
+        if host[6]:
+            raise ValueError(f"sequence {host[6] - 1} is in a state the decode step cannot be prepared from")
+        n_tokens, max_q, max_k, need_store = host[0], host[2], host[3], bool(host[4])
+    elif not d2f:
+        n_tokens, max_q, max_k = B * diffusion_block_size, diffusion_block_size, diffusion_block_size
+    else:
+        max_q = block_state.shape[-1] * diffusion_block_size if block_state.dim() == 2 else cap
+    n_tokens = max(n_tokens, int(padded_tokens))
+    md = PagedAttnMetaData(
+        is_prefill=False, cu_seqlens_q=o["cu_seqlens_q"][:rows + 1], cu_seqlens_k=o["cu_seqlens_k"][:rows + 1],
+        max_seqlen_q=max_q, max_seqlen_k=max_k, slot_mapping=o["slot_mapping"][:n_tokens],
+        context_lens=o["context_lens"][:rows], block_tables=block_tables, page_block_size=int(page_size),
+        attn_type="full_attention" if d2f else "block_attention", diffusion_block_size=int(diffusion_block_size),
+        decode_mode="varlen" if d2f else "static", seq_lens_ts=o["seq_lens"][:rows] if d2f else None,
+        kv_cache_layout=kv_cache_layout, need_kv_cache_store=need_store)
+    md.positions = o["positions"][:n_tokens]
+    md.summary = o["summary"]
+    return md
+
+
 FN_TYPE_AttnMetaDataFetch = Callable[[], AttnMetaDataBase]
 
 fetch_attn_metadata: FN_TYPE_AttnMetaDataFetch = ...

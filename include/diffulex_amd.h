@@ -243,6 +243,82 @@ int64_t dfx_stream_capture_id(dfx_stream_t stream);
 int dfx_paged_attn_plan(const dfx_attn_params* params, void* plan, int64_t plan_bytes, dfx_stream_t stream);
 
 /*
+ * Attention metadata of one decode step, built on the device.
+ * Replaces: the Python loops of prepare_decode and the six host-to-device copies that follow them
+ *           (diffulex/strategy/block_diffusion/engine/model_runner.py:114-173 with
+ *           BDSequence.diffusion_decoding_inputs, block_diffusion/engine/sequence.py:186-191;
+ *           diffulex/strategy/d2f/engine/model_runner.py:137-262 with
+ *           D2FSequence.diffusion_decoding_inputs, d2f/engine/sequence.py:357-370), and the
+ *           zero-fill-then-copy of the graph buffers in run_model
+ *           (block_diffusion/engine/model_runner.py:176-197).  The layout CHECK_SLOT_MAPPING
+ *           demands (diffulex/utils/checker.py:1-27) holds by construction.
+ *
+ * A sequence is described by what those loops read from it (all arrays on the device, so a
+ * scheduler that keeps its state there needs no copy at all):
+ *   DFX_META_BLOCK_DIFFUSION: num_tokens[s] = len(seq) after next_diffusion_step, block_state[s *
+ *     block_state_stride] = state of its last diffusion block, num_pages[s] = len(seq.block_table).
+ *     The step feeds the last diffusion_block_size tokens: context_lens[s] = num_tokens[s] - dbs,
+ *     cu_seqlens_q and cu_seqlens_k advance by dbs; an ACTIVE block contributes dbs entries -1 to the
+ *     slot mapping, a TO_CACHE block the slots of the last dbs / page_size pages of its table row
+ *     (page by page, page_size slots each), an IN_CACHE block nothing.
+ *   DFX_META_D2F: prompt_len[s] = seq.input_num_tokens (the size of diffusion block 0),
+ *     num_diffusion_blocks[s] and block_state[s * block_state_stride + b] for each of its blocks, in
+ *     the only order the reference's state machine produces: IN_CACHE* TO_CACHE* ACTIVE*, block 0 in the
+ *     cache.  Blocks after the first have dbs tokens; num_tokens (optional) gives len(seq) where the
+ *     last block is shorter.  The step feeds every block after the cached ones: context_lens[s] =
+ *     cached tokens, cu_seqlens_q advances by len(seq) - cached, cu_seqlens_k by len(seq), seq_lens[s] =
+ *     fed tokens; a token to be cached at position g of the sequence gets slot
+ *     block_tables[s][g / page_size] * page_size + g % page_size, every token from the first active
+ *     block on gets -1.
+ * positions[i] (int64) = position in its sequence of the i-th fed token.
+ *
+ * padded_seqs / padded_tokens (0: none): the output arrays are the buffers of a captured graph of
+ * that batch size; entries beyond the step's own are set to 0, as the reference's run_model leaves
+ * them (cu_seqlens_*[num_seqs + 1 .. padded_seqs], context_lens / seq_lens[num_seqs .. padded_seqs),
+ * positions / slot_mapping up to padded_tokens).  Block-table rows are the caller's.
+ *
+ * summary[8] (int32, device; read it only if the host needs the numbers): fed tokens, slot-mapping
+ * entries, max_seqlen_q, max_seqlen_k, need_kv_cache_store, 1 if token_capacity was too small
+ * (nothing is written beyond it), 1 + index of the first sequence in a state the reference's loop
+ * would raise on (such a sequence contributes nothing; 0: none), sum of cu_seqlens_k steps.
+ *
+ * One launch of one workgroup, no host synchronisation, no allocation; safe to capture.
+ * DFX_ERR_UNSUPPORTED: more than 8192 sequences.
+ */
+typedef enum dfx_block_state { DFX_BLOCK_IN_CACHE = 0, DFX_BLOCK_TO_CACHE = 1, DFX_BLOCK_ACTIVE = 2 } dfx_block_state;
+typedef enum dfx_meta_strategy { DFX_META_BLOCK_DIFFUSION = 0, DFX_META_D2F = 1 } dfx_meta_strategy;
+
+typedef struct dfx_metadata_params {
+    int32_t strategy; /* dfx_meta_strategy */
+    int32_t num_seqs;
+    int32_t page_size;            /* tokens per page (the reference's kvcache_block_size) */
+    int32_t diffusion_block_size;
+    /* inputs */
+    const int32_t* num_tokens;           /* [num_seqs]; optional for D2F */
+    const int32_t* prompt_len;           /* [num_seqs]; D2F only */
+    const uint8_t* block_state;          /* dfx_block_state codes, see above */
+    int64_t block_state_stride;          /* elements between sequences */
+    const int32_t* num_diffusion_blocks; /* [num_seqs]; D2F only */
+    const int32_t* block_tables;         /* [num_seqs, block_table_stride] page ids */
+    int64_t block_table_stride;
+    const int32_t* num_pages;            /* [num_seqs]; block diffusion only */
+    /* outputs */
+    int64_t* positions;    /* [token_capacity] */
+    int32_t* slot_mapping; /* [token_capacity] */
+    int64_t token_capacity;
+    int32_t* cu_seqlens_q; /* [max(num_seqs, padded_seqs) + 1] */
+    int32_t* cu_seqlens_k;
+    int32_t* context_lens; /* [max(num_seqs, padded_seqs)] */
+    int32_t* seq_lens;     /* the same size, or NULL */
+    int32_t padded_seqs;
+    int32_t reserved;
+    int64_t padded_tokens;
+    int32_t* summary; /* [8] */
+} dfx_metadata_params;
+
+int dfx_build_decode_metadata(const dfx_metadata_params* params, dfx_stream_t stream);
+
+/*
  * dfx_paged_attn without a caller-provided workspace, for callers that cannot allocate device
  * memory (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).
  * No counterpart in the reference.

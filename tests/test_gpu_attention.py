@@ -357,6 +357,55 @@ def test_graphs_captured_as_the_reference_runner_does(dev):
 
 
 @pytest.mark.parametrize("flags", PATHS)
+@pytest.mark.parametrize("name,over,n_real", [
+    ("c3", dict(num_seqs=8, ctx=(200, 900)), 5),
+    ("c3", dict(num_seqs=16, ctx=(100, 2000), page=32), 9),
+    ("c5", dict(num_seqs=8, ctx=(300, 1200)), 3),
+])
+def test_graph_buffers_padded_the_way_the_reference_pads_them(dev, name, over, n_real, flags):
+    """The reference replays a graph captured for a larger batch on zero-filled buffers with the
+    step's values in front (strategy/block_diffusion/engine/model_runner.py:176-197): behind the
+    real sequences cu_seqlens drop back to 0 (the first padded sequence has a negative length),
+    context_lens are 0 and the block-table rows are all page 0.  The real sequences' rows come out
+    as without the padding; at capture time cu_seqlens_k counts in steps of max_model_len (:221-223),
+    offsets far beyond the fresh rows, which must not be followed."""
+    wl = make_workload(name, seed=97, **over).to(dev)
+    n_pad, dbs = wl.num_seqs, wl.q_len
+    cu = wl.cu_seqlens_q.clone()
+    cu[n_real + 1:] = 0
+    ctx = wl.context_lens.clone()
+    ctx[n_real:] = 0
+    bt = wl.block_tables.clone()
+    bt[n_real:] = 0
+    common = dict(max_seqlen_q=dbs, mask_mode=wl.mask_mode, diffusion_block_size=wl.diffusion_block_size,
+                  k_scale=wl.k_scale, v_scale=wl.v_scale, flags=flags)
+    t = n_real * dbs
+    want = dfx.paged_attention(wl.q[:t], wl.k_new[:t], wl.v_new[:t], wl.k_cache, wl.v_cache, wl.scale,
+                               block_tables=wl.block_tables[:n_real], context_lens=wl.context_lens[:n_real],
+                               cu_seqlens_q=wl.cu_seqlens_q[:n_real + 1], cu_seqlens_new=wl.cu_seqlens_q[:n_real + 1],
+                               **common)
+    out = torch.full_like(wl.q, 3.0)
+    dfx.paged_attention(wl.q, wl.k_new, wl.v_new, wl.k_cache, wl.v_cache, wl.scale, block_tables=bt, context_lens=ctx,
+                        cu_seqlens_q=cu, cu_seqlens_new=cu, out=out, **common)
+    torch.cuda.synchronize()
+    assert torch.equal(out[:t], want)
+    assert (out[t:] == 3.0).all()                       # rows of the padding are not touched
+    assert max_abs_err(want, oracle_fp32(wl)[:t]) <= (ATOL_FP8 if name == "c5" else ATOL_BF16)
+    # capture-time metadata: zero lengths and tables, fresh-row offsets in steps of max_model_len
+    far = (torch.arange(n_pad + 1, device=dev, dtype=torch.int32) * 4096)
+    kc, vc = wl.k_cache.clone(), wl.v_cache.clone()
+    slots = torch.zeros(n_pad * dbs, dtype=torch.int32, device=dev)
+    got = dfx.paged_attention(wl.q, wl.k_new, wl.v_new, kc, vc, wl.scale, block_tables=torch.zeros_like(bt),
+                              context_lens=torch.zeros_like(ctx), cu_seqlens_q=wl.cu_seqlens_q, cu_seqlens_new=far,
+                              store_slot_mapping=slots, **common)
+    torch.cuda.synchronize()
+    # only sequence 0 has fresh rows inside k_new: offsets 0 .. 4096 are cut to the rows there are
+    clamped = torch.clamp(far, max=n_pad * dbs).cpu()
+    ref = oracle_fp32(wl, context_lens=torch.zeros_like(ctx).cpu(), cu_seqlens_new=clamped)
+    assert max_abs_err(got[:dbs], ref[:dbs]) <= (ATOL_FP8 if name == "c5" else ATOL_BF16)
+
+
+@pytest.mark.parametrize("flags", PATHS)
 @pytest.mark.parametrize("name,over", [
     ("c1", {}),
     ("c3", dict(num_seqs=5, ctx=(200, 700))),

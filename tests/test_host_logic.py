@@ -28,7 +28,8 @@ def test_library_exports_every_declared_symbol():
     assert lib.dfx_status_string(-2) == b"unsupported shape"
 
 
-@pytest.mark.parametrize("ctype,mirror", [("dfx_attn_params", _lib.AttnParams), ("dfx_rope_params", _lib.RopeParams)])
+@pytest.mark.parametrize("ctype,mirror", [("dfx_attn_params", _lib.AttnParams), ("dfx_rope_params", _lib.RopeParams),
+                                          ("dfx_metadata_params", _lib.MetadataParams)])
 def test_struct_layout_matches_header(tmp_path, ctype, mirror):
     """Size and every field offset of the ctypes mirror against what a C compiler makes of the header."""
     names = [f[0] for f in mirror._fields_]

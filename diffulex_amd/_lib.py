@@ -50,6 +50,7 @@ class AttnParams(C.Structure):
         ("max_workgroups", C.c_int32), ("flags", C.c_int32), ("scale", C.c_float),
         ("store_slot_mapping", C.c_void_p), ("store_slot_index_type", C.c_int32),
         ("plan", C.c_void_p), ("plan_bytes", C.c_int64), ("num_new_tokens", C.c_int64),
+        ("cache_layout", C.c_int32), ("reserved1", C.c_int32), ("kc_stride", C.c_int64 * 5), ("vc_stride", C.c_int64 * 4),
     ]
 
 
@@ -84,6 +85,7 @@ class MetadataParams(C.Structure):
 
 DFX_BLOCK_IN_CACHE, DFX_BLOCK_TO_CACHE, DFX_BLOCK_ACTIVE = 0, 1, 2
 DFX_META_BLOCK_DIFFUSION, DFX_META_D2F = 0, 1
+DFX_CACHE_UNIFIED, DFX_CACHE_DISTINCT = 0, 1
 
 
 class DfxError(RuntimeError):

@@ -60,6 +60,8 @@ class Attention(nn.Module):
                 o = dllm_flash_attn_decode(q, k, v, k_cache, v_cache, self.scale, attn_metadata,
                                            store_slot_mapping=fused_slots)
             else:
-                raise NotImplementedError("Distinct layout is not supported yet...")
+                # (the reference raises NotImplementedError here, attn_impl.py:66-69)
+                o = dllm_flash_attn_decode(q, k, v, k_cache, v_cache, self.scale, attn_metadata,
+                                           kv_cache_layout="distinct")
 
         return o.reshape(o.shape[0], self.num_heads * self.head_dim).contiguous()

@@ -50,6 +50,9 @@ struct KArgs {
     uint32_t plan_signature;  // of this launch's configuration: a plan made for another one is ignored
     int64_t q_st, q_sh, kn_st, kn_sh, vn_st, vn_sh, o_st, o_sh;
     int64_t c_sp, c_st, c_sh;  // cache strides in elements: page, token, head
+    // "distinct" cache layout (generic path only), strides in elements: K [page, head, d / 8, token, 8],
+    // V [page, head, d, token]
+    int64_t kd_sp, kd_sh, kd_sc, vd_sp, vd_sh, vd_sd;
     int64_t bt_stride, n_pages;
     int num_seqs, h_kv, group, page_size, page_shift, max_pages, dbs, mask_mode, n_wg;
     int fixed_wg;  // the caller fixed the number of workgroups: all of them take part

@@ -26,7 +26,10 @@ struct GenericCfg : Shape<HD, NB> {
     static constexpr int CH8 = S::TN * HD / 16 / kThreads;       // 16-byte chunks per lane, fp8 tile
 };
 
-template <int HD, int NB, bool FP8>
+// DISTINCT: the cache is in the "distinct" layout, K [pages, H, hd / 8, page, 8] and V [pages, H,
+// hd, page] (bf16): a 16-byte load still brings one 8-element chunk of a K row, but 8 consecutive
+// tokens of one d for V, which are scattered into the row-major LDS tile two bytes at a time.
+template <int HD, int NB, bool FP8, bool DISTINCT = false>
 struct GenericAttn : TileMath<HD, NB, kWaves> {
     using Base = TileMath<HD, NB, kWaves>;
     using L = TileLayout<HD>;
@@ -48,7 +51,7 @@ struct GenericAttn : TileMath<HD, NB, kWaves> {
     int* table;        // block-table entries [table_p0, table_p0 + table_n) of sequence s, if table_n > 0
     int table_p0, table_n;
     u32x4 kst[C::CH16], vst[C::CH16];
-    bool staged_fp8;
+    bool staged_fp8, staged_distinct;
 
     DFX_D GenericAttn(const KArgs& args, uint8_t* smem)
         : Base(args), lds(smem), prefix(reinterpret_cast<int*>(smem)),
@@ -76,14 +79,80 @@ struct GenericAttn : TileMath<HD, NB, kWaves> {
     DFX_D uint8_t* k_stage(int b) const { return lds + C::STAGES_OFF + b * C::STAGE_BYTES; }
     DFX_D uint8_t* v_stage(int b) const { return k_stage(b) + C::K_BYTES; }
 
-    DFX_D int64_t cache_row_offset(int tok, bool& ok) const {
+    // physical page of context token `tok` and the token's place in it; ok is cleared if the
+    // block table has no valid entry for it
+    DFX_D int64_t page_of(int tok, bool& ok, int& off) const {
         const int p = a.page_shift >= 0 ? (tok >> a.page_shift) : (tok / a.page_size);
-        const int off = tok - p * a.page_size;
+        off = tok - p * a.page_size;
         int64_t page = -1;
         if (table_n > 0) page = table[p - table_p0];
         else if (p < a.max_pages) page = a.block_tables[static_cast<int64_t>(s) * a.bt_stride + p];
         ok = ok && page >= 0 && page < a.n_pages;
+        return page;
+    }
+
+    DFX_D int64_t cache_row_offset(int tok, bool& ok) const {
+        int off;
+        const int64_t page = page_of(tok, ok, off);
         return page * a.c_sp + off * a.c_st + kvh * a.c_sh;
+    }
+
+    // Distinct layout, global -> registers.  K: the 64 lanes of a wave take one chunk column of 64
+    // consecutive tokens (1 KiB contiguous inside a page); V: eight consecutive lanes take the
+    // eight 8-token groups of one d (128 contiguous bytes).
+    DFX_D void issue_distinct(int base, int limit) {
+        const uint16_t* kc = reinterpret_cast<const uint16_t*>(a.k_cache);
+        const uint16_t* vc = reinterpret_cast<const uint16_t*>(a.v_cache);
+#pragma unroll
+        for (int i = 0; i < C::CH16; ++i) {
+            const int c = tid + kThreads * i;
+            {
+                const int row = c % C::TN, cc = c / C::TN;
+                const int tok = base + row;
+                bool ok = tok < limit;
+                u32x4 kk = {0, 0, 0, 0};
+                if (ok) {
+                    int off;
+                    const int64_t page = page_of(tok, ok, off);
+                    if (ok) kk = *reinterpret_cast<const u32x4*>(kc + page * a.kd_sp + kvh * a.kd_sh + cc * a.kd_sc + off * 8);
+                }
+                kst[i] = kk;
+            }
+            {
+                const int tg = c % 8, d = c / 8;
+                const int tok = base + tg * 8;
+                bool ok = tok < limit;
+                u32x4 vv = {0, 0, 0, 0};
+                if (ok) {
+                    int off;  // a multiple of 8: pages hold a multiple of 8 tokens
+                    const int64_t page = page_of(tok, ok, off);
+                    if (ok) vv = *reinterpret_cast<const u32x4*>(vc + page * a.vd_sp + kvh * a.vd_sh + d * a.vd_sd + off);
+                    const int n_valid = limit - tok;  // tokens past the end of the context read as zeros
+                    if (n_valid < 8) {
+#pragma unroll
+                        for (int j = 0; j < 8; ++j) {
+                            if (j >= n_valid) vv[j >> 1] &= (j & 1) ? 0x0000ffffu : 0xffff0000u;
+                        }
+                    }
+                }
+                vst[i] = vv;
+            }
+        }
+    }
+
+    DFX_D void commit_distinct(uint8_t* ks, uint8_t* vs) const {
+#pragma unroll
+        for (int i = 0; i < C::CH16; ++i) {
+            const int c = tid + kThreads * i;
+            *reinterpret_cast<u32x4*>(ks + L::chunk_offset(c % C::TN, c / C::TN)) = kst[i];
+            const int tg = c % 8, d = c / 8;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const uint32_t w = vst[i][j >> 1];
+                *reinterpret_cast<uint16_t*>(vs + L::chunk_offset(tg * 8 + j, d >> 3) + (d & 7) * 2) =
+                    static_cast<uint16_t>((j & 1) ? (w >> 16) : w);
+            }
+        }
     }
 
     // global -> registers (rows past the end of the sequence become zeros)
@@ -91,7 +160,11 @@ struct GenericAttn : TileMath<HD, NB, kWaves> {
         const bool is_ctx = tile < sh.n_ctx_tiles;
         const int base = (is_ctx ? tile : tile - sh.n_ctx_tiles) * C::TN;
         const int limit = is_ctx ? sh.ctx : sh.new_len;
-        if (FP8 && is_ctx) {
+        staged_distinct = DISTINCT && is_ctx;
+        if (DISTINCT && is_ctx) {
+            staged_fp8 = false;
+            issue_distinct(base, limit);
+        } else if (FP8 && is_ctx) {
             staged_fp8 = true;
             constexpr int CPR = HD / 16;
 #pragma unroll
@@ -144,7 +217,9 @@ struct GenericAttn : TileMath<HD, NB, kWaves> {
     DFX_D void commit(int buf) const {
         uint8_t* ks = k_stage(buf);
         uint8_t* vs = v_stage(buf);
-        if (FP8 && staged_fp8) {
+        if (DISTINCT && staged_distinct) {
+            commit_distinct(ks, vs);
+        } else if (FP8 && staged_fp8) {
             constexpr int CPR = HD / 16;  // 16-code chunks per row, each widening to two bf16 chunks
 #pragma unroll
             for (int i = 0; i < C::CH8; ++i) {
@@ -176,7 +251,8 @@ struct GenericAttn : TileMath<HD, NB, kWaves> {
         if (t.is_ctx) {  // tokens on pages without a valid block-table entry are skipped: one token per lane
             const int tok = t.base + this->lane;
             bool ok = true;
-            if (tok < t.limit) cache_row_offset(tok, ok);
+            int off;
+            if (tok < t.limit) page_of(tok, ok, off);
             t.holes = __ballot(!ok);
         }
         f32x16 sc[2][NB];
@@ -186,8 +262,7 @@ struct GenericAttn : TileMath<HD, NB, kWaves> {
         this->accumulate(v_stage(buf), pb);
     }
 
-    DFX_D void run_segment(int rt, int tile0, int tile1, int item_tiles, int64_t item_begin, const WgSplit& split,
-                           int slot) {
+    DFX_D void run_segment(int rt, int tile0, int tile1, int item_tiles, int64_t item_begin, const WgSplit& split) {
         const bool complete = tile0 == 0 && tile1 == item_tiles;
         this->load_queries(rt);
         __syncthreads();  // the previous segment's last tile and block-table entries may still be read from LDS
@@ -210,11 +285,11 @@ struct GenericAttn : TileMath<HD, NB, kWaves> {
     }
 };
 
-template <int HD, int NB, bool FP8>
+template <int HD, int NB, bool FP8, bool DISTINCT = false>
 __global__ void __launch_bounds__(kThreads) paged_attn_generic_kernel(const KArgs a) {
     extern __shared__ __attribute__((aligned(256))) uint8_t smem[];
-    GenericAttn<HD, NB, FP8> at(a, smem);
-    store_fresh_rows<HD, FP8>(a);
+    GenericAttn<HD, NB, FP8, DISTINCT> at(a, smem);
+    if constexpr (!DISTINCT) store_fresh_rows<HD, FP8>(a);
     const UnitSummary summary = build_unit_prefix<Shape<HD, NB>::RT>(a, at.prefix, at.misc);
     const int per_head = summary.per_head;
     const int64_t total = static_cast<int64_t>(per_head) * a.h_kv;
@@ -240,7 +315,7 @@ __global__ void __launch_bounds__(kThreads) paged_attn_generic_kernel(const KArg
         locate_unit(at.sh, u, rt, tile0, n_tiles);
         const int64_t seg_end = min(pos + (n_tiles - tile0), end);
         const int tile1 = tile0 + static_cast<int>(seg_end - pos);
-        at.run_segment(rt, tile0, tile1, n_tiles, pos - tile0, split, partial_slot(w, pos, begin));
+        at.run_segment(rt, tile0, tile1, n_tiles, pos - tile0, split);
         u += tile1 - tile0;
         pos = seg_end;
         if (pos >= end) break;

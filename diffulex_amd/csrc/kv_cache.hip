@@ -94,6 +94,87 @@ kv_store_distinct_kernel(const uint16_t* __restrict__ key, const uint16_t* __res
     v_cache[blk * st.v[0] + h * st.v[1] + d * st.v[2] + off * st.v[3]] = value[t * value_stride + e];
 }
 
+// The same store for x == 8 two-byte elements and dense inner dimensions, 64 tokens of one head per
+// workgroup, staged through LDS so that both sides move 16 bytes per lane: rows are read the way
+// they lie in the operands (256 contiguous bytes per token and head), K leaves as one chunk
+// column of consecutive tokens (their 16-byte pieces are adjacent in the cache when their slots
+// are), and V leaves transposed, eight consecutive tokens of one d per store where those eight
+// have consecutive slots starting at a multiple of 8 in one page (two bytes at a time otherwise).
+constexpr int kDistinctTokens = 64;
+
+template <typename SlotT, int HD>
+__global__ void __launch_bounds__(kThreads)
+kv_store_distinct_tiled(const uint16_t* __restrict__ key, const uint16_t* __restrict__ value, int64_t key_stride,
+                        int64_t value_stride, uint16_t* __restrict__ k_cache, uint16_t* __restrict__ v_cache,
+                        DistinctStrides st, const SlotT* __restrict__ slots, int64_t n_tokens, int64_t n_pages,
+                        int page_size) {
+    constexpr int CPR = HD / 8;             // 16-byte chunks per row
+    constexpr int VPITCH = HD * 2 + 4;      // V rows padded by one word: column reads then spread over the banks
+    __shared__ __attribute__((aligned(16))) uint8_t k_tile[kDistinctTokens * HD * 2];
+    __shared__ __attribute__((aligned(16))) uint8_t v_tile[kDistinctTokens * VPITCH];
+    __shared__ int64_t slot_of[kDistinctTokens];
+    const int64_t t0 = static_cast<int64_t>(blockIdx.x) * kDistinctTokens;
+    const int h = blockIdx.y;
+    const int tid = threadIdx.x;
+    if (tid < kDistinctTokens) {
+        const int64_t t = t0 + tid;
+        int64_t slot = t < n_tokens ? static_cast<int64_t>(slots[t]) : -1;
+        if (slot >= 0 && slot / page_size >= n_pages) slot = -1;
+        slot_of[tid] = slot;
+    }
+    for (int c = tid; c < kDistinctTokens * CPR; c += kThreads) {
+        const int r = c / CPR, cc = c % CPR;
+        const int64_t t = t0 + r;
+        u32x4 kk = {0, 0, 0, 0}, vv = {0, 0, 0, 0};
+        if (t < n_tokens) {
+            kk = *reinterpret_cast<const u32x4*>(key + t * key_stride + h * HD + cc * 8);
+            vv = *reinterpret_cast<const u32x4*>(value + t * value_stride + h * HD + cc * 8);
+        }
+        *reinterpret_cast<u32x4*>(k_tile + r * (HD * 2) + ((cc ^ (r % CPR)) * 16)) = kk;
+        uint32_t* vrow = reinterpret_cast<uint32_t*>(v_tile + r * VPITCH + cc * 16);
+        vrow[0] = vv.x; vrow[1] = vv.y; vrow[2] = vv.z; vrow[3] = vv.w;
+    }
+    __syncthreads();
+    // K: consecutive lanes take consecutive tokens of one chunk column
+    for (int c = tid; c < kDistinctTokens * CPR; c += kThreads) {
+        const int r = c % kDistinctTokens, cc = c / kDistinctTokens;
+        const int64_t slot = slot_of[r];
+        if (slot < 0) continue;
+        const int64_t blk = slot / page_size, off = slot - blk * page_size;
+        const u32x4 kk = *reinterpret_cast<const u32x4*>(k_tile + r * (HD * 2) + ((cc ^ (r % CPR)) * 16));
+        *reinterpret_cast<u32x4*>(k_cache + blk * st.k[0] + h * st.k[1] + cc * st.k[2] + off * 8) = kk;
+    }
+    // V: eight consecutive lanes take the eight 8-token groups of one d
+    for (int c = tid; c < (kDistinctTokens / 8) * HD; c += kThreads) {
+        const int tg = c % (kDistinctTokens / 8), d = c / (kDistinctTokens / 8);
+        const int r0 = tg * 8;
+        uint16_t e[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) e[j] = *reinterpret_cast<const uint16_t*>(v_tile + (r0 + j) * VPITCH + d * 2);
+        const int64_t s0 = slot_of[r0];
+        bool run = s0 >= 0 && (s0 % 8) == 0 && (s0 % page_size) + 8 <= page_size;
+#pragma unroll
+        for (int j = 1; j < 8; ++j) run = run && slot_of[r0 + j] == s0 + j;
+        if (run) {
+            const int64_t blk = s0 / page_size, off = s0 - blk * page_size;
+            u32x4 w;
+            w.x = e[0] | (static_cast<uint32_t>(e[1]) << 16);
+            w.y = e[2] | (static_cast<uint32_t>(e[3]) << 16);
+            w.z = e[4] | (static_cast<uint32_t>(e[5]) << 16);
+            w.w = e[6] | (static_cast<uint32_t>(e[7]) << 16);
+            *reinterpret_cast<u32x4*>(v_cache + blk * st.v[0] + h * st.v[1] + d * st.v[2] + off) = w;
+        } else {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const int64_t slot = slot_of[r0 + j];
+                if (slot < 0) continue;
+                const int64_t blk = slot / page_size, off = slot - blk * page_size;
+                v_cache[blk * st.v[0] + h * st.v[1] + d * st.v[2] + off] = e[j];
+            }
+        }
+    }
+}
+
 // ---------------------------------------------------------------- load (gather)
 // grid = (row blocks, sequences).  A block copies kRowsPerBlock consecutive output rows of
 // one sequence; each lane moves 16 output bytes of K and of V per step.
@@ -221,8 +302,25 @@ extern "C" int dfx_kv_store_distinct(const void* key, const void* value, int64_t
     for (int i = 0; i < 5; ++i) ds.k[i] = kc_stride[i];
     for (int i = 0; i < 4; ++i) ds.v[i] = vc_stride[i];
     hipStream_t st = static_cast<hipStream_t>(stream);
+    // 16-byte moves on both sides where the shapes allow (x == 8, dense inner dimensions, aligned)
+    const bool tiled = x == 8 && (head_dim == 64 || head_dim == 128) && ds.k[4] == 1 && ds.k[3] == 8 && ds.v[3] == 1 &&
+                       ds.k[0] % 8 == 0 && ds.k[1] % 8 == 0 && ds.k[2] % 8 == 0 && ds.v[0] % 8 == 0 &&
+                       ds.v[1] % 8 == 0 && ds.v[2] % 8 == 0 && key_stride % 8 == 0 && value_stride % 8 == 0 &&
+                       aligned16(key) && aligned16(value) && aligned16(k_cache) && aligned16(v_cache) &&
+                       n_kv_heads <= 65535;
     return with_slot_type(slot_index_type, [&](auto* tag) {
         using SlotT = std::remove_const_t<std::remove_pointer_t<decltype(tag)>>;
+        if (tiled) {
+            const int64_t tiles = (n_tokens + kDistinctTokens - 1) / kDistinctTokens;
+            if (tiles > INT32_MAX) return static_cast<int>(DFX_ERR_UNSUPPORTED);
+            const dim3 grid(static_cast<unsigned>(tiles), static_cast<unsigned>(n_kv_heads));
+            auto kern = head_dim == 128 ? kv_store_distinct_tiled<SlotT, 128> : kv_store_distinct_tiled<SlotT, 64>;
+            hipLaunchKernelGGL(kern, grid, dim3(kThreads), 0, st, static_cast<const uint16_t*>(key),
+                               static_cast<const uint16_t*>(value), key_stride, value_stride,
+                               static_cast<uint16_t*>(k_cache), static_cast<uint16_t*>(v_cache), ds,
+                               static_cast<const SlotT*>(slot_mapping), n_tokens, n_pages, page_size);
+            return launch_status();
+        }
         const int64_t blocks = (n_tokens * row + kThreads - 1) / kThreads;
         if (blocks > INT32_MAX) return static_cast<int>(DFX_ERR_UNSUPPORTED);
         hipLaunchKernelGGL((kv_store_distinct_kernel<SlotT>), dim3(static_cast<unsigned>(blocks)), dim3(kThreads), 0,

@@ -31,6 +31,7 @@ struct Plan {
     int hd, nb, n_wg;
     bool fp8;
     bool stream;   // streaming tile path (else generic)
+    bool distinct; // the cache is in the "distinct" layout (generic path)
     bool compact;  // streaming path, two workgroups per compute unit
     bool pipelined;  // streaming path, bf16 KV, 4-stage ring: software-pipelined tile step
     int64_t slot_floats;
@@ -63,7 +64,10 @@ int make_plan(const dfx_attn_params* p, Plan& plan) {
     plan.fp8 = p->kv_dtype == DFX_KV_FP8_E4M3 && p->k_cache != nullptr;
     // The streaming path addresses a K row and its V row with one offset: page size a multiple
     // of 16, fresh K and V laid out alike.  FP8 streaming exists for head_dim 128.
-    plan.stream = !(p->flags & DFX_ATTN_GENERIC_PATH) &&
+    plan.distinct = p->cache_layout == DFX_CACHE_DISTINCT && p->k_cache != nullptr;
+    if (p->cache_layout != DFX_CACHE_UNIFIED && p->cache_layout != DFX_CACHE_DISTINCT) return DFX_ERR_INVALID_ARG;
+    if (plan.distinct && plan.fp8) return DFX_ERR_UNSUPPORTED;
+    plan.stream = !(p->flags & DFX_ATTN_GENERIC_PATH) && !plan.distinct &&
                   (p->k_cache == nullptr || (p->page_size > 0 && p->page_size % 16 == 0)) &&
                   p->kn_stride_token == p->vn_stride_token && p->kn_stride_head == p->vn_stride_head &&
                   (!plan.fp8 || p->head_dim == 128);
@@ -107,7 +111,7 @@ bool ensure_lds_limit(const void* kernel, int slot, int lds) {
     return true;
 }
 
-// PATH: 0 generic bf16, 1 generic FP8, 2 streaming bf16, 3 streaming FP8.
+// PATH: 0 generic bf16, 1 generic FP8, 2 streaming bf16, 3 streaming FP8, 4 generic bf16 on a distinct-layout cache.
 // pa == nullptr: the attention launch.  Otherwise the two plan kernels for that launch (streaming
 // paths only).
 template <int HD, int NB, int PATH>
@@ -154,6 +158,10 @@ int launch(const KArgs& ka, const Plan& plan, hipStream_t st, const PlanArgs* pa
             fill_lds = C::STAGES_OFF;
         }
         threads = 64 * NW;
+    } else if constexpr (PATH == 4) {
+        main_k = paged_attn_generic_kernel<HD, NB, false, true>;
+        lds = GenericCfg<HD, NB>::LDS_BYTES;
+        slot = 24 + kSlotBase / 4;
     } else {
         main_k = paged_attn_generic_kernel<HD, NB, PATH == 1>;
         lds = GenericCfg<HD, NB>::LDS_BYTES;
@@ -220,7 +228,15 @@ int check_args(const dfx_attn_params* p, Plan& plan, bool& empty) {
     if (p->o_stride_token % 4 != 0 || p->o_stride_head % 4 != 0) return DFX_ERR_INVALID_ARG;
     if (!aligned16(p->q) || !aligned16(p->k_new) || !aligned16(p->v_new) || !aligned16(p->out))
         return DFX_ERR_INVALID_ARG;
-    if (has_cache) {
+    if (plan.distinct) {
+        // 16-byte loads: x == 8 two-byte elements, tokens dense in V, everything else a multiple of 8
+        if (p->kc_stride[4] != 1 || p->kc_stride[3] != 8 || p->vc_stride[3] != 1) return DFX_ERR_UNSUPPORTED;
+        if (p->page_size % 8 != 0) return DFX_ERR_UNSUPPORTED;
+        for (int i = 0; i < 3; ++i)
+            if (p->kc_stride[i] < 0 || p->kc_stride[i] % 8 || p->vc_stride[i] < 0 || p->vc_stride[i] % 8) return DFX_ERR_INVALID_ARG;
+        if (p->store_slot_mapping != nullptr) return DFX_ERR_UNSUPPORTED;  // dfx_kv_store_distinct stores into this layout
+        if (!aligned16(p->k_cache) || !aligned16(p->v_cache)) return DFX_ERR_INVALID_ARG;
+    } else if (has_cache) {
         const int64_t gran = plan.fp8 ? 16 : 8;
         if (p->cache_stride_page % gran || p->cache_stride_token % gran || p->cache_stride_head % gran)
             return DFX_ERR_INVALID_ARG;
@@ -310,6 +326,8 @@ int run_paged_attn(const dfx_attn_params* p, void* workspace, int64_t workspace_
     ka.c_sp = p->cache_stride_page;
     ka.c_st = p->cache_stride_token;
     ka.c_sh = p->cache_stride_head;
+    ka.kd_sp = p->kc_stride[0]; ka.kd_sh = p->kc_stride[1]; ka.kd_sc = p->kc_stride[2];
+    ka.vd_sp = p->vc_stride[0]; ka.vd_sh = p->vc_stride[1]; ka.vd_sd = p->vc_stride[2];
     ka.bt_stride = p->block_table_stride;
     ka.n_pages = p->n_pages;
     ka.num_seqs = p->num_seqs;
@@ -348,6 +366,7 @@ int run_paged_attn(const dfx_attn_params* p, void* workspace, int64_t workspace_
             if constexpr (HD_ == 128) return launch<HD_, NB_, 3>(ka, plan, st, pap); \
         }                                                                     \
         if (plan.stream) return launch<HD_, NB_, 2>(ka, plan, st, pap);       \
+        if (plan.distinct) return launch<HD_, NB_, 4>(ka, plan, st, pap);     \
         if (plan.fp8) return launch<HD_, NB_, 1>(ka, plan, st, pap);          \
         return launch<HD_, NB_, 0>(ka, plan, st, pap);                        \
     }

@@ -58,7 +58,8 @@ def _workspace(device: torch.device, stream: int, nbytes: int) -> torch.Tensor:
 def paged_attention(q, k, v, k_cache, v_cache, scale, *, block_tables, context_lens, cu_seqlens_q,
                     cu_seqlens_new, max_seqlen_q, mask_mode=_lib.DFX_MASK_FULL, diffusion_block_size=32,
                     k_scale=None, v_scale=None, max_workgroups=0, out=None, flags=0,
-                    store_slot_mapping=None, static_scratch=False, plan_cache=None) -> torch.Tensor:
+                    store_slot_mapping=None, static_scratch=False, plan_cache=None,
+                    cache_layout="unified") -> torch.Tensor:
     """Marshal tensors into ``dfx_attn_params`` and launch ``dfx_paged_attn`` on the
     current stream.  q: [T, H_q, hd]; k, v: [T_new, H_kv, hd]; caches
     [pages, page, H_kv, hd] or None.  ``store_slot_mapping`` ([T_new] int32/int64): the same
@@ -71,7 +72,9 @@ def paged_attention(q, k, v, k_cache, v_cache, scale, *, block_tables, context_l
     the workgroups, page address of every tile) is built on the first call and reused by later
     calls with the same dict -- the attention layers of one decoding step, whose lengths and block
     tables are the same.  In-place updates of those tensors and graph captures are noticed (they
-    change the cache key); a caller that rewrites them behind PyTorch's back drops the dict."""
+    change the cache key); a caller that rewrites them behind PyTorch's back drops the dict.
+    ``cache_layout="distinct"``: k_cache [pages, H_kv, hd / 8, page, 8], v_cache [pages, H_kv, hd,
+    page] (what ``store_kvcache_distinct_layout`` writes); bf16, generic tile path, no fused store."""
     lib = _lib.load()
     assert q.is_cuda and q.dtype == torch.bfloat16 and k.dtype == torch.bfloat16 and v.dtype == torch.bfloat16
     assert q.dim() == 3 and k.dim() == 3 and v.shape == k.shape
@@ -88,7 +91,29 @@ def paged_attention(q, k, v, k_cache, v_cache, scale, *, block_tables, context_l
     p = _lib.AttnParams()
     keep = ()
     has_cache = k_cache is not None and k_cache.numel() > 0
-    if has_cache:
+    distinct = cache_layout == "distinct"
+    assert cache_layout in ("unified", "distinct")
+    if has_cache and distinct:
+        assert k_cache.dim() == 5 and v_cache.dim() == 4 and k_cache.dtype == torch.bfloat16 == v_cache.dtype
+        n_pages, _, _, page, x = k_cache.shape
+        assert k_cache.shape[1] == H_kv and k_cache.shape[2] * x == hd and x == 8
+        assert v_cache.shape == (n_pages, H_kv, hd, page)
+        assert store_slot_mapping is None, "the distinct layout has a store launch of its own"
+        plan_cache = None
+    if has_cache and distinct:
+        assert block_tables is not None and block_tables.dtype == torch.int32 and block_tables.stride(-1) == 1
+        assert context_lens is not None and context_lens.dtype == torch.int32 and context_lens.is_contiguous()
+        assert block_tables.shape[0] == num_seqs and context_lens.numel() == num_seqs
+        p.k_cache, p.v_cache = k_cache.data_ptr(), v_cache.data_ptr()
+        p.block_tables, p.context_lens = block_tables.data_ptr(), context_lens.data_ptr()
+        p.block_table_stride = block_tables.stride(0)
+        p.n_pages, p.page_size = k_cache.shape[0], k_cache.shape[3]
+        p.max_pages_per_seq = block_tables.shape[1]
+        p.kv_dtype = _lib.DFX_KV_BF16
+        p.cache_layout = _lib.DFX_CACHE_DISTINCT
+        p.kc_stride = (C.c_int64 * 5)(*k_cache.stride())
+        p.vc_stride = (C.c_int64 * 4)(*v_cache.stride())
+    elif has_cache:
         assert k_cache.shape == v_cache.shape and k_cache.dim() == 4
         assert k_cache.shape[2] == H_kv and k_cache.shape[3] == hd
         assert k_cache.stride() == v_cache.stride() and k_cache.stride(-1) == 1
@@ -211,9 +236,12 @@ def dllm_flash_attn_decode(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, k_
                            v_cache: torch.Tensor, scale: float, attn_metadata,
                            k_scale: Optional[torch.Tensor] = None,
                            v_scale: Optional[torch.Tensor] = None,
-                           store_slot_mapping: Optional[torch.Tensor] = None) -> torch.Tensor:
+                           store_slot_mapping: Optional[torch.Tensor] = None,
+                           kv_cache_layout: str = "unified") -> torch.Tensor:
     """dllm_flash_attn.py:599-637.  ``store_slot_mapping`` (extension): also store the fresh
     K/V rows into these cache slots in the same launch (see ``paged_attention``).
+    ``kv_cache_layout="distinct"`` (extension): the caches are in the layout
+    ``store_kvcache_distinct_layout`` writes.
 
     ``decode_mode == "static"``: ``cu_seqlens_k`` indexes the fresh K/V rows
     (strategy/block_diffusion/engine/model_runner.py:134-139).
@@ -233,6 +261,12 @@ def dllm_flash_attn_decode(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, k_
     mask = _lib.DFX_MASK_FULL
     if getattr(attn_metadata, "decode_mask", "full") == "block_causal":
         mask = _lib.DFX_MASK_BLOCK_CAUSAL
+    if kv_cache_layout == "distinct":
+        return paged_attention(
+            q, k, v, k_cache, v_cache, scale, block_tables=attn_metadata.block_tables,
+            context_lens=attn_metadata.context_lens, cu_seqlens_q=attn_metadata.cu_seqlens_q,
+            cu_seqlens_new=cu_new, max_seqlen_q=_max_seqlen_q(attn_metadata, attn_metadata.cu_seqlens_q),
+            mask_mode=mask, diffusion_block_size=attn_metadata.diffusion_block_size, cache_layout="distinct")
     if k_cache.dtype in _FP8_DTYPES:
         k_scale = k_scale if k_scale is not None else getattr(attn_metadata, "k_scale", None)
         v_scale = v_scale if v_scale is not None else getattr(attn_metadata, "v_scale", None)

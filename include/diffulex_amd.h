@@ -42,6 +42,8 @@ typedef enum dfx_mask_mode {
     DFX_MASK_BLOCK_CAUSAL = 1 /* fresh token j visible to query i iff j < (i / dbs + 1) * dbs */
 } dfx_mask_mode;
 
+typedef enum dfx_cache_layout { DFX_CACHE_UNIFIED = 0, DFX_CACHE_DISTINCT = 1 } dfx_cache_layout;
+
 typedef enum dfx_index_type { DFX_INDEX_I32 = 0, DFX_INDEX_I64 = 1 } dfx_index_type;
 
 /* dfx_attn_params.flags */
@@ -196,6 +198,18 @@ typedef struct dfx_attn_params {
      * reference's graph-capture metadata, carry such offsets).  0: unknown, the offsets are trusted;
      * required (> 0) with store_slot_mapping. */
     int64_t num_new_tokens;
+    /* Layout of k_cache / v_cache.  DFX_CACHE_UNIFIED (0): [pages, page_size, H_kv, head_dim] through
+     * cache_stride_*.  DFX_CACHE_DISTINCT: the layout dfx_kv_store_distinct writes, K [pages, H_kv,
+     * head_dim / 8, page_size, 8] and V [pages, H_kv, head_dim, page_size], bf16, through the element
+     * strides below (kc_stride[3] == 8, kc_stride[4] == 1, vc_stride[3] == 1, the others multiples of
+     * 8; page_size a multiple of 8).  The reference stores into this layout
+     * (diffulex_kernel/python/kv_cache_kernels.py:35-83) but its decode refuses it
+     * (diffulex/attention/attn_impl.py:66-69); here it runs on the generic tile path.  No fused store,
+     * no FP8, no plan with it. */
+    int32_t cache_layout;
+    int32_t reserved1;
+    int64_t kc_stride[5];
+    int64_t vc_stride[4];
 } dfx_attn_params;
 
 /* Bytes of scratch dfx_paged_attn needs for these shapes (depends on the sizes

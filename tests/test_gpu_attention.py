@@ -207,10 +207,70 @@ def test_attention_module_store_then_decode(dev):
     assert max_abs_err(o.view(t, wl.num_q_heads, wl.head_dim), want) <= ATOL_BF16
     slots = wl.slot_mapping.long()
     assert torch.equal(kc.view(-1, wl.num_kv_heads, wl.head_dim)[slots], wl.k_new)
+
+
+def _to_distinct(cache, x=8):
+    """[pages, page, H, hd] -> K [pages, H, hd / x, page, x] and V [pages, H, hd, page], the
+    rearrangement the reference's layout check spells out (examples: 'b h n s x -> b s h (n x)')."""
+    pages, page, h, hd = cache.shape
+    k = cache.view(pages, page, h, hd // x, x).permute(0, 2, 3, 1, 4).contiguous()
+    v = cache.permute(0, 2, 3, 1).contiguous()
+    return k, v
+
+
+@pytest.mark.parametrize("name,over", [
+    ("c1", dict(page=16)),
+    ("c1", dict(num_seqs=3, ctx=[100, 0, 37], page=8)),
+    ("c3", dict(num_seqs=5, ctx=(50, 900), page=32)),
+    ("c3", dict(num_seqs=3, ctx=[700, 513, 1000])),
+    ("c4", dict(num_seqs=2, ctx=[300, 95], page=48)),
+    ("c3", dict(num_seqs=4, ctx=(100, 600), h_q=8, h_kv=2, hd=64, page=64)),
+])
+@pytest.mark.parametrize("max_wg", [0, 3])
+def test_decode_on_the_distinct_cache_layout(dev, name, over, max_wg):
+    """The reference stores into the distinct layout but refuses to decode from it
+    (diffulex/attention/attn_impl.py:66-69); here the same attention runs on it: equal, bit for
+    bit, to the generic path on the unified cache holding the same values, and within tolerance
+    of the oracle.  Skipped pages (negative table entries) behave alike."""
+    wl = make_workload(name, seed=89, **over)
+    bt = wl.block_tables.clone()
+    if wl.num_seqs > 2:
+        bt[2, 1] = -1
+        wl.block_tables = bt
+    want = oracle_fp32(wl)
+    g = wl.to(dev)
+    kd = _to_distinct(g.k_cache)[0]
+    vd = _to_distinct(g.v_cache)[1]
+    args = dict(block_tables=g.block_tables, context_lens=g.context_lens, cu_seqlens_q=g.cu_seqlens_q,
+                cu_seqlens_new=g.cu_seqlens_q, max_seqlen_q=g.q_len, mask_mode=g.mask_mode,
+                diffusion_block_size=g.diffusion_block_size, max_workgroups=max_wg)
+    got = dfx.paged_attention(g.q, g.k_new, g.v_new, kd, vd, g.scale, cache_layout="distinct", **args)
+    same = dfx.paged_attention(g.q, g.k_new, g.v_new, g.k_cache, g.v_cache, g.scale, flags=GENERIC, **args)
+    torch.cuda.synchronize()
+    assert max_abs_err(got, want) <= ATOL_BF16
+    assert torch.equal(got, same)
+
+
+def test_attention_module_on_the_distinct_layout(dev):
+    """Attention.forward with kv_cache_layout == "distinct": store through
+    store_kvcache_distinct_layout, then decode from that cache."""
+    wl = make_workload("c3", seed=91, num_seqs=4, ctx=(100, 700), page=32).to(dev)
+    want = oracle_fp32(wl)
+    att = dfx.Attention(wl.num_q_heads, wl.head_dim, wl.scale, wl.num_kv_heads)
+    att.k_cache, att.v_cache = _to_distinct(wl.k_cache)[0], _to_distinct(wl.v_cache)[1]
+    md = metadata_for(wl, "static")
     md.kv_cache_layout = "distinct"
-    md.need_kv_cache_store = False
-    with pytest.raises(NotImplementedError):
-        att(wl.q.reshape(t, -1), wl.k_new.reshape(t, -1), wl.v_new.reshape(t, -1))
+    dfx.set_fetch_fn_for_attn_metadata(lambda: md)
+    t = wl.q.shape[0]
+    o = att(wl.q.reshape(t, -1), wl.k_new.reshape(t, -1), wl.v_new.reshape(t, -1))
+    torch.cuda.synchronize()
+    assert max_abs_err(o.view(t, wl.num_q_heads, wl.head_dim), want) <= ATOL_BF16
+    # the block was stored where the slot mapping says
+    ku = att.k_cache.permute(0, 3, 1, 2, 4).reshape(wl.k_cache.shape)
+    vu = att.v_cache.permute(0, 3, 1, 2)
+    slots = wl.slot_mapping.long()
+    assert torch.equal(ku.reshape(-1, wl.num_kv_heads, wl.head_dim)[slots], wl.k_new)
+    assert torch.equal(vu.reshape(-1, wl.num_kv_heads, wl.head_dim)[slots], wl.v_new)
 
 
 def test_invariants_at_full_c3_size(dev):

@@ -114,6 +114,44 @@ def test_store_distinct_bit_exact_and_rearrangement_identity(dev):
     assert torch.equal(vd2.permute(0, 3, 1, 2), vu)
 
 
+@pytest.mark.parametrize("hd,h,page,x,scatter", [
+    (128, 4, 64, 8, False), (128, 4, 64, 8, True), (64, 2, 32, 8, True), (128, 3, 16, 8, True),
+    (128, 4, 64, 4, True),      # x != 8: the element-wise kernel
+    (96, 2, 32, 8, True),       # head_dim the tiled kernel has no variant for
+])
+def test_store_distinct_tiled_and_elementwise_kernels(dev, hd, h, page, x, scatter):
+    """Both kernels behind dfx_kv_store_distinct against the CPU restatement: slots in runs (a
+    block stored into its pages) and scattered one by one, skipped rows, rows beyond the cache."""
+    g = torch.Generator().manual_seed(hd + page + x)
+    n = 201
+    pages = max(7, -(-n // page) + 2)
+    key = torch.randn(n, h, hd, generator=g).to(torch.bfloat16)
+    value = torch.randn(n, h, hd, generator=g).to(torch.bfloat16)
+    if scatter:
+        slots = torch.randperm(pages * page, generator=g)[:n].to(torch.int32)
+    else:
+        slots = (torch.arange(n, dtype=torch.int32) + 40)
+    slots[5::9] = -1
+    kd0 = _sentinel_like(torch.empty(pages, h, hd // x, page, x, dtype=torch.bfloat16))
+    vd0 = _sentinel_like(torch.empty(pages, h, hd, page, dtype=torch.bfloat16))
+    want_k, want_v = kd0.clone(), vd0.clone()
+    okv.store_distinct(key, value, want_k, want_v, slots)
+    for slot_dtype in (torch.int32, torch.int64):
+        kd, vd = kd0.to(dev), vd0.to(dev)
+        s = slots.to(slot_dtype).clone()
+        dfx.store_kvcache_distinct_layout(key.to(dev), value.to(dev), kd, vd, s.to(dev), None)
+        assert torch.equal(_bits(kd), _bits(want_k)) and torch.equal(_bits(vd), _bits(want_v))
+    # a slot beyond the cache is skipped
+    s = slots.clone()
+    s[0] = pages * page + 3
+    s0 = slots.clone()
+    s0[0] = -1
+    okv.store_distinct(key, value, (wk := kd0.clone()), (wv := vd0.clone()), s0)
+    kd, vd = kd0.to(dev), vd0.to(dev)
+    dfx.store_kvcache_distinct_layout(key.to(dev), value.to(dev), kd, vd, s.to(dev), None)
+    assert torch.equal(_bits(kd), _bits(wk)) and torch.equal(_bits(vd), _bits(wv))
+
+
 @pytest.mark.parametrize("name,over", [
     ("c1", {}), ("c2", {}),
     ("c2", dict(num_seqs=5, page=32, ctx=[0, 32, 64, 33, 500], hd=64, h_kv=2, h_q=2)),   # exact page multiples

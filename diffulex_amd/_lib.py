@@ -139,6 +139,26 @@ def load() -> C.CDLL:
     return lib
 
 
+OPS_PATH = LIB_PATH.parent / "_torch_ops.so"
+_ops = None
+
+
+def ops():
+    """``torch.ops.diffulex_amd``: the operator library that binds the C ABI to PyTorch tensors
+    and streams (csrc/torch_ext.cpp).  The Python operators go through it; ``load()`` above (ctypes)
+    is the direct view of the same C functions."""
+    global _ops
+    if _ops is None:
+        import torch
+        if not OPS_PATH.exists():
+            raise ImportError(f"{OPS_PATH} is missing: build it first (python -m diffulex_amd.build). "
+                              "diffulex_amd has no fallback path.")
+        load()  # checks the ABI version of the kernel library the operator library links to
+        torch.ops.load_library(str(OPS_PATH))
+        _ops = torch.ops.diffulex_amd
+    return _ops
+
+
 def check(status: int, what: str) -> None:
     if status != DFX_OK:
         msg = load().dfx_status_string(int(status)).decode()

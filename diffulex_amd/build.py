@@ -1,9 +1,12 @@
-"""Build libdiffulex_amd.so (the C-ABI library with the gfx950 kernels) in-tree.
+"""Build libdiffulex_amd.so (the C-ABI library with the gfx950 kernels) and _torch_ops.so (the
+PyTorch operator library that binds it) in-tree.
 
     python -m diffulex_amd.build
 
-compiles every source under ``csrc/`` with hipcc for gfx950 and links them into
-``diffulex_amd/libdiffulex_amd.so``.  hipcc cross-compiles, so no GPU is needed.
+compiles every kernel source under ``csrc/`` with hipcc for gfx950 and links them into
+``diffulex_amd/libdiffulex_amd.so``, then compiles ``csrc/torch_ext.cpp`` (host code) against
+PyTorch's headers into ``diffulex_amd/_torch_ops.so``, which finds the kernel library next to
+itself.  hipcc cross-compiles, so no GPU is needed.
 """
 from __future__ import annotations
 
@@ -17,6 +20,7 @@ from pathlib import Path
 PKG_DIR = Path(__file__).resolve().parent
 CSRC = PKG_DIR / "csrc"
 LIB_PATH = PKG_DIR / "libdiffulex_amd.so"
+OPS_PATH = PKG_DIR / "_torch_ops.so"
 ARCH = "gfx950"
 
 # packed-fp32 instructions are kept out of the generated code on purpose
@@ -69,7 +73,28 @@ def build(verbose: bool = True) -> Path:
     os.replace(tmp, LIB_PATH)
     if verbose:
         print(f"built {LIB_PATH} ({LIB_PATH.stat().st_size} bytes)")
+    build_torch_ops(verbose)
     return LIB_PATH
+
+
+def build_torch_ops(verbose: bool = True) -> Path:
+    """The TORCH_LIBRARY module: host C++ only, linked against PyTorch and libdiffulex_amd.so."""
+    import torch
+    from torch.utils import cpp_extension
+    torch_lib = Path(torch.__file__).resolve().parent / "lib"
+    tmp = OPS_PATH.with_suffix(".so.tmp")
+    cmd = [_hipcc(), "-O2", "-std=c++17", "-fPIC", "-shared", "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1",
+           f"-D_GLIBCXX_USE_CXX11_ABI={int(torch._C._GLIBCXX_USE_CXX11_ABI)}",
+           *[f"-I{p}" for p in cpp_extension.include_paths("cuda")], str(CSRC / "torch_ext.cpp"), "-o", str(tmp),
+           f"-L{torch_lib}", "-ltorch", "-ltorch_cpu", "-lc10", "-lc10_hip", "-ltorch_hip",
+           f"-L{PKG_DIR}", f"-l:{LIB_PATH.name}", "-Wl,-rpath,$ORIGIN", f"-Wl,-rpath,{torch_lib}"]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError(f"hipcc failed for torch_ext.cpp:\n{res.stderr[-4000:]}")
+    os.replace(tmp, OPS_PATH)
+    if verbose:
+        print(f"built {OPS_PATH} ({OPS_PATH.stat().st_size} bytes)")
+    return OPS_PATH
 
 
 if __name__ == "__main__":

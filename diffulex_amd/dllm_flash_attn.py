@@ -7,13 +7,12 @@ the "varlen" mode needs no ``load_kvcache`` gather and no second pass over K/V.
 """
 from __future__ import annotations
 
-import ctypes as C
 from typing import Optional
 
 import torch
 
 from . import _lib
-from .kv_cache_kernels import _FP8_DTYPES, _index_type, _scales, _stream
+from .kv_cache_kernels import _FP8_DTYPES, _stream
 
 class _Workspace:
     __slots__ = ("tensor", "zeroed")
@@ -55,14 +54,17 @@ def _workspace(device: torch.device, stream: int, nbytes: int) -> torch.Tensor:
     return get((device.index, stream)).tensor
 
 
+_workspace_need = {}   # launch shape -> dfx_paged_attn_workspace_bytes
+
+
 def paged_attention(q, k, v, k_cache, v_cache, scale, *, block_tables, context_lens, cu_seqlens_q,
                     cu_seqlens_new, max_seqlen_q, mask_mode=_lib.DFX_MASK_FULL, diffusion_block_size=32,
                     k_scale=None, v_scale=None, max_workgroups=0, out=None, flags=0,
                     store_slot_mapping=None, static_scratch=False, plan_cache=None,
                     cache_layout="unified") -> torch.Tensor:
-    """Marshal tensors into ``dfx_attn_params`` and launch ``dfx_paged_attn`` on the
-    current stream.  q: [T, H_q, hd]; k, v: [T_new, H_kv, hd]; caches
-    [pages, page, H_kv, hd] or None.  ``store_slot_mapping`` ([T_new] int32/int64): the same
+    """Launch ``dfx_paged_attn`` on the current stream through ``torch.ops.diffulex_amd.paged_attention``
+    (which checks the tensors and fills ``dfx_attn_params``).  q: [T, H_q, hd]; k, v: [T_new, H_kv, hd];
+    caches [pages, page, H_kv, hd] or None.  ``store_slot_mapping`` ([T_new] int32/int64): the same
     launch also writes the fresh rows into those cache slots (what
     ``store_kvcache_unified_layout`` does in a launch of its own); the slots must lie outside
     every attended context.  ``static_scratch``: launch through ``dfx_paged_attn_static``, which
@@ -75,120 +77,72 @@ def paged_attention(q, k, v, k_cache, v_cache, scale, *, block_tables, context_l
     change the cache key); a caller that rewrites them behind PyTorch's back drops the dict.
     ``cache_layout="distinct"``: k_cache [pages, H_kv, hd / 8, page, 8], v_cache [pages, H_kv, hd,
     page] (what ``store_kvcache_distinct_layout`` writes); bf16, generic tile path, no fused store."""
-    lib = _lib.load()
-    assert q.is_cuda and q.dtype == torch.bfloat16 and k.dtype == torch.bfloat16 and v.dtype == torch.bfloat16
-    assert q.dim() == 3 and k.dim() == 3 and v.shape == k.shape
-    assert q.stride(-1) == 1 and k.stride(-1) == 1 and v.stride(-1) == 1
+    ops = _lib.ops()
     T, H_q, hd = q.shape
     H_kv = k.shape[1]
-    assert k.shape[2] == hd and H_q % H_kv == 0
     num_seqs = cu_seqlens_q.numel() - 1
-    assert cu_seqlens_new.numel() == num_seqs + 1
-    for t in (cu_seqlens_q, cu_seqlens_new):
-        assert t.dtype == torch.int32 and t.is_cuda and t.is_contiguous()
     if out is None:
         out = torch.empty((T, H_q, hd), dtype=q.dtype, device=q.device)
-    p = _lib.AttnParams()
-    keep = ()
     has_cache = k_cache is not None and k_cache.numel() > 0
-    distinct = cache_layout == "distinct"
     assert cache_layout in ("unified", "distinct")
-    if has_cache and distinct:
-        assert k_cache.dim() == 5 and v_cache.dim() == 4 and k_cache.dtype == torch.bfloat16 == v_cache.dtype
-        n_pages, _, _, page, x = k_cache.shape
-        assert k_cache.shape[1] == H_kv and k_cache.shape[2] * x == hd and x == 8
-        assert v_cache.shape == (n_pages, H_kv, hd, page)
-        assert store_slot_mapping is None, "the distinct layout has a store launch of its own"
-        plan_cache = None
-    if has_cache and distinct:
-        assert block_tables is not None and block_tables.dtype == torch.int32 and block_tables.stride(-1) == 1
-        assert context_lens is not None and context_lens.dtype == torch.int32 and context_lens.is_contiguous()
-        assert block_tables.shape[0] == num_seqs and context_lens.numel() == num_seqs
-        p.k_cache, p.v_cache = k_cache.data_ptr(), v_cache.data_ptr()
-        p.block_tables, p.context_lens = block_tables.data_ptr(), context_lens.data_ptr()
-        p.block_table_stride = block_tables.stride(0)
-        p.n_pages, p.page_size = k_cache.shape[0], k_cache.shape[3]
-        p.max_pages_per_seq = block_tables.shape[1]
-        p.kv_dtype = _lib.DFX_KV_BF16
-        p.cache_layout = _lib.DFX_CACHE_DISTINCT
-        p.kc_stride = (C.c_int64 * 5)(*k_cache.stride())
-        p.vc_stride = (C.c_int64 * 4)(*v_cache.stride())
-    elif has_cache:
-        assert k_cache.shape == v_cache.shape and k_cache.dim() == 4
-        assert k_cache.shape[2] == H_kv and k_cache.shape[3] == hd
-        assert k_cache.stride() == v_cache.stride() and k_cache.stride(-1) == 1
-        assert block_tables is not None and block_tables.dtype == torch.int32 and block_tables.stride(-1) == 1
-        assert context_lens is not None and context_lens.dtype == torch.int32 and context_lens.is_contiguous()
-        assert block_tables.shape[0] == num_seqs and context_lens.numel() == num_seqs
-        kv_dtype, ksp, vsp, keep = _scales(k_cache, None, k_scale, v_scale, H_kv)
-        p.k_cache, p.v_cache = k_cache.data_ptr(), v_cache.data_ptr()
-        p.block_tables, p.context_lens = block_tables.data_ptr(), context_lens.data_ptr()
-        p.k_scale, p.v_scale = ksp, vsp
-        p.cache_stride_page, p.cache_stride_token, p.cache_stride_head = k_cache.stride()[:3]
-        p.block_table_stride = block_tables.stride(0)
-        p.n_pages, p.page_size = k_cache.shape[0], k_cache.shape[1]
-        p.max_pages_per_seq = block_tables.shape[1]
-        p.kv_dtype = kv_dtype
-    else:
-        p.kv_dtype = _lib.DFX_KV_BF16
-    p.q, p.k_new, p.v_new, p.out = q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr()
-    p.cu_seqlens_q, p.cu_seqlens_new = cu_seqlens_q.data_ptr(), cu_seqlens_new.data_ptr()
-    p.q_stride_token, p.q_stride_head = q.stride(0), q.stride(1)
-    p.kn_stride_token, p.kn_stride_head = k.stride(0), k.stride(1)
-    p.vn_stride_token, p.vn_stride_head = v.stride(0), v.stride(1)
-    p.o_stride_token, p.o_stride_head = out.stride(0), out.stride(1)
-    p.num_seqs, p.num_q_heads, p.num_kv_heads, p.head_dim = num_seqs, H_q, H_kv, hd
-    p.num_new_tokens = k.shape[0]
-    p.max_seqlen_q = int(max_seqlen_q)
-    p.diffusion_block_size = int(diffusion_block_size)
-    p.mask_mode = int(mask_mode)
-    p.max_workgroups = int(max_workgroups)
-    p.flags = int(flags)
-    p.scale = float(scale)
+    distinct = cache_layout == "distinct"
+    fp8 = has_cache and not distinct and k_cache.dtype in _FP8_DTYPES
+    ks = vs = None
+    if fp8:
+        assert k_scale is not None and v_scale is not None, "an FP8 KV cache needs k_scale and v_scale"
+        ks = k_scale.to(device=q.device, dtype=torch.float32).contiguous()
+        vs = v_scale.to(device=q.device, dtype=torch.float32).contiguous()
+    if not has_cache:
+        k_cache = v_cache = block_tables = context_lens = None
     if store_slot_mapping is not None:
-        assert has_cache and store_slot_mapping.is_cuda and store_slot_mapping.is_contiguous()
         assert store_slot_mapping.numel() == k.shape[0], \
             f"`N`: {k.shape[0]}, `slot_mapping.numel()`: {store_slot_mapping.numel()}"
-        p.store_slot_mapping = store_slot_mapping.data_ptr()
-        p.store_slot_index_type = _index_type(store_slot_mapping)
-    stream = _stream()
-    if plan_cache is not None and has_cache:
+    layout = _lib.DFX_CACHE_DISTINCT if distinct else _lib.DFX_CACHE_UNIFIED
+    tail = (float(scale), int(max_seqlen_q), int(mask_mode), int(diffusion_block_size), int(max_workgroups),
+            int(flags), layout)
+    head = (q, k, v, k_cache, v_cache, out, block_tables, context_lens, cu_seqlens_q, cu_seqlens_new, ks, vs,
+            store_slot_mapping)
+    plan = None
+    if plan_cache is not None and has_cache and not distinct:
         # A plan is only as good as the lengths and tables it was made from: the key carries the
         # tensors' version counters (any in-place update makes a new key) and the graph capture the
         # call is recorded into (a plan built outside that capture is not part of its graph).
         meta = (block_tables, context_lens, cu_seqlens_q, cu_seqlens_new)
-        key = (H_q, H_kv, hd, int(p.kv_dtype), int(mask_mode), int(diffusion_block_size), int(max_seqlen_q), int(flags),
-               int(max_workgroups), k.stride(0), k.stride(1), k_cache.stride()[:3], num_seqs,
-               tuple((t.data_ptr(), t._version) for t in meta), int(lib.dfx_stream_capture_id(stream)))
+        key = (H_q, H_kv, hd, fp8, tail[1:], k.stride(0), k.stride(1), k_cache.stride()[:3], num_seqs,
+               tuple((t.data_ptr(), t._version) for t in meta), int(ops.stream_capture_id()))
         plan = plan_cache.get(key, False)
         if plan is False:
-            plan = _build_plan(lib, p, q.device, stream, H_q // H_kv, k.shape[0])
-            plan_cache[key] = plan
-        if plan is not None:
-            p.plan, p.plan_bytes = plan.data_ptr(), plan.numel()
-    if static_scratch:
-        _lib.check(lib.dfx_paged_attn_static(C.byref(p), stream), "dfx_paged_attn_static")
-        return out
-    need = lib.dfx_paged_attn_workspace_bytes(C.byref(p))
-    if need < 0:
-        _lib.check(int(need), "dfx_paged_attn_workspace_bytes")
-    ws = _workspace(q.device, stream, int(need))
-    p.workspace, p.workspace_bytes = ws.data_ptr(), ws.numel()
-    _lib.check(lib.dfx_paged_attn(C.byref(p), stream), "dfx_paged_attn")
+            plan = plan_cache[key] = _build_plan(ops, head, tail, H_q // H_kv, int(max_seqlen_q), num_seqs,
+                                                 block_tables.shape[1], k_cache.shape[1], k.shape[0])
+    try:
+        if static_scratch:
+            ops.paged_attention(*head, plan, *tail, None, True)
+            return out
+        shape_key = (num_seqs, H_q, H_kv, hd, tail[1:], has_cache, fp8, k.stride() == v.stride(),
+                     k_cache.shape[1] if has_cache and not distinct else 0)
+        need = _workspace_need.get(shape_key)
+        if need is None:
+            need = _workspace_need[shape_key] = int(ops.paged_attention_workspace_bytes(*head, None, *tail))
+        ws = _workspace(q.device, _stream(), need)
+        ops.paged_attention(*head, plan, *tail, ws, False)
+    except RuntimeError as e:
+        if "dfx_" in str(e):
+            raise _lib.DfxError(str(e).split("\n")[0]) from None
+        raise
     return out
 
 
-def _build_plan(lib, p, device, stream, group, t_new):
-    """Launch ``dfx_paged_attn_plan`` for the configuration in ``p``; None where no plan applies
-    (generic tile path).  The unit capacity is an upper bound from the shapes alone: no device data
-    is read."""
-    row_tiles = -(-group * int(p.max_seqlen_q) // 128)
-    tiles = int(p.num_seqs) * (-(-int(p.max_pages_per_seq) * int(p.page_size) // 64) + 1) + t_new // 64
-    nbytes = lib.dfx_paged_attn_plan_bytes(C.byref(p), int(p.num_kv_heads) * row_tiles * tiles)
+def _build_plan(ops, head, tail, group, max_seqlen_q, num_seqs, max_pages, page_size, t_new):
+    """Launch ``dfx_paged_attn_plan`` for this configuration; None where no plan applies (generic
+    tile path).  The unit capacity is an upper bound from the shapes alone: no device data is read."""
+    row_tiles = -(-group * max_seqlen_q // 128)
+    tiles = num_seqs * (-(-max_pages * page_size // 64) + 1) + t_new // 64
+    h_kv = head[1].shape[1]
+    nbytes = int(ops.paged_attention_plan_bytes(*head, None, *tail, h_kv * row_tiles * tiles))
     if nbytes < 0:
         return None
-    plan = torch.empty(int(nbytes), dtype=torch.uint8, device=device)
-    _lib.check(lib.dfx_paged_attn_plan(C.byref(p), plan.data_ptr(), plan.numel(), stream), "dfx_paged_attn_plan")
+    plan = torch.empty(nbytes, dtype=torch.uint8, device=head[0].device)
+    ops.paged_attention_plan(*head, None, *tail, plan)
     return plan
 
 

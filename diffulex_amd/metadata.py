@@ -76,10 +76,8 @@ def build_decode_metadata(strategy: str, *, block_tables: torch.Tensor, block_st
     tensors are made.  Nothing is read back unless ``sync_summary`` is set: ``max_seqlen_q`` is then
     the true maximum, otherwise an upper bound from the shapes (enough for the attention operators).
     Returns the metadata object with ``positions`` and ``summary`` attached as attributes."""
-    import ctypes as C
     from . import _lib
-    from .kv_cache_kernels import _stream
-    lib = _lib.load()
+    from .kv_cache_kernels import _call
     dev = block_tables.device
     B = block_tables.shape[0]
     rows = max(B, padded_seqs)
@@ -93,27 +91,10 @@ def build_decode_metadata(strategy: str, *, block_tables: torch.Tensor, block_st
     o.setdefault("context_lens", torch.empty(rows, **i32))
     o.setdefault("seq_lens", torch.empty(rows, **i32))
     o.setdefault("summary", torch.empty(8, **i32))
-    assert block_tables.dtype == torch.int32 and block_tables.stride(-1) == 1
-    assert block_state.dtype == torch.uint8 and block_state.stride(-1) == 1
-    p = _lib.MetadataParams()
-    p.strategy = {"block_diffusion": _lib.DFX_META_BLOCK_DIFFUSION, "d2f": _lib.DFX_META_D2F}[strategy]
-    p.num_seqs, p.page_size, p.diffusion_block_size = B, int(page_size), int(diffusion_block_size)
-    for name, t in (("num_tokens", num_tokens), ("prompt_len", prompt_len), ("num_pages", num_pages),
-                    ("num_diffusion_blocks", num_diffusion_blocks)):
-        if t is not None:
-            assert t.dtype == torch.int32 and t.is_contiguous() and t.numel() == B and t.device == dev
-            setattr(p, name, t.data_ptr())
-    p.block_state = block_state.data_ptr()
-    p.block_state_stride = block_state.stride(0) if block_state.dim() == 2 else 1
-    p.block_tables, p.block_table_stride = block_tables.data_ptr(), block_tables.stride(0)
-    for name in ("positions", "slot_mapping", "cu_seqlens_q", "cu_seqlens_k", "context_lens", "seq_lens", "summary"):
-        assert o[name].is_contiguous() and o[name].device == dev
-        setattr(p, name, o[name].data_ptr())
-    assert o["positions"].dtype == torch.int64 and o["positions"].numel() >= cap and o["slot_mapping"].numel() >= cap
-    assert o["cu_seqlens_q"].numel() >= rows + 1 and o["cu_seqlens_k"].numel() >= rows + 1
-    assert o["context_lens"].numel() >= rows and o["seq_lens"].numel() >= rows and o["summary"].numel() >= 8
-    p.token_capacity, p.padded_seqs, p.padded_tokens = cap, int(padded_seqs), int(padded_tokens)
-    _lib.check(lib.dfx_build_decode_metadata(C.byref(p), _stream()), "dfx_build_decode_metadata")
+    code = {"block_diffusion": _lib.DFX_META_BLOCK_DIFFUSION, "d2f": _lib.DFX_META_D2F}[strategy]
+    _call(_lib.ops().build_decode_metadata, code, block_tables, block_state, int(page_size), int(diffusion_block_size),
+          num_tokens, num_pages, prompt_len, num_diffusion_blocks, o["positions"], o["slot_mapping"], o["cu_seqlens_q"],
+          o["cu_seqlens_k"], o["context_lens"], o["seq_lens"], o["summary"], cap, int(padded_seqs), int(padded_tokens))
     d2f = strategy == "d2f"
     n_tokens = cap
     max_q = max_k = 0

@@ -11,7 +11,6 @@ a second time); the caller then runs attention with
 """
 from __future__ import annotations
 
-import ctypes as C
 from functools import lru_cache
 from typing import Optional, Tuple
 
@@ -19,7 +18,7 @@ import torch
 import torch.nn as nn
 
 from . import _lib
-from .kv_cache_kernels import _index_type, _scales, _stream
+from .kv_cache_kernels import _call, _scales
 
 
 def _rows(x: torch.Tensor, head_size: int) -> Tuple[int, int, int]:
@@ -47,43 +46,19 @@ class RotaryEmbedding(nn.Module):
 
     def _launch(self, positions, query, key, q_out, k_out, value=None, k_cache=None, v_cache=None,
                 slot_mapping=None, attn_metadata=None, k_scale=None, v_scale=None) -> None:
-        lib = _lib.load()
         table = self.cos_sin_cache
-        assert table.is_cuda and table.dtype == torch.float32 and table.is_contiguous()
-        Tq, Hq, q_st = _rows(query, self.head_size)
-        Tk, Hk, k_st = _rows(key, self.head_size)
         positions = positions.reshape(-1)
-        assert Tq == Tk == positions.numel(), "one position per token row of query and key"
         if not positions.is_contiguous():
             positions = positions.contiguous()
-        p = _lib.RopeParams()
-        p.q, p.k, p.q_out, p.k_out = query.data_ptr(), key.data_ptr(), q_out.data_ptr(), k_out.data_ptr()
-        p.q_stride_token, p.k_stride_token = q_st, k_st
-        p.q_out_stride_token, p.k_out_stride_token = q_out.stride(0), k_out.stride(0)
-        p.positions, p.position_index_type = positions.data_ptr(), _index_type(positions)
-        p.cos_sin_cache, p.max_position = table.data_ptr(), table.shape[0]
-        p.n_tokens, p.num_q_heads, p.num_kv_heads, p.head_dim = Tq, Hq, Hk, self.head_size
-        p.kv_dtype = _lib.DFX_KV_BF16
-        keep = ()
+        ks = vs = slots = None
         if slot_mapping is not None:
-            Tv, Hv, v_st = _rows(value, self.head_size)
-            assert Tv == Tk and Hv == Hk
-            D = Hk * self.head_size
-            assert k_cache.is_contiguous() and v_cache.is_contiguous()
-            assert k_cache.dim() == 4 and k_cache.stride(1) == D and v_cache.stride(1) == D
             slots = slot_mapping.reshape(-1)
-            assert slots.numel() == Tk, f"`N`: {Tk}, `slot_mapping.numel()`: {slots.numel()}"
             if not slots.is_contiguous():
                 slots = slots.contiguous()
-            kv_dtype, ksp, vsp, keep = _scales(k_cache, attn_metadata, k_scale, v_scale, Hk)
-            p.v, p.v_stride_token = value.data_ptr(), v_st
-            p.k_cache, p.v_cache = k_cache.data_ptr(), v_cache.data_ptr()
-            p.slot_mapping, p.slot_index_type = slots.data_ptr(), _index_type(slots)
-            p.n_slots = k_cache.shape[0] * k_cache.shape[1]
-            p.kv_dtype, p.k_scale, p.v_scale = kv_dtype, ksp, vsp
-            keep = keep + (slots,)
-        _lib.check(lib.dfx_rope_kv_store(C.byref(p), _stream()), "dfx_rope_kv_store")
-        del keep
+            Hk = key.shape[1] if key.dim() == 3 else key.shape[-1] // self.head_size
+            ks, vs = _scales(k_cache, attn_metadata, k_scale, v_scale, Hk)
+        _call(_lib.ops().rope_kv_store, positions, query, key, q_out, k_out, table, self.head_size, value, k_cache,
+              v_cache, slots, ks, vs)
 
     def forward(self, positions: torch.Tensor, query: torch.Tensor, key: torch.Tensor
                 ) -> Tuple[torch.Tensor, torch.Tensor]:

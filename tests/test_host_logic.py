@@ -28,6 +28,21 @@ def test_library_exports_every_declared_symbol():
     assert lib.dfx_status_string(-2) == b"unsupported shape"
 
 
+def test_operator_library_loads_and_defines_every_operator():
+    """The PyTorch operator library (csrc/torch_ext.cpp) links against the kernel library and
+    registers its operators; nothing is computed without a GPU."""
+    ops = _lib.ops()
+    for name in ("paged_attention", "paged_attention_workspace_bytes", "paged_attention_plan_bytes",
+                 "paged_attention_plan", "stream_capture_id", "kv_store_unified", "kv_store_distinct", "kv_load",
+                 "rope_kv_store", "build_decode_metadata"):
+        assert hasattr(ops, name), name
+    import torch
+    if not torch.cuda.is_available():
+        with pytest.raises((RuntimeError, NotImplementedError)):   # registered for device tensors only
+            ops.kv_store_distinct(torch.zeros(1, 1, 8), torch.zeros(1, 1, 8), torch.zeros(1, 1, 1, 1, 8),
+                                  torch.zeros(1, 1, 8, 1), torch.zeros(1, dtype=torch.int32))
+
+
 @pytest.mark.parametrize("ctype,mirror", [("dfx_attn_params", _lib.AttnParams), ("dfx_rope_params", _lib.RopeParams),
                                           ("dfx_metadata_params", _lib.MetadataParams)])
 def test_struct_layout_matches_header(tmp_path, ctype, mirror):

@@ -1,13 +1,17 @@
 #!/usr/bin/env python3
 """Headline benchmark: block-diffusion paged attention at the Dream-7B shape on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c4|c5] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c4|c5|layer|...] [--no-cpu]
 
 One step = one pass of the decode attention (``dfx_paged_attn``) over one synthetic batch
 (workload C3: 64 sequences, 28 query / 4 KV heads, head_dim 128, 256-token bf16 pages, prefix
 lengths uniform in [512, 2048], one 32-token diffusion block of queries per sequence).  Inputs
-are resident in HBM before the timed region; the KV cache is rotated over several independent
-copies so that consecutive steps cannot be served from the 256 MB Infinity Cache.
+are resident in HBM before the timed region; every tensor the launch touches (KV cache, Q, fresh
+K/V, output) is rotated over several independent copies so that consecutive steps cannot be
+served from the 256 MB Infinity Cache.  The launch plan (``dfx_paged_attn_plan``) is used the way
+a model uses it: built once per decoding step and read by the attention launches of all its
+layers (28 for Dream-7B), so the timed region holds one plan build per 28 launches; the same loop
+with a plan per launch and with no plan is timed next to it.
 
 Prints ONE JSON line: the metric (attention query tokens per second), the roofline position of
 the kernel (algorithmic bytes per launch / measured launch time against the 8 TB/s HBM peak)
@@ -29,9 +33,38 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0
-# HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this command, scaled by
-# what the same counters read for a plain copy of known size (one summary per workload under profiles/).
-MEASURED_TRAFFIC_BYTES = {"c3": 251.5e6, "c4": 1455.4e6, "c5": 821.6e6}
+LAYERS_PER_DECODE_STEP = 28  # Dream-7B / Qwen2.5-7B: attention launches that share one plan
+# HBM bytes per launch as rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this command measured them
+# (scaled by what the same counters read for a plain copy of known size): written next to the
+# profile summaries, read here, never typed in.
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "traffic.json")
+
+
+def measured_traffic(workload: str, algorithmic: int):
+    """(bytes per launch, source) from profiles/traffic.json if it was measured on this very
+    workload shape (same algorithmic bytes), else (None, None)."""
+    try:
+        with open(TRAFFIC_FILE) as f:
+            entry = json.load(f).get(workload)
+    except (OSError, ValueError):
+        return None, None
+    if not entry or int(entry.get("algorithmic_bytes", -1)) != int(algorithmic):
+        return None, None
+    return entry["bytes"], entry.get("source")
+
+
+def timed(step, steps: int, first: int = 0):
+    """(GPU ms per step by events on the launch stream, host wall ms per step to issue them)."""
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    start.record()
+    for i in range(first, first + steps):
+        step(i)
+    stop.record()
+    issue_ms = (time.perf_counter() - t0) * 1e3
+    torch.cuda.synchronize()
+    return start.elapsed_time(stop) / steps, issue_ms / steps
 
 
 def algorithmic_bytes(wl) -> int:
@@ -262,6 +295,139 @@ def bench_prefill(args, dev):
     }))
 
 
+def bench_store_distinct(args, dev):
+    """Paged KV-cache store into the "distinct" layout (K [pages, H, hd / 8, page, 8], V [pages, H, hd,
+    page]) at the C2 shape: one fresh 32-token block per sequence, slots in runs inside their pages."""
+    import ctypes as C
+    from diffulex_amd import _lib
+    from diffulex_amd.workloads import make_workload
+    lib = _lib.load()
+    wl = make_workload("c2", device=dev)
+    st = torch.cuda.current_stream().cuda_stream
+    n_new, h, hd = wl.k_new.shape
+    pages, page, x, n_sets = wl.k_cache.shape[0], wl.page_size, 8, 8
+    sets = [(torch.randn(n_new, h, hd, device=dev).to(torch.bfloat16), torch.randn(n_new, h, hd, device=dev).to(torch.bfloat16),
+             torch.zeros(pages, h, hd // x, page, x, dtype=torch.bfloat16, device=dev),
+             torch.zeros(pages, h, hd, page, dtype=torch.bfloat16, device=dev)) for _ in range(n_sets)]
+    kcs = (C.c_int64 * 5)(*sets[0][2].stride())
+    vcs = (C.c_int64 * 4)(*sets[0][3].stride())
+
+    def step(i):
+        k, v, kc, vc = sets[i % n_sets]
+        rc = lib.dfx_kv_store_distinct(k.data_ptr(), v.data_ptr(), k.stride(0), v.stride(0), kc.data_ptr(), vc.data_ptr(),
+                                       kcs, vcs, wl.slot_mapping.data_ptr(), _lib.DFX_INDEX_I32, n_new, pages, page, x,
+                                       h, hd, st)
+        _lib.check(rc, "dfx_kv_store_distinct")
+
+    n_spin = spin_up(step)
+    for i in range(args.warmup):
+        step(i)
+    ms, _ = timed(step, args.steps)
+    nbytes = 2 * 2 * n_new * h * hd * 2   # K and V rows read once, written once
+    gbs = nbytes / (ms * 1e-3) / 1e9
+    print(json.dumps({
+        "metric": "paged KV-cache store, distinct layout, tokens per second and achieved HBM GB/s, 1 GPU",
+        "value": n_new / (ms * 1e-3), "unit": "kv-tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "u16 (bit copy)",
+        "data": "synthetic",
+        "config": {"workload": f"store-distinct: {n_new} fresh tokens (B={wl.num_seqs} x 32) by slot_mapping into "
+                               f"K [pages, {h}, {hd // x}, {page}, {x}] / V [pages, {h}, {hd}, {page}]",
+                   "tensor_sets_rotated": n_sets, "spin_up_launches": n_spin},
+        "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS,
+                     "traffic": None, "algorithmic_bytes": nbytes,
+                     "kernel": "kv_store_distinct_tiled<int, 128>, duration = timed region / steps (launch-bound at this size)"},
+    }))
+
+
+def bench_layer(args, dev):
+    """The attention part of one decoder layer of a decoding step as Diffulex runs it, through the
+    Python operators: rotary embedding of the layer's Q/K projections, then ``Attention.forward``
+    (KV-cache store of the fresh block + paged attention) at the C3 shape.  Timed eagerly and as a
+    replayed HIP graph of one decoding step's 28 layers; the plan is built once per step in both."""
+    import diffulex_amd as dfx
+    from diffulex_amd.workloads import make_workload
+    wl = make_workload("c3", device=dev)
+    T, hq, hkv, hd = wl.q.shape[0], wl.num_q_heads, wl.num_kv_heads, wl.head_dim
+    n_sets = max(args.copies, 4)
+    g = torch.Generator("cpu").manual_seed(11)
+    rope = dfx.RotaryEmbedding(hd, hd, 8192, 1.0e6).to(dev)
+    positions = (wl.context_lens.repeat_interleave(wl.q_len) + torch.arange(wl.q_len, device=dev).repeat(wl.num_seqs)).long()
+    layers = []
+    for _ in range(n_sets):
+        att = dfx.Attention(hq, hd, wl.scale, hkv)
+        att.k_cache, att.v_cache = wl.k_cache.clone(), wl.v_cache.clone()
+        qkv = torch.randn(T, (hq + 2 * hkv) * hd, generator=g).to(torch.bfloat16).to(dev)
+        layers.append((att, qkv))
+    state = {}
+
+    def new_decode_step():
+        state["md"] = dfx.PagedAttnMetaData(
+            is_prefill=False, cu_seqlens_q=wl.cu_seqlens_q, cu_seqlens_k=wl.cu_seqlens_q, max_seqlen_q=wl.q_len,
+            slot_mapping=wl.slot_mapping, context_lens=wl.context_lens, block_tables=wl.block_tables,
+            page_block_size=wl.page_size, diffusion_block_size=wl.diffusion_block_size, decode_mode="static",
+            need_kv_cache_store=True)
+    dfx.set_fetch_fn_for_attn_metadata(lambda: state["md"])
+
+    def layer(i):
+        if i % LAYERS_PER_DECODE_STEP == 0:
+            new_decode_step()
+        att, qkv = layers[i % n_sets]
+        q, k, v = qkv.split([hq * hd, hkv * hd, hkv * hd], dim=-1)
+        q, k = rope(positions, q, k)
+        return att(q, k, v)
+
+    n_spin = spin_up(layer)
+    for i in range(args.warmup):
+        layer(i)
+    steps = max(LAYERS_PER_DECODE_STEP, args.steps // LAYERS_PER_DECODE_STEP * LAYERS_PER_DECODE_STEP)
+    eager_ms, eager_issue_ms = timed(layer, steps)
+
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for i in range(LAYERS_PER_DECODE_STEP):
+            layer(i)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    with torch.cuda.graph(graph):
+        for i in range(LAYERS_PER_DECODE_STEP):
+            layer(i)
+    for _ in range(5):
+        graph.replay()
+    replays = steps // LAYERS_PER_DECODE_STEP
+    graph_ms, graph_issue_ms = timed(lambda i: graph.replay(), replays)
+    graph_ms /= LAYERS_PER_DECODE_STEP
+    graph_issue_ms /= LAYERS_PER_DECODE_STEP
+
+    row = hd * 2
+    nbytes = (int(wl.context_lens.sum()) * hkv * row * 2            # cached K and V read by the attention
+              + T * (hq + 2 * hkv) * row                            # projections read by the rotary embedding
+              + T * (hq + hkv) * row                                # rotated q and k written
+              + T * (hq + 2 * hkv) * row                            # q, k, v read by the attention
+              + 2 * T * hkv * row + T * hq * row)                   # block stored into the cache, output written
+    ms = graph_ms
+    gbs = nbytes / (ms * 1e-3) / 1e9
+    print(json.dumps({
+        "metric": "decode layer step (rotary embedding + KV store + paged attention through the Python operators), "
+                  "query-tokens/sec, 1 GPU",
+        "value": T / (ms * 1e-3), "unit": "query-tokens/s", "n_gpus": 1, "steps": steps, "warmup": args.warmup,
+        "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": f"layer: c3 shapes (B={wl.num_seqs}, {T} tokens, H_q={hq}, H_kv={hkv}, head_dim={hd}); per layer "
+                               "RotaryEmbedding.forward then Attention.forward (store fused into the attention launch)",
+                   "mode": f"HIP graph of {LAYERS_PER_DECODE_STEP} layers replayed (ms_per_step); eager beside it",
+                   "eager_ms_per_step": eager_ms, "eager_host_wall_ms_per_step": eager_issue_ms,
+                   "graph_ms_per_step": graph_ms, "graph_host_wall_ms_per_step": graph_issue_ms,
+                   "host_wall_ms_per_step": graph_issue_ms,
+                   "tensor_sets_rotated": n_sets, "spin_up_launches": n_spin},
+        "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS,
+                     "traffic": None, "algorithmic_bytes": nbytes,
+                     "kernel": "rope_kv_store_kernel + paged_attn_pipe_kernel<8> (+ plan kernels once per graph), "
+                               "duration = graph replay / layers"},
+    }))
+
+
 SPIN_UP_SECONDS = 0.25
 
 
@@ -285,7 +451,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=1000)
     ap.add_argument("--warmup", type=int, default=100)
-    ap.add_argument("--workload", default="c3", choices=["c3", "c4", "c5", "c1", "c2", "rope", "prefill"])
+    ap.add_argument("--workload", default="c3", choices=["c3", "c4", "c5", "c1", "c2", "rope", "prefill", "layer", "store-distinct"])
     ap.add_argument("--copies", type=int, default=4, help="independent KV-cache copies rotated between steps")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -321,36 +487,57 @@ def main():
     if args.workload == "prefill":
         bench_prefill(args, dev)
         return
+    if args.workload == "layer":
+        bench_layer(args, dev)
+        return
+    if args.workload == "store-distinct":
+        bench_store_distinct(args, dev)
+        return
     wl = make_workload(args.workload, device=dev)
-    caches = [(wl.k_cache, wl.v_cache)]
+    # every tensor a launch touches exists `copies` times; step i uses set i % copies
+    sets = [(wl.q, wl.k_new, wl.v_new, torch.empty_like(wl.q), wl.k_cache, wl.v_cache)]
     for _ in range(args.copies - 1):
-        caches.append((wl.k_cache.clone(), wl.v_cache.clone()))
+        sets.append((wl.q.clone(), wl.k_new.clone(), wl.v_new.clone(), torch.empty_like(wl.q), wl.k_cache.clone(),
+                     wl.v_cache.clone()))
     kw = dict(block_tables=wl.block_tables, context_lens=wl.context_lens, cu_seqlens_q=wl.cu_seqlens_q,
               cu_seqlens_new=wl.cu_seqlens_q, max_seqlen_q=wl.q_len, mask_mode=wl.mask_mode,
               diffusion_block_size=wl.diffusion_block_size, k_scale=wl.k_scale, v_scale=wl.v_scale)
-    out = torch.empty_like(wl.q)
+    plans = {"cache": {}}
 
-    def step(i):
-        kc, vc = caches[i % len(caches)]
-        dfx.paged_attention(wl.q, wl.k_new, wl.v_new, kc, vc, wl.scale, out=out, **kw)
+    def step_reused_plan(i):
+        if i % LAYERS_PER_DECODE_STEP == 0:
+            plans["cache"] = {}          # a new decoding step: lengths and tables changed, plan again
+        q, kn, vn, out, kc, vc = sets[i % len(sets)]
+        dfx.paged_attention(q, kn, vn, kc, vc, wl.scale, out=out, plan_cache=plans["cache"], **kw)
 
-    n_spin = spin_up(step)
+    def step_plan_per_call(i):
+        q, kn, vn, out, kc, vc = sets[i % len(sets)]
+        dfx.paged_attention(q, kn, vn, kc, vc, wl.scale, out=out, plan_cache={}, **kw)
+
+    def step_no_plan(i):
+        q, kn, vn, out, kc, vc = sets[i % len(sets)]
+        dfx.paged_attention(q, kn, vn, kc, vc, wl.scale, out=out, **kw)
+
+    # cold: the device has been idle, nothing but the code is loaded (one launch), clocks are down
+    step_reused_plan(0)
+    torch.cuda.synchronize()
+    time.sleep(0.5)
+    cold_ms, _ = timed(step_reused_plan, 28)
+
+    n_spin = spin_up(step_reused_plan)
     for i in range(args.warmup):
-        step(i)
-    torch.cuda.synchronize()
-    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    t0 = time.perf_counter()
-    start.record()
-    for i in range(args.steps):
-        step(i)
-    stop.record()
-    torch.cuda.synchronize()
-    wall_ms = (time.perf_counter() - t0) * 1e3
-    ms = start.elapsed_time(stop) / args.steps
+        step_reused_plan(i)
+    ms, issue_ms = timed(step_reused_plan, args.steps)
+    side = max(LAYERS_PER_DECODE_STEP, min(args.steps, 280))
+    ms_per_call, _ = timed(step_plan_per_call, side)
+    ms_no_plan, _ = timed(step_no_plan, side)
 
     nbytes, nflops = algorithmic_bytes(wl), algorithmic_flops(wl)
     gbs = nbytes / (ms * 1e-3) / 1e9
     tflops = nflops / (ms * 1e-3) / 1e12
+    traffic, traffic_source = measured_traffic(args.workload, nbytes)
+    kernel = ("paged_attn_stream_fp8_kernel<128, 8>" if wl.kv_fp8 else
+              "paged_attn_pipe_kernel<8>" if args.workload == "c3" else "paged_attn_stream_kernel")
     result = {
         "metric": "attn query-tokens/sec + achieved HBM GB/s (% of peak), Dream-7B shape, 1 GPU",
         "value": wl.total_q_tokens / (ms * 1e-3), "unit": "query-tokens/s",
@@ -363,17 +550,21 @@ def main():
                         f"ctx in [{int(wl.context_lens.min())},{int(wl.context_lens.max())}] "
                         f"(sum {int(wl.context_lens.sum())}), q_len={wl.q_len}, "
                         f"mask={'block-causal' if wl.mask_mode else 'full'}, kv={'fp8-e4m3' if wl.kv_fp8 else 'bf16'}",
-            "kv_cache_copies_rotated": len(caches),
-            "host_wall_ms_per_step": wall_ms / args.steps,
+            "plan": f"built once per {LAYERS_PER_DECODE_STEP} launches inside the timed region (one decoding step's layers)",
+            "ms_per_step_plan_per_launch": ms_per_call,
+            "ms_per_step_no_plan": ms_no_plan,
+            "cold_ms_per_step": cold_ms,
+            "tensor_sets_rotated": len(sets),
+            "host_wall_ms_per_step": issue_ms,
             "spin_up_launches": n_spin,
         },
         "roofline": {
             "bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS,
-            "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
+            "traffic": traffic, "traffic_source": traffic_source,
             "algorithmic_bytes": nbytes, "algorithmic_flops": nflops,
             "mfma_tflops": tflops, "mfma_frac": tflops / MFMA_BF16_PEAK_TFLOPS,
-            "kernel": "paged_attn_stream_kernel (bf16 KV) / paged_attn_stream_fp8_kernel (FP8 KV), one launch per step, "
-                      "duration = timed region / steps",
+            "kernel": f"{kernel}, one launch per step; duration = timed region (HIP events on the launch stream) / steps, "
+                      f"which includes the plan kernels once per {LAYERS_PER_DECODE_STEP} launches",
         },
     }
     if not args.no_cpu:

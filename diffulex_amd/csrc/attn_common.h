@@ -46,6 +46,7 @@ struct KArgs {
     const void* store_slots;  // fused KV-cache store: slot per fresh row, or null
     int store_slots_i64;
     int64_t n_new;            // rows of k_new / v_new (and of the slot mapping)
+    int64_t v_fresh_delta;    // streaming paths: (token stride of v_new - token stride of k_new) in bytes
     const uint8_t* plan;      // launch plan built by the plan kernels, or null
     uint32_t plan_signature;  // of this launch's configuration: a plan made for another one is ignored
     int64_t q_st, q_sh, kn_st, kn_sh, vn_st, vn_sh, o_st, o_sh;

@@ -39,9 +39,10 @@ struct UnitDesc {
 };
 static_assert(sizeof(UnitDesc) == 48, "UnitDesc is read as three 16-byte LDS words");
 struct BandDesc {
-    int64_t off;   // byte offset of the band's first row from the K (== from the V) base pointer
+    int64_t off;   // byte offset of the band's first row from the K base pointer (the V base too, for cached rows)
     int32_t last;  // last valid row of the band; later rows re-read it
-    int32_t is_ctx;
+    int32_t is_ctx;  // 1: cached rows; fresh rows: -(1 + index of the band's first row in k_new / v_new), from
+                     // which the V offset follows where v_new has another token stride than k_new
 };
 // ---- the launch plan (plan.h builds it; layout of the buffer described there) ----------------------
 constexpr uint32_t kPlanMagic = 0x44465850u;  // "DFXP"
@@ -234,7 +235,7 @@ struct StreamAttn : TileMath<HD, NB, NW, HIDDEN> {
                 b.off = ((static_cast<int64_t>(a.cu_new[sq]) + band) * a.kn_st + kv_head * a.kn_sh) * 2;
             }
             b.last = limit - 1 - band;
-            b.is_ctx = is_ctx ? 1 : 0;
+            b.is_ctx = is_ctx ? 1 : -(1 + a.cu_new[sq] + band);
             bands[slot_in_ring * NW + w] = b;
             // the NW lanes of a unit are neighbours in a wave: its holes as a bit per band
             const uint64_t votes = __ballot(hole);
@@ -248,25 +249,32 @@ struct StreamAttn : TileMath<HD, NB, NW, HIDDEN> {
     DFX_D void issue_unit(int rel) const {
         const BandDesc b = bands[rel * NW + wave];
         const int last = uniform(b.last);
-        const bool is_ctx = uniform(b.is_ctx) != 0;
+        const int tag = uniform(b.is_ctx);
+        const bool is_ctx = tag > 0;
         const int64_t off = (static_cast<int64_t>(uniform(static_cast<int>(b.off >> 32))) << 32) |
                             static_cast<uint32_t>(uniform(static_cast<int>(b.off)));
         const uint8_t* kbase = (is_ctx ? a.k_cache : reinterpret_cast<const uint8_t*>(a.k_new)) + off;
-        const uint8_t* vbase = (is_ctx ? a.v_cache : reinterpret_cast<const uint8_t*>(a.v_new)) + off;
+        // fresh V rows may lie further apart than fresh K rows (V a slice of a projection, K rotated
+        // into a buffer of its own): same head offset, another token stride
+        const uint8_t* vbase = is_ctx ? a.v_cache + off
+                                      : reinterpret_cast<const uint8_t*>(a.v_new) + off + static_cast<int64_t>(-1 - tag) * a.v_fresh_delta;
         const uint32_t row_stride = static_cast<uint32_t>(is_ctx ? a.c_st * KVB : a.kn_st * 2);
+        const uint32_t row_stride_v = static_cast<uint32_t>(is_ctx ? a.c_st * KVB : a.vn_st * 2);
         const uint32_t dst = stages_lds + (rel % C::kStages) * C::STAGE_BYTES + wave * (C::IPW * 1024);
 #pragma unroll
         for (int j = 0; j < C::IPW; ++j) {
             const int r = j * C::RPI + lane / C::CPR;  // row inside the band
             const int lds_row = wave * C::ROWS_PER_WAVE + r;
             const int chunk = (lane % C::CPR) ^ C::swizzle(lds_row);
-            uint32_t voff = static_cast<uint32_t>(min(r, last)) * row_stride + chunk * 16;
+            const uint32_t rl = static_cast<uint32_t>(min(r, last));
+            uint32_t voff = rl * row_stride + chunk * 16;
+            uint32_t voff_v = rl * row_stride_v + chunk * 16;
             // Fresh rows are bf16 and are fetched by widen_unit() itself; the loads are issued all
             // the same (every lane re-reads the band's first bytes) so that every unit advances
             // the completion counter by the same amount.
-            if (KVB == 1 && !is_ctx) voff = 0;
+            if (KVB == 1 && !is_ctx) voff = voff_v = 0;
             async_load16(kbase, voff, dst + j * 1024);
-            async_load16(vbase, voff, dst + C::MAT_BYTES + j * 1024);
+            async_load16(vbase, voff_v, dst + C::MAT_BYTES + j * 1024);
         }
     }
 
@@ -276,7 +284,8 @@ struct StreamAttn : TileMath<HD, NB, NW, HIDDEN> {
     DFX_D uint8_t* wide_tile(int rel) const { return lds + C::WIDE_OFF + (rel & 1) * C::WIDE_BYTES; }
     DFX_D void widen_unit(int rel) const {
         const BandDesc b = bands[rel * NW + wave];
-        const bool is_ctx = uniform(b.is_ctx) != 0;
+        const int tag = uniform(b.is_ctx);
+        const bool is_ctx = tag > 0;
         uint8_t* kt = wide_tile(rel);
         uint8_t* vt = kt + L::MAT_BYTES;
         const uint8_t* raw = lds + C::STAGES_OFF + (rel % C::kStages) * C::STAGE_BYTES + wave * (C::IPW * 1024) + lane * 16;
@@ -300,17 +309,18 @@ struct StreamAttn : TileMath<HD, NB, NW, HIDDEN> {
             const int64_t off = (static_cast<int64_t>(uniform(static_cast<int>(b.off >> 32))) << 32) |
                                 static_cast<uint32_t>(uniform(static_cast<int>(b.off)));
             const uint8_t* kbase = reinterpret_cast<const uint8_t*>(a.k_new) + off;
-            const uint8_t* vbase = reinterpret_cast<const uint8_t*>(a.v_new) + off;
+            const uint8_t* vbase = reinterpret_cast<const uint8_t*>(a.v_new) + off + static_cast<int64_t>(-1 - tag) * a.v_fresh_delta;
 #pragma unroll
             for (int j = 0; j < C::IPW; ++j) {
                 const int r = j * C::RPI + lane / C::CPR;
                 const int row = wave * C::ROWS_PER_WAVE + r;
                 const int cc = lane % C::CPR;
                 const int64_t voff = static_cast<int64_t>(min(r, last)) * a.kn_st * 2 + cc * 32;
+                const int64_t voff_v = static_cast<int64_t>(min(r, last)) * a.vn_st * 2 + cc * 32;
                 const u32x4 k0 = *reinterpret_cast<const u32x4*>(kbase + voff);
                 const u32x4 k1 = *reinterpret_cast<const u32x4*>(kbase + voff + 16);
-                const u32x4 v0 = *reinterpret_cast<const u32x4*>(vbase + voff);
-                const u32x4 v1 = *reinterpret_cast<const u32x4*>(vbase + voff + 16);
+                const u32x4 v0 = *reinterpret_cast<const u32x4*>(vbase + voff_v);
+                const u32x4 v1 = *reinterpret_cast<const u32x4*>(vbase + voff_v + 16);
                 // Wait here, inside the branch: a wait the compiler places where the two branches
                 // meet again would drain the asynchronous loads in every step.
                 __builtin_amdgcn_s_waitcnt(0x0f70);

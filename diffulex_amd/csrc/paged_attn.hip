@@ -62,14 +62,15 @@ int make_plan(const dfx_attn_params* p, Plan& plan) {
     plan.hd = p->head_dim;
     plan.nb = rows <= 32 * kWaves ? 1 : 2;
     plan.fp8 = p->kv_dtype == DFX_KV_FP8_E4M3 && p->k_cache != nullptr;
-    // The streaming path addresses a K row and its V row with one offset: page size a multiple
-    // of 16, fresh K and V laid out alike.  FP8 streaming exists for head_dim 128.
+    // The streaming path addresses a cached K row and its V row with one offset: page size a
+    // multiple of 16; fresh K and V may differ in their token stride, not in their head stride.
+    // FP8 streaming exists for head_dim 128.
     plan.distinct = p->cache_layout == DFX_CACHE_DISTINCT && p->k_cache != nullptr;
     if (p->cache_layout != DFX_CACHE_UNIFIED && p->cache_layout != DFX_CACHE_DISTINCT) return DFX_ERR_INVALID_ARG;
     if (plan.distinct && plan.fp8) return DFX_ERR_UNSUPPORTED;
     plan.stream = !(p->flags & DFX_ATTN_GENERIC_PATH) && !plan.distinct &&
                   (p->k_cache == nullptr || (p->page_size > 0 && p->page_size % 16 == 0)) &&
-                  p->kn_stride_token == p->vn_stride_token && p->kn_stride_head == p->vn_stride_head &&
+                  p->kn_stride_head == p->vn_stride_head &&
                   (!plan.fp8 || p->head_dim == 128);
     plan.compact = plan.stream && !plan.fp8 && plan.nb == 1 && p->num_seqs <= kCompactMaxSeqs;
     // (8 waves only: with 4 waves a wave has twice the tile loads to address, and the 32 registers
@@ -259,7 +260,7 @@ uint32_t plan_signature(const dfx_attn_params* p, const Plan& plan) {
     mix(plan.hd); mix(plan.nb); mix(plan.n_wg); mix(plan.fp8); mix(plan.stream); mix(plan.compact);
     mix(p->num_seqs); mix(p->num_q_heads); mix(p->num_kv_heads); mix(p->page_size); mix(p->max_pages_per_seq);
     mix(p->max_seqlen_q); mix(p->num_new_tokens); mix(p->diffusion_block_size); mix(p->mask_mode); mix(p->max_workgroups);
-    mix(p->kn_stride_token); mix(p->kn_stride_head); mix(p->cache_stride_page); mix(p->cache_stride_token);
+    mix(p->kn_stride_token); mix(p->kn_stride_head); mix(p->vn_stride_token); mix(p->cache_stride_page); mix(p->cache_stride_token);
     mix(p->cache_stride_head); mix(p->block_table_stride); mix(p->n_pages); mix(p->k_cache != nullptr);
     mix(reinterpret_cast<uintptr_t>(p->block_tables)); mix(reinterpret_cast<uintptr_t>(p->context_lens));
     mix(reinterpret_cast<uintptr_t>(p->cu_seqlens_q)); mix(reinterpret_cast<uintptr_t>(p->cu_seqlens_new));
@@ -350,6 +351,7 @@ int run_paged_attn(const dfx_attn_params* p, void* workspace, int64_t workspace_
     }
     ka.c = p->scale * kLog2e;
     ka.n_new = p->num_new_tokens > 0 ? p->num_new_tokens : INT64_MAX;
+    ka.v_fresh_delta = (p->vn_stride_token - p->kn_stride_token) * 2;
     ka.plan = nullptr;
     ka.plan_signature = plan_signature(p, plan);
     if (plan_out == nullptr && plan.stream && p->plan != nullptr) {

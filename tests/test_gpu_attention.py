@@ -153,6 +153,49 @@ def test_fresh_k_and_v_with_different_strides(dev):
         assert max_abs_err(got, want) <= (ATOL_FP8 if name == "c5" else ATOL_BF16)
 
 
+@pytest.mark.parametrize("flags", PATHS + [_lib.DFX_ATTN_NO_PIPELINE])
+@pytest.mark.parametrize("name,over", [
+    ("c3", dict(num_seqs=6, ctx=(100, 900))),            # 8 waves, the pipelined tile loop
+    ("c1", {}),                                          # head_dim 64, two workgroups per compute unit
+    ("c5", dict(num_seqs=4, ctx=(200, 900))),            # FP8 cache: fresh rows fetched by the widening step
+    ("c4", dict(num_seqs=3, ctx=(100, 500))),            # block-causal, 96 fresh rows per sequence
+])
+def test_fresh_v_sliced_out_of_the_projection(dev, name, over, flags):
+    """What a decoder layer passes: K rotated into a buffer of its own, V still a column slice of
+    the fused QKV projection, so fresh V rows lie further apart than fresh K rows (same head
+    stride).  The streaming kernels take that as it is; with and without a plan, and with the fused
+    store, the result equals the one on contiguous copies, bit for bit."""
+    wl = make_workload(name, seed=101, **over).to(dev)
+    t, h, d = wl.v_new.shape
+    qkv = torch.randn(t, (wl.num_q_heads + 2 * h) * d, device=dev).to(torch.bfloat16)
+    v_view = qkv[:, (wl.num_q_heads + h) * d:].view(t, h, d)
+    v_view.copy_(wl.v_new)
+    assert v_view.stride(0) != wl.k_new.stride(0) and v_view.stride(1) == wl.k_new.stride(1)
+    want = _run(wl, flags=flags)
+    assert max_abs_err(want, oracle_fp32(wl)) <= (ATOL_FP8 if name == "c5" else ATOL_BF16)
+    contiguous_v = wl.v_new
+    wl.v_new = v_view
+    for max_wg in (0, 5):
+        ref = _run(wl, max_wg, flags=flags) if max_wg == 0 else None
+        got = _run(wl, max_wg, flags=flags, plan_cache={})
+        if ref is not None:
+            assert torch.equal(ref, want) and torch.equal(got, want)
+        else:
+            wl.v_new = contiguous_v
+            assert torch.equal(got, _run(wl, max_wg, flags=flags))
+            wl.v_new = v_view
+    kc, vc = wl.k_cache.clone(), wl.v_cache.clone()
+    dfx.store_kvcache_unified_layout(wl.k_new, contiguous_v, kc, vc, wl.slot_mapping, metadata_for(wl, "static"))
+    kc2, vc2 = wl.k_cache.clone(), wl.v_cache.clone()
+    got = dfx.paged_attention(wl.q, wl.k_new, wl.v_new, kc2, vc2, wl.scale, block_tables=wl.block_tables,
+                              context_lens=wl.context_lens, cu_seqlens_q=wl.cu_seqlens_q, cu_seqlens_new=wl.cu_seqlens_q,
+                              max_seqlen_q=wl.q_len, mask_mode=wl.mask_mode, diffusion_block_size=wl.diffusion_block_size,
+                              k_scale=wl.k_scale, v_scale=wl.v_scale, flags=flags, store_slot_mapping=wl.slot_mapping)
+    torch.cuda.synchronize()
+    assert torch.equal(got, want)
+    assert torch.equal(kc2.view(torch.uint8), kc.view(torch.uint8)) and torch.equal(vc2.view(torch.uint8), vc.view(torch.uint8))
+
+
 @pytest.mark.parametrize("flags", PATHS)
 def test_d2f_block_causal_small_c4(dev, flags):
     wl = make_workload("c4", num_seqs=3, ctx=(100, 700))

@@ -134,7 +134,8 @@ struct TileInfo {
     int limit;     // number of valid tokens of that kind
     bool is_ctx;
     float c_tile;  // logit -> log2 domain factor (scale * log2 e, times k_scale for FP8 context)
-    float v_mul;   // factor applied to P before the PV product (v_scale for FP8 context, else 1)
+    float v_mul;   // factor applied to P before the PV product: 1, except 1 / v_scale for the fresh (bf16)
+                   // tiles of a launch on an FP8 cache, whose O^T is kept in units of v_scale
     uint64_t holes;  // bit b: tokens base + b * HOLE_ROWS .. + HOLE_ROWS - 1 (HOLE_ROWS: a parameter of
                      // softmax_tile) sit on a page whose block-table entry is negative or out of range
                      // and are skipped, as the reference skips such pages
@@ -157,6 +158,7 @@ struct AttnState {
     f32x16 o[S::NDB][NB];
     float m_run[NB], l_run[NB];
     int vis_limit[NB];
+    float out_mul = 1.0f;  // O^T is accumulated in units of this (v_scale of the item's head on an FP8 cache)
 
     DFX_D explicit AttnState(const KArgs& args)
         : a(args), tid(threadIdx.x), lane(threadIdx.x & 63), wave(threadIdx.x >> 6), col(threadIdx.x & 31),
@@ -187,9 +189,9 @@ struct AttnState {
         t.c_tile = a.c;
         t.v_mul = 1.0f;
         t.holes = 0;
-        if (fp8 && t.is_ctx) {
-            t.c_tile = fmaxf(a.c * a.k_scale[kv_head], 1e-30f);
-            t.v_mul = a.v_scale[kv_head];
+        if (fp8) {
+            if (t.is_ctx) t.c_tile = fmaxf(a.c * a.k_scale[kv_head], 1e-30f);
+            else t.v_mul = 1.0f / a.v_scale[kv_head];
         }
         return t;
     }
@@ -287,7 +289,10 @@ struct AttnState {
                 for (int e = 0; e < 16; ++e) {
                     p[e] = fast_exp2(__builtin_fmaf(sc[tb][qb][e], t.c_tile, -m_safe));
                     lsum += p[e];
-                    if (SCALE_P) p[e] *= t.v_mul;
+                }
+                if (SCALE_P && t.v_mul != 1.0f) {  // (wave-uniform; fresh tiles of an FP8 launch only)
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) p[e] *= t.v_mul;
                 }
 #pragma unroll
                 for (int sl = 0; sl < 2; ++sl) {
@@ -328,7 +333,7 @@ struct AttnState {
             const int i = valid ? r - g * sh.q_len : 0;
             // a row none of whose keys is visible (every page of its context a hole, no fresh rows)
             // has a zero sum: it gets zeros, not 0 * inf
-            const float inv = l_tot[qb] > 0.0f ? 1.0f / l_tot[qb] : 0.0f;
+            const float inv = l_tot[qb] > 0.0f ? out_mul / l_tot[qb] : 0.0f;
             uint16_t* op = a.out + (q0 + i) * a.o_st + (kvh * a.group + g) * a.o_sh + half * 8;
 #pragma unroll
             for (int db = 0; db < S::NDB; ++db) {

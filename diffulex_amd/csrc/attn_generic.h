@@ -311,6 +311,7 @@ __global__ void __launch_bounds__(kThreads) paged_attn_generic_kernel(const KArg
     int64_t pos = begin;
     while (pos < end) {
         at.set_sequence(s, kvh);
+        if constexpr (FP8) at.out_mul = a.v_scale[kvh];
         int rt, tile0, n_tiles;
         locate_unit(at.sh, u, rt, tile0, n_tiles);
         const int64_t seg_end = min(pos + (n_tiles - tile0), end);

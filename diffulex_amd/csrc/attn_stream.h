@@ -160,7 +160,7 @@ struct StreamAttn : TileMath<HD, NB, NW, HIDDEN> {
     int64_t begin, end;
     int64_t rel_base;  // what UnitDesc::item_rel is relative to: the first unit of the workgroup's work
     int per_head;
-    float k_mul, v_mul;  // the current item's FP8 scales
+    float k_mul, v_inv;  // FP8: the current item's K scale and the reciprocal of its V scale
 
     DFX_D StreamAttn(const KArgs& args, uint8_t* smem)
         : Base(args), lds(smem), prefix(reinterpret_cast<int*>(smem)),
@@ -351,7 +351,8 @@ struct StreamAttn : TileMath<HD, NB, NW, HIDDEN> {
         this->sh.q_len = uniform(d.q_len);
         if (KVB == 1) {
             k_mul = a.k_scale[this->kvh];
-            v_mul = a.v_scale[this->kvh];
+            this->out_mul = a.v_scale[this->kvh];
+            v_inv = 1.0f / this->out_mul;
         }
         this->load_queries(uniform(d.rt));
         if (wait) touch_queries();
@@ -545,11 +546,13 @@ __global__ void __launch_bounds__(64 * NW, COMPACT ? 2 : 1) paged_attn_stream_ke
 // instructions of the previous step have just released, then computes unit rel from the other
 // bf16 tile.  The ring needs no barrier (a stage's band is written and read by one wave only);
 // the one barrier per step orders the two bf16 tiles.
-template <int HD, int NW>
+// NB query blocks per wave: 1 with head_dim 128 (8 waves for up to 256 rows); with head_dim 64 a
+// 64-token tile of codes is 4 KiB, one load instruction each for 4 waves, so 4 waves take 1 or 2.
+template <int HD, int NB, int NW>
 __global__ void __launch_bounds__(64 * NW, 1) paged_attn_stream_fp8_kernel(const KArgs a) {
     extern __shared__ __attribute__((aligned(256))) uint8_t smem[];
-    using C = StreamCfg<HD, 1, NW, false, 1>;
-    StreamAttn<HD, 1, NW, false, 1> at(a, smem);
+    using C = StreamCfg<HD, NB, NW, false, 1>;
+    StreamAttn<HD, NB, NW, false, 1> at(a, smem);
     store_fresh_rows<HD, true>(a);  // first, as in the bf16 kernel
     at.for_each_chunk([&](int n_units) {
         const WgSplit& split = at.split;
@@ -582,12 +585,12 @@ __global__ void __launch_bounds__(64 * NW, 1) paged_attn_stream_fp8_kernel(const
                 t.is_ctx = (uniform(u.flags) & kUnitCtx) != 0;
                 t.holes = static_cast<uint32_t>(uniform(u.flags)) >> kUnitHoleShift;  // a bit per band of rows
                 t.c_tile = t.is_ctx ? a.c * at.k_mul : a.c;
-                t.v_mul = t.is_ctx ? at.v_mul : 1.0f;
+                t.v_mul = t.is_ctx ? 1.0f : at.v_inv;
                 const uint8_t* k_tile = at.wide_tile(rel);
                 if (at.wave < a.busy_waves) {
-                    f32x16 sc[2][1];
+                    f32x16 sc[2][NB];
                     at.scores(k_tile, sc);
-                    bf16x8 pb[1][2][2];
+                    bf16x8 pb[NB][2][2];
                     at.template softmax_tile<true, C::ROWS_PER_WAVE>(sc, t, pb, [&] { at.outputs_ready(); });
                     at.accumulate(k_tile + TileLayout<HD>::MAT_BYTES, pb);
                 } else {

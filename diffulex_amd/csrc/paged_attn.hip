@@ -64,14 +64,13 @@ int make_plan(const dfx_attn_params* p, Plan& plan) {
     plan.fp8 = p->kv_dtype == DFX_KV_FP8_E4M3 && p->k_cache != nullptr;
     // The streaming path addresses a cached K row and its V row with one offset: page size a
     // multiple of 16; fresh K and V may differ in their token stride, not in their head stride.
-    // FP8 streaming exists for head_dim 128.
+
     plan.distinct = p->cache_layout == DFX_CACHE_DISTINCT && p->k_cache != nullptr;
     if (p->cache_layout != DFX_CACHE_UNIFIED && p->cache_layout != DFX_CACHE_DISTINCT) return DFX_ERR_INVALID_ARG;
     if (plan.distinct && plan.fp8) return DFX_ERR_UNSUPPORTED;
     plan.stream = !(p->flags & DFX_ATTN_GENERIC_PATH) && !plan.distinct &&
                   (p->k_cache == nullptr || (p->page_size > 0 && p->page_size % 16 == 0)) &&
-                  p->kn_stride_head == p->vn_stride_head &&
-                  (!plan.fp8 || p->head_dim == 128);
+                  p->kn_stride_head == p->vn_stride_head;
     plan.compact = plan.stream && !plan.fp8 && plan.nb == 1 && p->num_seqs <= kCompactMaxSeqs;
     // (8 waves only: with 4 waves a wave has twice the tile loads to address, and the 32 registers
     // the pipelined kernel leaves the compiler no longer hold that without spilling in the loop)
@@ -124,13 +123,15 @@ int launch(const KArgs& ka, const Plan& plan, hipStream_t st, const PlanArgs* pa
     constexpr int NW = 4 * NB;  // streaming paths: one 32-row query block per wave
     constexpr int kSlotBase = (HD == 128 ? 0 : 8) + (NB == 1 ? 0 : 4);
     if constexpr (PATH == 3) {
-        main_k = paged_attn_stream_fp8_kernel<HD, NW>;
-        using C = StreamCfg<HD, 1, NW, false, 1>;
+        // head_dim 128: one query block per wave, 4 or 8 waves; head_dim 64: 4 waves of 1 or 2 blocks
+        constexpr int FNB = HD == 128 ? 1 : NB, FNW = HD == 128 ? NW : 4;
+        main_k = paged_attn_stream_fp8_kernel<HD, FNB, FNW>;
+        using C = StreamCfg<HD, FNB, FNW, false, 1>;
         lds = C::LDS_BYTES;
         plan_k = paged_attn_plan_kernel<C::RT>;
-        fill_k = paged_attn_plan_fill_kernel<HD, 1, NW, false, 1>;
+        fill_k = paged_attn_plan_fill_kernel<HD, FNB, FNW, false, 1>;
         fill_lds = C::STAGES_OFF;
-        threads = 64 * NW;
+        threads = 64 * FNW;
         slot = kSlotBase + 3;
     } else if constexpr (PATH == 2) {
         // 4 waves for up to 128 rows (then two workgroups per compute unit where the batch allows),
@@ -268,7 +269,7 @@ uint32_t plan_signature(const dfx_attn_params* p, const Plan& plan) {
     return sig == 0 ? 1u : sig;
 }
 
-int plan_waves(const Plan& plan) { return plan.compact ? 4 : 4 * plan.nb; }
+int plan_waves(const Plan& plan) { return (plan.compact || (plan.fp8 && plan.hd == 64)) ? 4 : 4 * plan.nb; }
 
 // Checks and launch; `workspace` replaces p->workspace.  plan_out != nullptr: instead of the
 // attention launch, build its plan into plan_out (plan_bytes of room).
@@ -364,9 +365,7 @@ int run_paged_attn(const dfx_attn_params* p, void* workspace, int64_t workspace_
     const PlanArgs* pap = plan_out != nullptr ? &pa : nullptr;
 #define DFX_ATTN_CASE(HD_, NB_)                                               \
     if (plan.hd == HD_ && plan.nb == NB_) {                                   \
-        if (plan.stream && plan.fp8) {                                        \
-            if constexpr (HD_ == 128) return launch<HD_, NB_, 3>(ka, plan, st, pap); \
-        }                                                                     \
+        if (plan.stream && plan.fp8) return launch<HD_, NB_, 3>(ka, plan, st, pap); \
         if (plan.stream) return launch<HD_, NB_, 2>(ka, plan, st, pap);       \
         if (plan.distinct) return launch<HD_, NB_, 4>(ka, plan, st, pap);     \
         if (plan.fp8) return launch<HD_, NB_, 1>(ka, plan, st, pap);          \

@@ -122,6 +122,10 @@ FP8_EDGE_CASES = [
     dict(num_seqs=2, h_q=8, h_kv=1, hd=128, page=32, ctx=[100, 200], q_len=64, dbs=64),
     dict(num_seqs=3, h_q=6, h_kv=3, hd=128, page=24, ctx=[23, 24, 100], q_len=32, dbs=32),
     dict(num_seqs=70, h_q=4, h_kv=1, hd=128, page=64, ctx=(0, 200), q_len=32, dbs=32),   # more units than one plan holds
+    # head_dim 64: 4 waves with one (up to 128 rows) or two (up to 256 rows) query blocks each, several row tiles
+    dict(num_seqs=4, h_q=8, h_kv=2, hd=64, page=32, ctx=[0, 63, 64, 500], q_len=32, dbs=32),
+    dict(num_seqs=3, h_q=14, h_kv=2, hd=64, page=256, ctx=[255, 700, 1300], q_len=32, dbs=32),
+    dict(num_seqs=3, h_q=16, h_kv=2, hd=64, page=16, ctx=[100, 300, 17], q_len=64, dbs=32),
 ]
 
 
@@ -135,6 +139,8 @@ def test_fp8_edge_cases(dev, case, mask, flags):
     for max_wg in (1, 5, 0):
         got = _run(g, max_wg, flags=flags)
         assert max_abs_err(got, want) <= ATOL_FP8
+    if flags == 0:
+        assert torch.equal(_run(g, 0, plan_cache={}), _run(g, 0))   # a planned launch gives the same bits
 
 
 def test_fresh_k_and_v_with_different_strides(dev):

@@ -58,8 +58,8 @@ KERNELS = [
     ("_ZN3dfx24paged_attn_stream_kernelILi128ELi1ELi4ELb0E", 3),
     ("_ZN3dfx24paged_attn_stream_kernelILi64ELi1ELi8ELb0E", 3),
     ("_ZN3dfx24paged_attn_stream_kernelILi64ELi1ELi4ELb1E", 3),
-    ("_ZN3dfx28paged_attn_stream_fp8_kernelILi128ELi8E", 3 + 2),
-    ("_ZN3dfx28paged_attn_stream_fp8_kernelILi128ELi4E", 3 + 3),
+    ("_ZN3dfx28paged_attn_stream_fp8_kernelILi128ELi1ELi8E", 3 + 2),
+    ("_ZN3dfx28paged_attn_stream_fp8_kernelILi128ELi1ELi4E", 3 + 3),
 ]
 
 

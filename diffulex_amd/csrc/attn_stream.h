@@ -358,22 +358,36 @@ struct StreamAttn : TileMath<HD, NB, NW, HIDDEN> {
         if (wait) touch_queries();
     }
 
-    // Pipelined kernel: adopt the item of unit d; its query rows go into the Q operand registers
-    // and O^T is cleared (attn_pipe_gen.h).  Waits for every outstanding load of the wave.
-    DFX_D void begin_item_hidden(const UnitDesc& d) {
+    // Pipelined kernel.  The query rows of an item go straight into the Q operand registers
+    // (attn_pipe_gen.h), which no matrix instruction reads during the last step of the item before:
+    // request_queries(d) may be called from there on, adopt_item(d) once that item is finished and
+    // the loads have been waited for.
+    DFX_D void request_queries(const UnitDesc& d) const {
         static_assert(HIDDEN, "pipelined kernel only");
+        const int q_len = uniform(d.q_len);
+        const int r = this->row_of(uniform(d.rt), 0);
+        const bool valid = r < a.group * q_len;
+        const int g = valid ? r / q_len : 0;
+        const int i = valid ? r - g * q_len : 0;
+        // (lanes without a row read row 0 of the item: finite data whose results are never stored)
+        pipe_issue_queries(a.q + (uniform(d.q0) + i) * a.q_st + (uniform(d.kvh) * a.group + g) * a.q_sh + half * 8);
+    }
+    DFX_D void adopt_item(const UnitDesc& d) {
         this->s = uniform(d.s);
         this->kvh = uniform(d.kvh);
         this->q0 = uniform(d.q0);
         this->sh.q_len = uniform(d.q_len);
         const int r = this->row_of(uniform(d.rt), 0);
         const bool valid = r < a.group * this->sh.q_len;
-        const int g = valid ? r / this->sh.q_len : 0;
-        const int i = valid ? r - g * this->sh.q_len : 0;
+        const int i = valid ? r % this->sh.q_len : 0;
         this->vis_limit[0] = (i / a.dbs + 1) * a.dbs;
-        const uint16_t* qp = a.q + (this->q0 + i) * a.q_st + (this->kvh * a.group + g) * a.q_sh + half * 8;
-        pipe_load_queries(qp, __ballot(valid));
         this->reset_accumulators();
+    }
+    // Both at once, waiting for every outstanding load of the wave.
+    DFX_D void begin_item_hidden(const UnitDesc& d) {
+        request_queries(d);
+        wait_async_loads<0>();
+        adopt_item(d);
     }
 
     DFX_D TileInfo tile_info_of(int rel) const {
@@ -623,6 +637,9 @@ paged_attn_pipe_kernel(const KArgs a) {
     static_assert(kHoleRows == 8 || kHoleRows == 16, "mask blocks of attn_pipe_gen.h");
     at.for_each_chunk([&](int n_units) {
         const WgSplit& split = at.split;
+        // An item that opens with this chunk: its query rows first.  Requested behind the ring fill,
+        // the wait for them would also wait for every tile of the fill.
+        if (uniform(at.units[0].flags) & kUnitFirst) at.begin_item_hidden(at.units[0]);
         int issued = 0;  // ring fill: kStages - 1 units in flight
         for (; issued < C::kStages - 1 && issued < n_units; ++issued) at.issue_unit(issued);
 
@@ -665,7 +682,7 @@ paged_attn_pipe_kernel(const KArgs a) {
             // a run of units of one item: all of this workgroup's piece of it, or up to the end of the plan
             const UnitDesc d = at.units[rel];
             const int run_end = min(rel + uniform(d.run), n_units);
-            if (uniform(d.flags) & kUnitFirst) at.begin_item_hidden(d);
+            // (an item that opens inside the chunk was adopted when the run before it ended)
 
             // S^T of the run's first tile (into score set A), with nothing to overlap it with
             if (admit(rel, rel)) at.issue_unit(issued++);
@@ -691,9 +708,14 @@ paged_attn_pipe_kernel(const KArgs a) {
                 if (compute_first) prepare();
             }
             // step r: softmax and O^T of unit r, S^T of unit r + 1; the two score sets swap roles
+            // The next item of this chunk, if there is one: its query rows are requested in the last
+            // step of this run and waited for behind that step's matrix work, one step later than the
+            // youngest tile load in flight was issued, instead of in front of an idle matrix unit.
+            const bool next_opens = run_end < n_units;
             auto step = [&](int r, bool cur_is_a) {
                 const bool has_next = r + 1 < run_end;
                 const bool fetch = has_next && admit(r + 1, r);
+                if (!has_next && next_opens) at.request_queries(at.units[run_end]);
                 if (!compute_first || !busy) {
                     if (fetch) at.issue_unit(issued);
                     if (busy) prepare();
@@ -730,7 +752,9 @@ paged_attn_pipe_kernel(const KArgs a) {
                 step(rel++, true);
                 if (rel < run_end) step(rel++, false);
             }
+            if (next_opens) wait_async_loads<0>();  // the next item's query rows (and the tiles requested before them)
             at.finish_run(rel - 1, split);
+            if (next_opens) at.adopt_item(at.units[run_end]);
         }
     });
 }

@@ -338,17 +338,13 @@ namespace dfx {
         resc += [f"v_accvgpr_write_b32 {ar(O_BASE + i)}, {vr(TMP + i - g)}" for i in range(g, g + 4)]
     parts.append(asm_fn("pipe_rescale_outputs", "float alpha", join(resc), ins=['[alpha] "v"(alpha)'],
                         comment="O^T *= alpha (per lane: one query row per lane column), behind the wait states for the matrix results."))
-    # queries: 8 x 16-byte loads of the lane's row half into score set A (dead when an item begins),
-    # zeroed for lanes without a row, then into the Q operand registers
-    ql = [f"global_load_dwordx4 {vr(SA + 4 * s, 4)}, %[p], off offset:{s * 32}" for s in range(NSLAB)]
-    ql.append("s_waitcnt vmcnt(0)")
-    ql += [f"v_cndmask_b32 {vr(SA + i)}, 0, {vr(SA + i)}, %[valid]" for i in range(4 * NSLAB)]
-    ql += [f"v_accvgpr_write_b32 {ar(Q_BASE + i)}, {vr(SA + i)}" for i in range(4 * NSLAB)]
-    parts.append(asm_fn("pipe_load_queries", "const void* row, uint64_t valid", join(ql),
-                        ins=['[p] "v"(row)', '[valid] "s"(valid)'], clobbers=["memory"],
-                        comment="Q operand: the lane's half (64 bytes of every 128: slab s at byte 32 s) of its query row at `row`,\n"
-                                "zeros for lanes whose bit in `valid` is clear (their `row` must still be readable).  Waits for\n"
-                                "every outstanding vector memory operation of the wave (vmcnt(0))."))
+    # queries: 8 x 16-byte loads of the lane's row half straight into the Q operand registers
+    ql = [f"global_load_dwordx4 {ar(Q_BASE + 4 * s, 4)}, %[p], off offset:{s * 32}" for s in range(NSLAB)]
+    parts.append(asm_fn("pipe_issue_queries", "const void* row", join(ql), ins=['[p] "v"(row)'], clobbers=["memory"],
+                        comment="Q operand: requests the lane's half (64 bytes of every 128: slab s at byte 32 s) of the query row at\n"
+                                "`row` (lanes without a row of their own pass any readable row: their columns of S^T and O^T are\n"
+                                "never stored).  The caller waits for the loads (vmcnt) before the next matrix instruction, and\n"
+                                "no matrix instruction that reads the previous Q operand may still be in flight."))
     for d in range(NDB):
         outs = [f'"=v"(x[{e}])' for e in range(16)]
         body = join(f"v_accvgpr_read_b32 %{e}, {ar(O_BASE + 16 * d + e)}" for e in range(16))

@@ -94,13 +94,13 @@ kv_store_distinct_kernel(const uint16_t* __restrict__ key, const uint16_t* __res
     v_cache[blk * st.v[0] + h * st.v[1] + d * st.v[2] + off * st.v[3]] = value[t * value_stride + e];
 }
 
-// The same store for x == 8 two-byte elements and dense inner dimensions, 64 tokens of one head per
+// The same store for x == 8 two-byte elements and dense inner dimensions, 16 tokens of one head per
 // workgroup, staged through LDS so that both sides move 16 bytes per lane: rows are read the way
 // they lie in the operands (256 contiguous bytes per token and head), K leaves as one chunk
 // column of consecutive tokens (their 16-byte pieces are adjacent in the cache when their slots
 // are), and V leaves transposed, eight consecutive tokens of one d per store where those eight
 // have consecutive slots starting at a multiple of 8 in one page (two bytes at a time otherwise).
-constexpr int kDistinctTokens = 64;
+constexpr int kDistinctTokens = 16;
 
 template <typename SlotT, int HD>
 __global__ void __launch_bounds__(kThreads)

@@ -30,7 +30,8 @@ GIB = 1 << 30
 
 
 def short(name: str) -> str:
-    return name.split("(")[0].replace("void dfx::(anonymous namespace)::", "").replace("void dfx::", "")[-90:]
+    name = name.replace("(anonymous namespace)::", "")
+    return name.split("(")[0].replace("void dfx::", "").replace("void ", "")[-90:]
 
 
 def kernel_stats(d):
@@ -58,7 +59,25 @@ def main():
     ap.add_argument("--dir", required=True)
     ap.add_argument("--kernel", default="paged_attn", help="substring naming the kernel whose traffic is recorded")
     ap.add_argument("--write-traffic", action="store_true")
+    ap.add_argument("--counters", nargs="*", default=[],
+                    help="sub-directories of --dir holding other `rocprofv3 --pmc ...` runs of the same command: their "
+                         "counters are listed as means per dispatch of the kernel named by --kernel")
     args = ap.parse_args()
+    if args.counters:
+        print(f"## counters of `{args.kernel}` kernels, workload {args.workload} (mean per dispatch, summed over the chip)\n")
+        print("| counter | kernel | mean per dispatch | dispatches |")
+        print("|---|---|---|---|")
+        for sub in args.counters:
+            total, count = collections.defaultdict(float), collections.Counter()
+            for fn in glob.glob(os.path.join(args.dir, sub, "**", "*counter_collection.csv"), recursive=True):
+                for r in csv.DictReader(open(fn)):
+                    k = short(r["Kernel_Name"])
+                    if args.kernel in k and "plan" not in k:
+                        total[(r["Counter_Name"], k)] += float(r["Counter_Value"])
+                        count[(r["Counter_Name"], k)] += 1
+            for (c, k) in sorted(total):
+                print(f"| `{c}` | `{k}` | {total[(c, k)] / count[(c, k)]:,.0f} | {count[(c, k)]} |")
+        return
 
     bench = None
     path = os.path.join(args.dir, "bench.json")

@@ -270,14 +270,17 @@ struct AttnState {
             mx = wave_xor32_max(mx);
             const float m_tile = mx * t.c_tile;
             if (__any(m_tile > m_run[qb] + kRescaleThreshold)) {
-                before_rescale();
                 const float m_new = fmaxf(m_run[qb], m_tile);
-                const float alpha = (m_new == -INFINITY) ? 1.0f : fast_exp2(m_run[qb] - m_new);
-                l_run[qb] *= alpha;
+                // (the first tile of a piece finds every row at -inf and O^T at zero: nothing to rescale)
+                if (__any(m_run[qb] != -INFINITY)) {
+                    before_rescale();
+                    const float alpha = (m_new == -INFINITY) ? 1.0f : fast_exp2(m_run[qb] - m_new);
+                    l_run[qb] *= alpha;
 #pragma unroll
-                for (int db = 0; db < S::NDB; ++db)
+                    for (int db = 0; db < S::NDB; ++db)
 #pragma unroll
-                    for (int e = 0; e < 16; ++e) o[db][qb][e] *= alpha;
+                        for (int e = 0; e < 16; ++e) o[db][qb][e] *= alpha;
+                }
                 m_run[qb] = m_new;
             }
             const float m_safe = (m_run[qb] == -INFINITY) ? 0.0f : m_run[qb];

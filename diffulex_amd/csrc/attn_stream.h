@@ -695,9 +695,12 @@ paged_attn_pipe_kernel(const KArgs a) {
                 float& m_run = at.m_run[0];
                 if (__any(m_tile > m_run + kRescaleThreshold)) {
                     const float m_new = fmaxf(m_run, m_tile);
-                    const float alpha = (m_new == -INFINITY) ? 1.0f : fast_exp2(m_run - m_new);
-                    at.l_run[0] *= alpha;
-                    pipe_rescale_outputs(alpha);
+                    // (the first tile of a piece finds every row at -inf and O^T at zero: nothing to rescale)
+                    if (__any(m_run != -INFINITY)) {
+                        const float alpha = (m_new == -INFINITY) ? 1.0f : fast_exp2(m_run - m_new);
+                        at.l_run[0] *= alpha;
+                        pipe_rescale_outputs(alpha);
+                    }
                     m_run = m_new;
                 }
                 neg_m = (m_run == -INFINITY) ? 0.0f : -m_run;

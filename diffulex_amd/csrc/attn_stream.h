@@ -253,6 +253,14 @@ struct StreamAttn : TileMath<HD, NB, NW, HIDDEN> {
         const bool is_ctx = tag > 0;
         const int64_t off = (static_cast<int64_t>(uniform(static_cast<int>(b.off >> 32))) << 32) |
                             static_cast<uint32_t>(uniform(static_cast<int>(b.off)));
+        if constexpr (HIDDEN && NW == 8 && KVB == 2) {
+            // the common case, a full band of cached rows: offsets precomputed per lane, no vector arithmetic
+            if (is_ctx && last >= C::ROWS_PER_WAVE - 1) {
+                pipe_issue_band(a.k_cache + off, a.v_cache + off,
+                                uniform(static_cast<int>(stages_lds + (rel % C::kStages) * C::STAGE_BYTES + wave * (C::IPW * 1024))));
+                return;
+            }
+        }
         const uint8_t* kbase = (is_ctx ? a.k_cache : reinterpret_cast<const uint8_t*>(a.k_new)) + off;
         // fresh V rows may lie further apart than fresh K rows (V a slice of a projection, K rotated
         // into a buffer of its own): same head offset, another token stride
@@ -631,6 +639,16 @@ paged_attn_pipe_kernel(const KArgs a) {
     using SA = StreamAttn<HD, 1, NW, false, 2, true>;
     SA at(a, smem);
     pipe_reserve();
+    {
+        uint32_t o[2];
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int r = j * C::RPI + at.lane / C::CPR;
+            const int chunk = (at.lane % C::CPR) ^ C::swizzle(at.wave * C::ROWS_PER_WAVE + r);
+            o[j] = static_cast<uint32_t>(r) * static_cast<uint32_t>(a.c_st * 2) + chunk * 16;
+        }
+        pipe_set_load_offsets(o[0], o[1]);
+    }
     store_fresh_rows<HD, false>(a);
     const bool busy = at.wave < a.busy_waves;  // waves whose 32 rows exist in no item of this launch only fetch
     constexpr int kHoleRows = C::ROWS_PER_WAVE;

@@ -23,6 +23,7 @@ Register map (head_dim 128; one 32-row query block per wave; 128 + 128 registers
     v[80:111]  score set B
     v[112:127] operand ring: four 4-register buffers (K operands in phase X, V^T in phase Y)
     v[32:42]   temporaries: exp2 pair, K operand address, 8 V^T operand addresses
+    v[43:44]   the lane's byte offsets inside a band of cached rows (tile loads, pipe_issue_band)
     v[0:31], a[0:31]  the compiler's
 The two score sets swap roles every step (steps AB and BA), so nothing is ever moved.  P (the
 bf16 pairs, the B operand of the second product) overwrites the current score set as it is
@@ -56,6 +57,8 @@ SA, SB, RING = 48, 80, 112
 T_EXP = [TMP + 0, TMP + 1]  # exp2 arguments / results of the pair in flight
 T_ADDR = TMP + 2            # K operand address of the slab being read (phase X); scratch elsewhere
 T_VADDR = TMP + 3           # 8 V^T operand addresses (phase Y)
+LOAD_OFF = 43               # two registers: byte offsets of the lane's chunk in its two rows of a band of cached rows
+MAT_BYTES = 64 * ROWB       # K tile; the V tile of a ring stage follows it
 NEG_INF = "0xff800000"
 MFMA_TO_VALU = ["s_nop 15", "s_nop 1"]  # 18 wait states: the longest the ISA asks for
 
@@ -345,6 +348,19 @@ namespace dfx {
                                 "`row` (lanes without a row of their own pass any readable row: their columns of S^T and O^T are\n"
                                 "never stored).  The caller waits for the loads (vmcnt) before the next matrix instruction, and\n"
                                 "no matrix instruction that reads the previous Q operand may still be in flight."))
+    parts.append(asm_fn("pipe_set_load_offsets", "uint32_t o0, uint32_t o1",
+                        join(f"v_mov_b32 {vr(LOAD_OFF + j)}, %{j}" for j in range(2)), ins=['"v"(o0)', '"v"(o1)'],
+                        comment="Once per kernel: the lane's byte offsets (row * row stride + swizzled chunk * 16) for the two\n"
+                                "wave-wide loads that fetch its wave's 8 rows of a tile of cached rows."))
+    issue = []
+    for j in range(2):
+        issue += [f"s_add_u32 m0, %[d], {j * 1024}", f"global_load_lds_dwordx4 {vr(LOAD_OFF + j)}, %[kb] nt",
+                  f"s_add_u32 m0, %[d], {MAT_BYTES + j * 1024}", f"global_load_lds_dwordx4 {vr(LOAD_OFF + j)}, %[vb] nt"]
+    parts.append(asm_fn("pipe_issue_band", "const void* k_rows, const void* v_rows, uint32_t lds_dst", join(issue),
+                        ins=['[kb] "s"(k_rows)', '[vb] "s"(v_rows)', '[d] "s"(lds_dst)'], clobbers=["memory", "m0", "scc"],
+                        comment="The wave's four direct-to-LDS loads of a tile whose 8 rows of the wave are all cached rows (K rows at\n"
+                                "k_rows, V rows at v_rows, both wave-uniform; lds_dst: the wave's place in the K tile of the ring stage):\n"
+                                "no vector instruction, the offsets are those of pipe_set_load_offsets."))
     for d in range(NDB):
         outs = [f'"=v"(x[{e}])' for e in range(16)]
         body = join(f"v_accvgpr_read_b32 %{e}, {ar(O_BASE + 16 * d + e)}" for e in range(16))

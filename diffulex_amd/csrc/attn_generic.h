@@ -28,7 +28,7 @@ struct GenericCfg : Shape<HD, NB> {
 
 // DISTINCT: the cache is in the "distinct" layout, K [pages, H, hd / 8, page, 8] and V [pages, H,
 // hd, page] (bf16): a 16-byte load still brings one 8-element chunk of a K row, but 8 consecutive
-// tokens of one d for V, which are scattered into the row-major LDS tile two bytes at a time.
+// tokens of one d for V -- one chunk of a d-major V tile, which is what the V^T operand reads.
 template <int HD, int NB, bool FP8, bool DISTINCT = false>
 struct GenericAttn : TileMath<HD, NB, kWaves> {
     using Base = TileMath<HD, NB, kWaves>;
@@ -101,58 +101,107 @@ struct GenericAttn : TileMath<HD, NB, kWaves> {
     // consecutive tokens (1 KiB contiguous inside a page); V: eight consecutive lanes take the
     // eight 8-token groups of one d (128 contiguous bytes).
     DFX_D void issue_distinct(int base, int limit) {
-        const uint16_t* kc = reinterpret_cast<const uint16_t*>(a.k_cache);
-        const uint16_t* vc = reinterpret_cast<const uint16_t*>(a.v_cache);
+        static_assert(kThreads % C::TN == 0 && kThreads % 8 == 0, "a thread's chunks share their token (K) and token group (V)");
+        // K: chunk c = tid + kThreads * i is (token c % TN, chunk column c / TN): one token per thread
+        {
+            const int tok = base + tid % C::TN;
+            bool ok = tok < limit;
+            int off = 0;
+            int64_t page = 0;
+            if (ok) page = page_of(tok, ok, off);
+            const uint16_t* kp = reinterpret_cast<const uint16_t*>(a.k_cache) + (ok ? page * a.kd_sp + kvh * a.kd_sh + off * 8 : 0) +
+                                 (tid / C::TN) * a.kd_sc;
 #pragma unroll
-        for (int i = 0; i < C::CH16; ++i) {
-            const int c = tid + kThreads * i;
-            {
-                const int row = c % C::TN, cc = c / C::TN;
-                const int tok = base + row;
-                bool ok = tok < limit;
+            for (int i = 0; i < C::CH16; ++i) {
                 u32x4 kk = {0, 0, 0, 0};
-                if (ok) {
-                    int off;
-                    const int64_t page = page_of(tok, ok, off);
-                    if (ok) kk = *reinterpret_cast<const u32x4*>(kc + page * a.kd_sp + kvh * a.kd_sh + cc * a.kd_sc + off * 8);
-                }
+                if (ok) kk = *reinterpret_cast<const u32x4*>(kp + i * (kThreads / C::TN) * a.kd_sc);
                 kst[i] = kk;
             }
-            {
-                const int tg = c % 8, d = c / 8;
-                const int tok = base + tg * 8;
-                bool ok = tok < limit;
-                u32x4 vv = {0, 0, 0, 0};
-                if (ok) {
-                    int off;  // a multiple of 8: pages hold a multiple of 8 tokens
-                    const int64_t page = page_of(tok, ok, off);
-                    if (ok) vv = *reinterpret_cast<const u32x4*>(vc + page * a.vd_sp + kvh * a.vd_sh + d * a.vd_sd + off);
-                    const int n_valid = limit - tok;  // tokens past the end of the context read as zeros
-                    if (n_valid < 8) {
+        }
+        // V: chunk c is (token group c % 8, d = c / 8): one group of 8 tokens per thread
+        {
+            const int tok = base + (tid % 8) * 8;
+            bool ok = tok < limit;
+            int off = 0;  // a multiple of 8: pages hold a multiple of 8 tokens
+            int64_t page = 0;
+            if (ok) page = page_of(tok, ok, off);
+            const uint16_t* vp = reinterpret_cast<const uint16_t*>(a.v_cache) + (ok ? page * a.vd_sp + kvh * a.vd_sh + off : 0) +
+                                 (tid / 8) * a.vd_sd;
 #pragma unroll
-                        for (int j = 0; j < 8; ++j) {
-                            if (j >= n_valid) vv[j >> 1] &= (j & 1) ? 0x0000ffffu : 0xffff0000u;
-                        }
-                    }
-                }
+            for (int i = 0; i < C::CH16; ++i) {
+                u32x4 vv = {0, 0, 0, 0};
+                if (ok) vv = *reinterpret_cast<const u32x4*>(vp + i * (kThreads / 8) * a.vd_sd);
                 vst[i] = vv;
+            }
+            // tokens past the end of the context read as zeros (the group that holds the end only):
+            // a mask per 32-bit word of two tokens
+            const int n_valid = limit - tok;
+            if (ok && n_valid < 8) {
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    const uint32_t keep = (2 * k < n_valid ? 0x0000ffffu : 0u) | (2 * k + 1 < n_valid ? 0xffff0000u : 0u);
+#pragma unroll
+                    for (int i = 0; i < C::CH16; ++i) vst[i][k] &= keep;
+                }
             }
         }
     }
 
+    // The V tile stays d-major in LDS, as it is in the distinct layout: row d holds the tile's 64
+    // tokens (128 bytes, eight 16-byte chunks), which is the V^T operand's shape already.  Inside
+    // a 16-token slab the matrix instruction's contraction index runs over tokens 0-3, 8-11 (lower
+    // half of the wave) and 4-7, 12-15 (upper half), as the score registers hold them; the two
+    // chunks of a slab are stored in that order, so that a lane's operand is one 16-byte read:
+    // chunk 2 * slab + h = tokens 4h..4h+3 then 8+4h..8+4h+3 of the slab.  Chunks are swizzled by
+    // (d / 2) % 8: 16 consecutive d of one chunk column then cover all 64 banks once.
+    DFX_HD static int vt_chunk_offset(int d, int chunk) { return d * (C::TN * 2) + ((chunk ^ ((d >> 1) & 7)) * 16); }
+    // byte offset of token `tok` (0..63) of row d
+    DFX_HD static int vt_token_offset(int d, int tok) {
+        const int r16 = tok & 15;
+        return vt_chunk_offset(d, (tok >> 4) * 2 + ((r16 >> 2) & 1)) + ((r16 >> 3) * 4 + (r16 & 3)) * 2;
+    }
+
     DFX_D void commit_distinct(uint8_t* ks, uint8_t* vs) const {
+        int t = tid;
+        asm volatile("" : "+v"(t));  // (addresses worked out here, not kept as invariants of the tile loop: see commit())
 #pragma unroll
         for (int i = 0; i < C::CH16; ++i) {
-            const int c = tid + kThreads * i;
+            const int c = t + kThreads * i;
             *reinterpret_cast<u32x4*>(ks + L::chunk_offset(c % C::TN, c / C::TN)) = kst[i];
+            // a chunk of the cache is tokens 8 tg .. 8 tg + 7 of one d: its halves go to the slab's two chunks
             const int tg = c % 8, d = c / 8;
-#pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                const uint32_t w = vst[i][j >> 1];
-                *reinterpret_cast<uint16_t*>(vs + L::chunk_offset(tg * 8 + j, d >> 3) + (d & 7) * 2) =
-                    static_cast<uint16_t>((j & 1) ? (w >> 16) : w);
-            }
+            const u32x2 lo = {vst[i][0], vst[i][1]}, hi = {vst[i][2], vst[i][3]};
+            *reinterpret_cast<u32x2*>(vs + vt_token_offset(d, tg * 8)) = lo;
+            *reinterpret_cast<u32x2*>(vs + vt_token_offset(d, tg * 8 + 4)) = hi;
         }
+    }
+
+    // O^T += V^T P^T from a d-major V tile (commit_distinct): the operand of (token slab tb, sl; d
+    // block db) is one 16-byte read per lane, row db * 32 + col, chunk tb * 4 + sl * 2 + half.
+    DFX_D void accumulate_dmajor(const uint8_t* v_tile, const bf16x8 (&pb)[NB][2][2]) {
+        using S = typename Base::S;
+        typedef __attribute__((address_space(3))) bf16x8 lds_bf16x8;
+        constexpr int kSteps = 4 * S::NDB;  // (tb, sl, db)
+        // Row db * 32 + col, chunk (tb * 4 + sl * 2 + half) ^ swizzle: the swizzle depends on col only and
+        // tb * 4 + sl * 2 is even, so the lane's part of the address is one constant, the slab an XOR
+        // on bits 5..6 of the finished address (tiles start at multiples of 256) and the d block an
+        // immediate offset -- four address registers instead of one per operand.
+        const uint32_t v0 = Base::lds_address(v_tile) + static_cast<uint32_t>(vt_chunk_offset(col, half));
+        auto read = [&](int st) {
+            const int tb = st / (2 * S::NDB), sl = (st / S::NDB) & 1, db = st % S::NDB;
+            return *(const lds_bf16x8*)static_cast<uintptr_t>((v0 ^ ((tb * 4 + sl * 2) * 16)) + db * 32 * (C::TN * 2));
+        };
+        bf16x8 va[3];
+        va[0] = read(0);
+        va[1] = read(1);
+#pragma unroll
+        for (int st = 0; st < kSteps; ++st) {
+            const int tb = st / (2 * S::NDB), sl = (st / S::NDB) & 1, db = st % S::NDB;
+            if (st + 2 < kSteps) va[(st + 2) % 3] = read(st + 2);
+#pragma unroll
+            for (int qb = 0; qb < NB; ++qb) mfma_output(o[db][qb], va[st % 3], pb[qb][tb][sl]);
+        }
+        this->outputs_ready();
     }
 
     // global -> registers (rows past the end of the sequence become zeros)
@@ -235,12 +284,27 @@ struct GenericAttn : TileMath<HD, NB, kWaves> {
             }
         } else {
             constexpr int CPR = HD / 8;
+            int t = tid;
+            // (fresh rows of the distinct kernel, one tile per item: their 8 * CH16 scatter addresses are
+            // worked out here, from a thread number the compiler cannot follow -- as loop invariants of
+            // the tile loop they would take more registers than there are, for both tile buffers)
+            if constexpr (DISTINCT) asm volatile("" : "+v"(t));
 #pragma unroll
             for (int i = 0; i < C::CH16; ++i) {
-                const int c = tid + kThreads * i;
+                const int c = t + kThreads * i;
                 const int row = c / CPR, cc = c % CPR;
                 *reinterpret_cast<u32x4*>(ks + L::chunk_offset(row, cc)) = kst[i];
-                *reinterpret_cast<u32x4*>(vs + L::chunk_offset(row, cc)) = vst[i];
+                if constexpr (DISTINCT) {
+                    // into the d-major V tile, two bytes at a time
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) {
+                        const uint32_t w = vst[i][j >> 1];
+                        *reinterpret_cast<uint16_t*>(vs + vt_token_offset(cc * 8 + j, row)) =
+                            static_cast<uint16_t>((j & 1) ? (w >> 16) : w);
+                    }
+                } else {
+                    *reinterpret_cast<u32x4*>(vs + L::chunk_offset(row, cc)) = vst[i];
+                }
             }
         }
     }
@@ -259,7 +323,8 @@ struct GenericAttn : TileMath<HD, NB, kWaves> {
         this->scores(k_stage(buf), sc);
         bf16x8 pb[NB][2][2];
         this->template softmax_tile<FP8, 1>(sc, t, pb, [&] { this->outputs_ready(); });
-        this->accumulate(v_stage(buf), pb);
+        if constexpr (DISTINCT) accumulate_dmajor(v_stage(buf), pb);  // (one form for every tile: two, chosen at run time, would
+        else this->accumulate(v_stage(buf), pb);                      //  have the accumulators copied where the paths meet)
     }
 
     DFX_D void run_segment(int rt, int tile0, int tile1, int item_tiles, int64_t item_begin, const WgSplit& split) {

@@ -81,7 +81,10 @@ DFX_HD PlanLayout plan_layout(int num_seqs, int n_wg, int64_t capacity, int wave
     return l;
 }
 
-enum : int32_t { kUnitCtx = 1, kUnitFirst = 2, kUnitLast = 4, kUnitComplete = 8, kUnitHoleShift = 8 };
+// UnitDesc::flags: bits 8..15 a bit per band of rows whose page is missing (holes); bits 16..21, set by
+// mark_plain_steps() only, the number of consecutive plain steps that begin with this unit
+enum : int32_t { kUnitCtx = 1, kUnitFirst = 2, kUnitLast = 4, kUnitComplete = 8, kUnitHoleShift = 8, kUnitPlainShift = 16 };
+DFX_HD uint32_t unit_holes(int flags) { return (static_cast<uint32_t>(flags) >> kUnitHoleShift) & 0xffu; }
 
 // COMPACT: a configuration small enough (2 stages, short plan, at most kCompactMaxSeqs sequences)
 // for two workgroups to share a compute unit.  Items with at most 128 rows run with four waves,
@@ -157,6 +160,7 @@ struct StreamAttn : TileMath<HD, NB, NW, HIDDEN> {
     UnitDesc* units;
     BandDesc* bands;
     uint32_t stages_lds;  // LDS byte address of stage 0
+    int wave_s;           // the wave's number as a wave-uniform value (a scalar register from the start)
     int64_t begin, end;
     int64_t rel_base;  // what UnitDesc::item_rel is relative to: the first unit of the workgroup's work
     int per_head;
@@ -167,7 +171,8 @@ struct StreamAttn : TileMath<HD, NB, NW, HIDDEN> {
           misc(reinterpret_cast<int*>(smem + C::PREFIX_BYTES)),
           units(reinterpret_cast<UnitDesc*>(smem + C::UNIT_TABLE_OFF)),
           bands(reinterpret_cast<BandDesc*>(smem + C::BAND_TABLE_OFF)),
-          stages_lds(static_cast<uint32_t>(reinterpret_cast<uintptr_t>(smem)) + C::STAGES_OFF) {}
+          stages_lds(static_cast<uint32_t>(reinterpret_cast<uintptr_t>(smem)) + C::STAGES_OFF),
+          wave_s(uniform(static_cast<int>(threadIdx.x >> 6))) {}
 
     // ---- planning --------------------------------------------------------------------------
     // Describe units [first, first + count) in the plan table (entry i is unit first + i); one
@@ -257,7 +262,7 @@ struct StreamAttn : TileMath<HD, NB, NW, HIDDEN> {
             // the common case, a full band of cached rows: offsets precomputed per lane, no vector arithmetic
             if (is_ctx && last >= C::ROWS_PER_WAVE - 1) {
                 pipe_issue_band(a.k_cache + off, a.v_cache + off,
-                                uniform(static_cast<int>(stages_lds + (rel % C::kStages) * C::STAGE_BYTES + wave * (C::IPW * 1024))));
+                                uniform(static_cast<int>(stages_lds + (static_cast<unsigned>(rel) % C::kStages) * C::STAGE_BYTES + wave * (C::IPW * 1024))));
                 return;
             }
         }
@@ -268,7 +273,7 @@ struct StreamAttn : TileMath<HD, NB, NW, HIDDEN> {
                                       : reinterpret_cast<const uint8_t*>(a.v_new) + off + static_cast<int64_t>(-1 - tag) * a.v_fresh_delta;
         const uint32_t row_stride = static_cast<uint32_t>(is_ctx ? a.c_st * KVB : a.kn_st * 2);
         const uint32_t row_stride_v = static_cast<uint32_t>(is_ctx ? a.c_st * KVB : a.vn_st * 2);
-        const uint32_t dst = stages_lds + (rel % C::kStages) * C::STAGE_BYTES + wave * (C::IPW * 1024);
+        const uint32_t dst = stages_lds + (static_cast<unsigned>(rel) % C::kStages) * C::STAGE_BYTES + wave * (C::IPW * 1024);
 #pragma unroll
         for (int j = 0; j < C::IPW; ++j) {
             const int r = j * C::RPI + lane / C::CPR;  // row inside the band
@@ -296,7 +301,7 @@ struct StreamAttn : TileMath<HD, NB, NW, HIDDEN> {
         const bool is_ctx = tag > 0;
         uint8_t* kt = wide_tile(rel);
         uint8_t* vt = kt + L::MAT_BYTES;
-        const uint8_t* raw = lds + C::STAGES_OFF + (rel % C::kStages) * C::STAGE_BYTES + wave * (C::IPW * 1024) + lane * 16;
+        const uint8_t* raw = lds + C::STAGES_OFF + (static_cast<unsigned>(rel) % C::kStages) * C::STAGE_BYTES + wave * (C::IPW * 1024) + lane * 16;
         if (is_ctx) {
 #pragma unroll
             for (int j = 0; j < C::IPW; ++j) {
@@ -385,11 +390,16 @@ struct StreamAttn : TileMath<HD, NB, NW, HIDDEN> {
         this->kvh = uniform(d.kvh);
         this->q0 = uniform(d.q0);
         this->sh.q_len = uniform(d.q_len);
-        const int r = this->row_of(uniform(d.rt), 0);
-        const bool valid = r < a.group * this->sh.q_len;
-        const int i = valid ? r % this->sh.q_len : 0;
-        this->vis_limit[0] = (i / a.dbs + 1) * a.dbs;
         this->reset_accumulators();
+    }
+    // First key position the lane's query row does not see under the block-causal mask (fresh tiles
+    // only).  Worked out where a tile needs it, once or twice per item, rather than kept per item: a
+    // value that lives through the tile loop takes one of the few registers the compiler has there.
+    DFX_D int visible_limit(const UnitDesc& d) const {
+        const int q_len = uniform(d.q_len);
+        const int r = this->row_of(uniform(d.rt), 0);
+        const int i = r < a.group * q_len ? r % q_len : 0;
+        return (i / a.dbs + 1) * a.dbs;
     }
     // Both at once, waiting for every outstanding load of the wave.
     DFX_D void begin_item_hidden(const UnitDesc& d) {
@@ -404,7 +414,7 @@ struct StreamAttn : TileMath<HD, NB, NW, HIDDEN> {
         t.base = uniform(u.base);
         t.limit = uniform(u.limit);
         t.is_ctx = (uniform(u.flags) & kUnitCtx) != 0;
-        t.holes = static_cast<uint32_t>(uniform(u.flags)) >> kUnitHoleShift;  // a bit per band of rows
+        t.holes = unit_holes(uniform(u.flags));
         t.c_tile = a.c;
         t.v_mul = 1.0f;
         return t;
@@ -424,6 +434,35 @@ struct StreamAttn : TileMath<HD, NB, NW, HIDDEN> {
         }
         return finish_cut_item(*this, uniform(e.rt), rel_base + uniform(e.item_rel), uniform(e.n_tiles), split,
                                uniform(e.partner), l_tot, misc + kMaxWaves + 1, rel_base) ? 3 : 2;
+    }
+
+    // Step r of the pipelined loop (softmax and O^T of unit r, S^T of unit r + 1, tile loads of unit
+    // r + 3) is "plain" if it needs none of the loop's case distinctions: unit r + 1 follows in the
+    // same run and needs no mask, and unit r + 3 is in the table with every wave's band a full band
+    // of cached rows.  Writes into the flags of every unit r the number of consecutive plain steps
+    // from step r on (kUnitPlainShift).  One wave, one lane per unit; the table is complete
+    // (barrier) and nobody else writes flags now; readers come behind a later barrier.
+    DFX_D void mark_plain_steps(int n_units) const {
+        static_assert(C::kPlanUnits <= 64, "a lane per unit of the table");
+        if (wave_s != NW - 1) return;
+        const int r = thread_number_here(0);
+        bool plain = false;
+        int flags = 0;
+        if (r + 3 < n_units) {
+            bool full = true;
+#pragma unroll
+            for (int w = 0; w < NW; ++w) {
+                const BandDesc& b = bands[(r + 3) * NW + w];
+                full = full && b.is_ctx > 0 && b.last >= C::ROWS_PER_WAVE - 1;
+            }
+            flags = units[r].flags;
+            const UnitDesc& nxt = units[r + 1];
+            const bool masked = nxt.base + C::TN > nxt.limit || unit_holes(nxt.flags) != 0 ||
+                                (!(nxt.flags & kUnitCtx) && a.mask_mode == DFX_MASK_BLOCK_CAUSAL);
+            plain = full && !(flags & kUnitLast) && !masked;
+        }
+        const uint64_t not_plain = ~(__ballot(plain) >> r);  // bit j: step r + j is not plain (bits past 63 - r: set)
+        if (plain) units[r].flags = flags | (__builtin_ctzll(not_plain) << kUnitPlainShift);
     }
 
     // ---- the workgroup's work -----------------------------------------------------------------
@@ -484,13 +523,16 @@ struct StreamAttn : TileMath<HD, NB, NW, HIDDEN> {
             const int n_units = static_cast<int>(min(static_cast<int64_t>(C::kPlanUnits), n_total - done));
             __syncthreads();  // every wave is done with the previous descriptors and their stages
             if (planned) {
-                // descriptors are multiples of 16 bytes: copied as such
+                // descriptors are multiples of 16 bytes: copied as such.  The lane's addresses are worked
+                // out here: computed ahead of the chunk loop they end up in scratch, and every reload is
+                // a trip to memory in front of the first tile.
+                const int t = thread_number_here(wave_s);
                 const u32x4* su = reinterpret_cast<const u32x4*>(g_units + w.ubase + done);
                 u32x4* du = reinterpret_cast<u32x4*>(units);
-                for (int i = tid; i < n_units * 3; i += C::THREADS) du[i] = su[i];
                 const u32x4* sb = reinterpret_cast<const u32x4*>(g_bands + (w.ubase + done) * NW);
                 u32x4* db = reinterpret_cast<u32x4*>(bands);
-                for (int i = tid; i < n_units * NW; i += C::THREADS) db[i] = sb[i];
+                for (int i = t; i < n_units * 3; i += C::THREADS) du[i] = su[i];
+                for (int i = t; i < n_units * NW; i += C::THREADS) db[i] = sb[i];
             } else {
                 plan_units(begin + done, n_units);
             }
@@ -544,10 +586,10 @@ __global__ void __launch_bounds__(64 * NW, COMPACT ? 2 : 1) paged_attn_stream_ke
                 t.base = uniform(u.base);
                 t.limit = uniform(u.limit);
                 t.is_ctx = (uniform(u.flags) & kUnitCtx) != 0;
-                t.holes = static_cast<uint32_t>(uniform(u.flags)) >> kUnitHoleShift;  // a bit per band of rows
+                t.holes = unit_holes(uniform(u.flags));
                 t.c_tile = a.c;
                 t.v_mul = 1.0f;
-                const uint8_t* k_tile = smem + C::STAGES_OFF + (rel % C::kStages) * C::STAGE_BYTES;
+                const uint8_t* k_tile = smem + C::STAGES_OFF + (static_cast<unsigned>(rel) % C::kStages) * C::STAGE_BYTES;
                 if (at.wave < a.busy_waves) {  // waves whose 32 rows exist in no item of this launch only fetch
                     f32x16 sc[2][NB];
                     at.scores(k_tile, sc);
@@ -605,7 +647,7 @@ __global__ void __launch_bounds__(64 * NW, 1) paged_attn_stream_fp8_kernel(const
                 t.base = uniform(u.base);
                 t.limit = uniform(u.limit);
                 t.is_ctx = (uniform(u.flags) & kUnitCtx) != 0;
-                t.holes = static_cast<uint32_t>(uniform(u.flags)) >> kUnitHoleShift;  // a bit per band of rows
+                t.holes = unit_holes(uniform(u.flags));
                 t.c_tile = t.is_ctx ? a.c * at.k_mul : a.c;
                 t.v_mul = t.is_ctx ? 1.0f : at.v_inv;
                 const uint8_t* k_tile = at.wide_tile(rel);
@@ -657,11 +699,22 @@ paged_attn_pipe_kernel(const KArgs a) {
         const WgSplit& split = at.split;
         // An item that opens with this chunk: its query rows first.  Requested behind the ring fill,
         // the wait for them would also wait for every tile of the fill.
-        if (uniform(at.units[0].flags) & kUnitFirst) at.begin_item_hidden(at.units[0]);
+        const bool opens = (uniform(at.units[0].flags) & kUnitFirst) != 0;
+        if (opens) at.request_queries(at.units[0]);
+        // While the query rows are on their way: the marks of the plain steps.  They are first read
+        // behind the barrier of the first run's first step; they only add bits to the flags that
+        // nobody looks at before.  (Not behind the ring fill: a spilled register reloaded here would
+        // wait for every tile of it.)
+        at.mark_plain_steps(n_units);
+        __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the marks are written before this wave reaches that barrier
+        if (opens) {
+            wait_async_loads<0>();
+            at.adopt_item(at.units[0]);
+        }
         int issued = 0;  // ring fill: kStages - 1 units in flight
         for (; issued < C::kStages - 1 && issued < n_units; ++issued) at.issue_unit(issued);
 
-        auto tile_of = [&](int r) { return smem + C::STAGES_OFF + (r % C::kStages) * C::STAGE_BYTES; };
+        auto tile_of = [&](int r) { return smem + C::STAGES_OFF + (static_cast<unsigned>(r) % C::kStages) * C::STAGE_BYTES; };
         // Unit r must have landed: only younger units may still be outstanding.  Behind the barrier
         // every wave has finished the units before `done` (their K and their V tile), and unit x
         // may overwrite the stage of unit x - kStages while x - kStages < done: `can_issue` says
@@ -683,7 +736,7 @@ paged_attn_pipe_kernel(const KArgs a) {
             const bool bc = !t.is_ctx && a.mask_mode == DFX_MASK_BLOCK_CAUSAL;
             if (!(t.base + C::TN > t.limit || t.holes != 0 || bc)) return;
             int lim = t.limit;
-            if (bc) lim = min(lim, at.vis_limit[0]);
+            if (bc) lim = min(lim, at.visible_limit(at.units[r]));
             const int thr = lim - t.base - 4 * at.half;
             const uint32_t holes = static_cast<uint32_t>(t.holes);
             if (set_a) {
@@ -704,6 +757,12 @@ paged_attn_pipe_kernel(const KArgs a) {
 
             // S^T of the run's first tile (into score set A), with nothing to overlap it with
             if (admit(rel, rel)) at.issue_unit(issued++);
+            // For the plain steps behind the run's first step (below), read now, with the first tile's
+            // matrix work between the reads and their use: how many there are, and the band offset
+            // of the unit the first of them fetches (in steady state, which is checked there, step
+            // rel + 1 fetches unit rel + 1 + kStages - 1, whatever the first step had to fetch).
+            const int plain_word = at.units[min(rel + 1, n_units - 1)].flags;
+            const uint64_t off_first = static_cast<uint64_t>(at.bands[min(rel + C::kStages, n_units - 1) * NW + at.wave].off);
             float mx_lane = 0.0f;  // the lane's maximum over the score set that is consumed next
             float neg_m = 0.0f;    // minus the running maximum the exponentials of the next step refer to
             // Raise the running maximum (and rescale O^T and the row sum) if the tile about to be
@@ -769,8 +828,55 @@ paged_attn_pipe_kernel(const KArgs a) {
                 }
                 if (fetch) ++issued;
             };
+            // A plain step (mark_plain_steps()): the same work with the decisions taken out; `off` is
+            // the offset of this wave's band of the unit to fetch.
+            auto plain_step = [&](int r, bool cur_is_a, int64_t off) {
+                wait_async_loads<C::LOADS_PER_UNIT>();  // unit r + 1 has landed; unit r + 2 may be on its way
+                __builtin_amdgcn_s_barrier();
+                const int dst = uniform(static_cast<int>(at.stages_lds + (static_cast<unsigned>(issued) % C::kStages) * C::STAGE_BYTES +
+                                                         at.wave * (C::IPW * 1024)));
+                if (!compute_first || !busy) {
+                    pipe_issue_band(a.k_cache + off, a.v_cache + off, dst);
+                    if (busy) prepare();
+                }
+                if (busy) {
+                    const uint32_t v_cur = at.lds_address(tile_of(r) + C::MAT_BYTES) + at.v_lane;
+                    const uint32_t k_next = at.lds_address(tile_of(r + 1)) + at.k_lane;
+                    if (cur_is_a) {
+                        pipe_step_ab_x(k_next, v_cur, a.c, neg_m, at.l_run[0]);
+                        pipe_step_ab_y(a.c, neg_m, at.l_run[0], mx_lane);
+                    } else {
+                        pipe_step_ba_x(k_next, v_cur, a.c, neg_m, at.l_run[0]);
+                        pipe_step_ba_y(a.c, neg_m, at.l_run[0], mx_lane);
+                    }
+                    if (compute_first) {
+                        pipe_issue_band(a.k_cache + off, a.v_cache + off, dst);
+                        prepare();
+                    }
+                }
+                ++issued;
+            };
+            auto band_offset = [&](int unit) { return static_cast<uint64_t>(at.bands[unit * NW + at.wave].off); };
+            auto uniform_offset = [&](uint64_t off) {
+                return (static_cast<int64_t>(uniform(static_cast<int>(off >> 32))) << 32) | static_cast<uint32_t>(uniform(static_cast<int>(off)));
+            };
+            // From its second step on a run is in steady state, three units ahead (its first step fetches
+            // a unit or not, depending on how the run before it ended).  The plain steps that follow the
+            // first step are taken in pairs (score sets B then A), each reading the band offset of the
+            // step after it a step ahead; what is left of the run goes through the general step.
+            bool first_step = true;
             while (rel < run_end) {
                 step(rel++, true);
+                if (first_step && rel < run_end && issued == rel + C::kStages - 1) {
+                    uint64_t off = off_first;
+                    for (int pairs = (uniform(plain_word) >> kUnitPlainShift) >> 1; pairs > 0; --pairs) {
+                        const uint64_t off_next = band_offset(issued + 1);  // (in the table: the second step of the pair is plain)
+                        plain_step(rel++, false, uniform_offset(off));
+                        off = band_offset(min(issued + 1, n_units - 1));  // used if another pair follows
+                        plain_step(rel++, true, uniform_offset(off_next));
+                    }
+                }
+                first_step = false;
                 if (rel < run_end) step(rel++, false);
             }
             if (next_opens) wait_async_loads<0>();  // the next item's query rows (and the tiles requested before them)

@@ -16,6 +16,16 @@
 namespace dfx {
 
 DFX_D int uniform(int v) { return __builtin_amdgcn_readfirstlane(v); }
+// The thread's number in its workgroup, worked out where this is called (two instructions and a
+// scalar) instead of being kept from the kernel's entry on: under register pressure the kept one,
+// and every address derived from it ahead of a loop, is spilled to scratch, and a reload is a
+// trip to memory.  `wave_number`: the wave's number as a wave-uniform value.
+DFX_D int thread_number_here(int wave_number) {
+    int zero = 0;
+    asm volatile("" : "+v"(zero));  // (so that the count below is not computed early either)
+    const int lane = static_cast<int>(__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, static_cast<uint32_t>(zero))));
+    return wave_number * 64 + lane;
+}
 
 // Two e4m3 codes (bytes 0,1 or 2,3 of w) -> two bf16 packed in a dword, in one instruction
 // (v_cvt_scalef32_pk_bf16_fp8 with scale 1).  An e4m3 value has 3 mantissa bits, so the widening is

@@ -49,6 +49,7 @@ struct KArgs {
     int64_t v_fresh_delta;    // streaming paths: (token stride of v_new - token stride of k_new) in bytes
     const uint8_t* plan;      // launch plan built by the plan kernels, or null
     uint32_t plan_signature;  // of this launch's configuration: a plan made for another one is ignored
+    int32_t plan_capacity;    // unit descriptors the plan buffer has room for (fixes where its tables start)
     int64_t q_st, q_sh, kn_st, kn_sh, vn_st, vn_sh, o_st, o_sh;
     int64_t c_sp, c_st, c_sh;  // cache strides in elements: page, token, head
     // "distinct" cache layout (generic path only), strides in elements: K [page, head, d / 8, token, 8],

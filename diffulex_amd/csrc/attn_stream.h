@@ -64,9 +64,12 @@ struct WgWork {
     int64_t a0, a1, b0, b1;  // linear unit ranges [a0, a1) then [b0, b1), each inside one item under pairing
     int32_t partner;         // pairing: the workgroup holding the other piece of the shared item, or -1
     int32_t ubase;           // index of the workgroup's first unit descriptor
+    // of the workgroup's first unit (copied from its descriptor): what it takes to request the
+    // query rows of the first item before the descriptors have been read
+    int32_t q0, q_len, kvh, rt;
     int32_t pad[2];
 };
-static_assert(sizeof(WgWork) == 48, "three 16-byte words");
+static_assert(sizeof(WgWork) == 64, "four 16-byte words");
 
 struct PlanLayout {
     int64_t prefix_off, work_off, units_off, bands_off, bytes;
@@ -473,33 +476,55 @@ struct StreamAttn : TileMath<HD, NB, NW, HIDDEN> {
     WgSplit split;
     template <typename Body>
     DFX_D void for_each_chunk(Body&& body) {
+        for_each_chunk(body, [](const WgWork&) {});
+    }
+    // on_work(w): called as soon as a plan has told what the workgroup does (w: uniform values),
+    // before its descriptors are fetched, if it has anything to do.
+    template <typename Body, typename OnWork>
+    DFX_D void for_each_chunk(Body&& body, OnWork&& on_work) {
         const PlanHeader* hdr = reinterpret_cast<const PlanHeader*>(a.plan);
-        const bool planned = hdr != nullptr && uniform(static_cast<int>(hdr->magic)) == static_cast<int>(kPlanMagic) &&
-                             uniform(static_cast<int>(hdr->signature)) == static_cast<int>(a.plan_signature);
+        bool planned = false;
         WgWork w;
         w.a0 = w.a1 = w.b0 = w.b1 = 0;
         w.partner = -1;
         w.ubase = 0;
-        int64_t total;
-        int n_active;
+        int64_t total = 0;
+        int n_active = 0;
         const UnitDesc* g_units = nullptr;
         const BandDesc* g_bands = nullptr;
-        if (planned) {
-            per_head = uniform(hdr->per_head);
-            total = uniform(hdr->total_units);
-            n_active = uniform(hdr->n_active);
-            if (total == 0) return;
-            const PlanLayout lay = plan_layout(a.num_seqs, a.n_wg, uniform(hdr->capacity), NW);
-            const WgWork* gw = reinterpret_cast<const WgWork*>(a.plan + lay.work_off) + blockIdx.x;
-            w.a0 = gw->a0;
-            w.a1 = gw->a1;
-            w.b0 = gw->b0;
-            w.b1 = gw->b1;
-            w.partner = gw->partner;
-            w.ubase = gw->ubase;
-            g_units = reinterpret_cast<const UnitDesc*>(a.plan + lay.units_off);
-            g_bands = reinterpret_cast<const BandDesc*>(a.plan + lay.bands_off);
-        } else {
+        if (hdr != nullptr) {
+            // One trip to memory: the header and this workgroup's entry together (the host has told
+            // where the tables start; a header that says otherwise makes the plan unusable).
+            const PlanLayout lay = plan_layout(a.num_seqs, a.n_wg, a.plan_capacity, NW);
+            const u32x4* gh = reinterpret_cast<const u32x4*>(hdr);
+            const u32x4* gw = reinterpret_cast<const u32x4*>(reinterpret_cast<const WgWork*>(a.plan + lay.work_off) + blockIdx.x);
+            const u32x4 h0 = gh[0], h1 = gh[1];
+            const u32x4 g0 = gw[0], g1 = gw[1], g2 = gw[2], g3 = gw[3];
+            auto u = [](uint32_t v) { return uniform(static_cast<int>(v)); };
+            auto u64 = [&](uint32_t lo, uint32_t hi) { return (static_cast<int64_t>(u(hi)) << 32) | static_cast<uint32_t>(u(lo)); };
+            planned = u(h0[0]) == static_cast<int>(kPlanMagic) && u(h0[1]) == static_cast<int>(a.plan_signature) &&
+                      u(h1[2]) == a.plan_capacity;
+            if (planned) {
+                n_active = u(h0[2]);
+                per_head = u(h1[0]);
+                total = u(h1[1]);
+                if (total == 0) return;
+                w.a0 = u64(g0[0], g0[1]);
+                w.a1 = u64(g0[2], g0[3]);
+                w.b0 = u64(g1[0], g1[1]);
+                w.b1 = u64(g1[2], g1[3]);
+                w.partner = u(g2[0]);
+                w.ubase = u(g2[1]);
+                w.q0 = u(g2[2]);
+                w.q_len = u(g2[3]);
+                w.kvh = u(g3[0]);
+                w.rt = u(g3[1]);
+                g_units = reinterpret_cast<const UnitDesc*>(a.plan + lay.units_off);
+                g_bands = reinterpret_cast<const BandDesc*>(a.plan + lay.bands_off);
+                if (w.a1 + w.b1 > w.a0 + w.b0) on_work(w);
+            }
+        }
+        if (!planned) {
             const UnitSummary summary = build_unit_prefix<C::RT>(a, prefix, misc);
             per_head = summary.per_head;
             total = static_cast<int64_t>(per_head) * a.h_kv;
@@ -695,12 +720,25 @@ paged_attn_pipe_kernel(const KArgs a) {
     const bool busy = at.wave < a.busy_waves;  // waves whose 32 rows exist in no item of this launch only fetch
     constexpr int kHoleRows = C::ROWS_PER_WAVE;
     static_assert(kHoleRows == 8 || kHoleRows == 16, "mask blocks of attn_pipe_gen.h");
+    // With a plan the query rows of the workgroup's first item are requested as soon as its entry of
+    // the plan has been read, together with the descriptors, instead of a trip to memory later.
+    bool requested_early = false;
+    auto on_work = [&](const WgWork& w) {
+        UnitDesc d;
+        d.q0 = w.q0;
+        d.q_len = w.q_len;
+        d.kvh = w.kvh;
+        d.rt = w.rt;
+        at.request_queries(d);
+        requested_early = true;
+    };
     at.for_each_chunk([&](int n_units) {
         const WgSplit& split = at.split;
         // An item that opens with this chunk: its query rows first.  Requested behind the ring fill,
         // the wait for them would also wait for every tile of the fill.
         const bool opens = (uniform(at.units[0].flags) & kUnitFirst) != 0;
-        if (opens) at.request_queries(at.units[0]);
+        if (opens && !requested_early) at.request_queries(at.units[0]);
+        requested_early = false;
         // While the query rows are on their way: the marks of the plain steps.  They are first read
         // behind the barrier of the first run's first step; they only add bits to the flags that
         // nobody looks at before.  (Not behind the ring fill: a spilled register reloaded here would
@@ -883,7 +921,7 @@ paged_attn_pipe_kernel(const KArgs a) {
             at.finish_run(rel - 1, split);
             if (next_opens) at.adopt_item(at.units[run_end]);
         }
-    });
+    }, on_work);
 }
 
 }  // namespace dfx

@@ -271,6 +271,13 @@ uint32_t plan_signature(const dfx_attn_params* p, const Plan& plan) {
 
 int plan_waves(const Plan& plan) { return (plan.compact || (plan.fp8 && plan.hd == 64)) ? 4 : 4 * plan.nb; }
 
+// Unit descriptors a plan buffer of `bytes` has room for behind its fixed part.
+int64_t plan_capacity(int64_t bytes, const PlanLayout& fixed, int waves) {
+    const int64_t per_unit = static_cast<int64_t>(sizeof(UnitDesc)) + waves * static_cast<int64_t>(sizeof(BandDesc));
+    const int64_t n = (bytes - fixed.bytes) / per_unit;
+    return n > 0x7fffffff ? 0x7fffffff : n;
+}
+
 // Checks and launch; `workspace` replaces p->workspace.  plan_out != nullptr: instead of the
 // attention launch, build its plan into plan_out (plan_bytes of room).
 int run_paged_attn(const dfx_attn_params* p, void* workspace, int64_t workspace_bytes, dfx_stream_t stream,
@@ -289,11 +296,9 @@ int run_paged_attn(const dfx_attn_params* p, void* workspace, int64_t workspace_
         if (!plan.stream) return DFX_ERR_UNSUPPORTED;
         if ((reinterpret_cast<uintptr_t>(plan_out) & 255u) != 0) return DFX_ERR_INVALID_ARG;
         const PlanLayout fixed = plan_layout(p->num_seqs, plan.n_wg, 0, plan_waves(plan));
-        const int64_t per_unit = static_cast<int64_t>(sizeof(UnitDesc)) + plan_waves(plan) * static_cast<int64_t>(sizeof(BandDesc));
         if (plan_bytes < fixed.bytes) return DFX_ERR_WORKSPACE;
         pa.buf = static_cast<uint8_t*>(plan_out);
-        pa.capacity = (plan_bytes - fixed.bytes) / per_unit;
-        if (pa.capacity > 0x7fffffff) pa.capacity = 0x7fffffff;
+        pa.capacity = plan_capacity(plan_bytes, fixed, plan_waves(plan));
         pa.n_wg = plan.n_wg;
         pa.waves = plan_waves(plan);
         pa.signature = plan_signature(p, plan);
@@ -354,11 +359,15 @@ int run_paged_attn(const dfx_attn_params* p, void* workspace, int64_t workspace_
     ka.n_new = p->num_new_tokens > 0 ? p->num_new_tokens : INT64_MAX;
     ka.v_fresh_delta = (p->vn_stride_token - p->kn_stride_token) * 2;
     ka.plan = nullptr;
+    ka.plan_capacity = 0;
     ka.plan_signature = plan_signature(p, plan);
     if (plan_out == nullptr && plan.stream && p->plan != nullptr) {
         const PlanLayout fixed = plan_layout(p->num_seqs, plan.n_wg, 0, plan_waves(plan));
         if (p->plan_bytes < fixed.bytes || (reinterpret_cast<uintptr_t>(p->plan) & 255u) != 0) return DFX_ERR_INVALID_ARG;
         ka.plan = static_cast<const uint8_t*>(p->plan);
+        // where the plan's tables start follows from the buffer's size: the same size as when it was built, or the
+        // kernel finds another capacity in the header and plans for itself
+        ka.plan_capacity = static_cast<int32_t>(plan_capacity(p->plan_bytes, fixed, plan_waves(plan)));
     }
 
     hipStream_t st = static_cast<hipStream_t>(stream);

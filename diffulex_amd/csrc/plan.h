@@ -6,7 +6,8 @@
 //   PlanHeader                                  64 bytes
 //   int32 prefix[num_seqs + 1]                  exclusive prefix of the sequences' units (per KV head)
 //   WgWork work[n_wg]                           what every workgroup does (partition.h: linear ranges
-//                                               of the unit space, or the pairing partition)
+//                                               of the unit space, or the pairing partition), and the
+//                                               item of its first unit
 //   UnitDesc units[capacity]                    one per unit, in each workgroup's processing order
 //   BandDesc bands[capacity * NW]               one per unit and wave
 // Two kernels fill it: paged_attn_plan_kernel (one workgroup: prefix, partition) and
@@ -187,6 +188,7 @@ __global__ void __launch_bounds__(512) paged_attn_plan_kernel(const KArgs a, con
             w.a0 = w.a1 = w.b0 = w.b1 = 0;
             w.partner = -1;
             w.ubase = 0;
+            w.q0 = w.q_len = w.kvh = w.rt = 0;  // (the fill kernel enters them)
             w.pad[0] = w.pad[1] = 0;
             if (k >= m) {
                 work[k] = w;
@@ -226,6 +228,7 @@ __global__ void __launch_bounds__(512) paged_attn_plan_kernel(const KArgs a, con
             w.a0 = w.a1 = w.b0 = w.b1 = 0;
             w.partner = -1;
             w.ubase = 0;
+            w.q0 = w.q_len = w.kvh = w.rt = 0;  // (the fill kernel enters them)
             w.pad[0] = w.pad[1] = 0;
             if (k < n_active && total > 0) {
                 w.a0 = split.first(k);
@@ -268,6 +271,7 @@ __global__ void __launch_bounds__(64 * NW) paged_attn_plan_fill_kernel(const KAr
     __syncthreads();
     int64_t done = w.ubase;
     at.rel_base = w.a0;
+    bool first_chunk = true;
     for (int seg = 0; seg < 2; ++seg) {
         at.begin = seg == 0 ? w.a0 : w.b0;
         at.end = seg == 0 ? w.a1 : w.b1;
@@ -275,6 +279,16 @@ __global__ void __launch_bounds__(64 * NW) paged_attn_plan_fill_kernel(const KAr
             const int n = static_cast<int>(min(static_cast<int64_t>(C::kPlanUnits), at.end - chunk));
             at.plan_units(chunk, n, seg == 0 ? w.partner : -1, seg);
             __syncthreads();
+            if (first_chunk && threadIdx.x == 0) {
+                // the first unit's item, for the attention kernel to request its query rows early
+                WgWork* mine = reinterpret_cast<WgWork*>(pa.buf + lay.work_off) + blockIdx.x;
+                const UnitDesc d = at.units[0];
+                mine->q0 = d.q0;
+                mine->q_len = d.q_len;
+                mine->kvh = d.kvh;
+                mine->rt = d.rt;
+            }
+            first_chunk = false;
             // descriptors are multiples of 16 bytes: copy as such
             const u32x4* su = reinterpret_cast<const u32x4*>(at.units);
             u32x4* du = reinterpret_cast<u32x4*>(g_units + done);

@@ -819,7 +819,7 @@ def _read_plan(plan, num_seqs, n_wg):
     raw = plan.cpu().numpy()
     hdr = raw[:64].view(np.int32)
     work_off = (64 + (num_seqs + 1) * 4 + 63) // 64 * 64
-    work = raw[work_off:work_off + n_wg * 48].reshape(n_wg, 48)
+    work = raw[work_off:work_off + n_wg * 64].reshape(n_wg, 64)   # WgWork: 64-byte records
     ranges = work[:, :32].copy().view(np.int64).reshape(n_wg, 4)
     partner = work[:, 32:36].copy().view(np.int32).reshape(n_wg)
     return dict(magic=int(hdr[0]) & 0xffffffff, n_active=int(hdr[2]), mode=int(hdr[3]), per_head=int(hdr[4]),

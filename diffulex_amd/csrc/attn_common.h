@@ -610,11 +610,13 @@ DFX_D bool finish_cut_item(AttnState<HD, NB, NW, HIDDEN>& at, int rt, int64_t it
 // round-robin to the threads of the whole grid; every workgroup calls this once.  The slots
 // written are outside every attended context (caller's contract), so nothing in this launch
 // reads them.
-template <int HD, bool FP8>
+// kBatch: chunks a thread has in flight (all loads of a batch are issued before its stores).  A kernel
+// that leaves the compiler few registers takes 1: four chunks' addresses and data do not fit there,
+// and data spilled to scratch makes two more trips to memory.
+template <int HD, bool FP8, int kBatch = 4>
 DFX_D void store_fresh_rows(const KArgs& a) {
     if (a.store_slots == nullptr) return;
     constexpr int kChunksPerHead = HD / 8;
-    constexpr int kBatch = 4;  // chunks a thread has in flight: all loads of a batch are issued before its stores
     const int chunks_per_token = a.h_kv * kChunksPerHead;
     // (never beyond the rows k_new / v_new and the slot mapping have, whatever the offsets say)
     const int64_t n_rows = min(static_cast<int64_t>(a.cu_new[a.num_seqs]), a.n_new);

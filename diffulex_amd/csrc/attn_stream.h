@@ -716,7 +716,7 @@ paged_attn_pipe_kernel(const KArgs a) {
         }
         pipe_set_load_offsets(o[0], o[1]);
     }
-    store_fresh_rows<HD, false>(a);
+    store_fresh_rows<HD, false, 1>(a);
     const bool busy = at.wave < a.busy_waves;  // waves whose 32 rows exist in no item of this launch only fetch
     constexpr int kHoleRows = C::ROWS_PER_WAVE;
     static_assert(kHoleRows == 8 || kHoleRows == 16, "mask blocks of attn_pipe_gen.h");

@@ -185,7 +185,9 @@ struct StreamAttn : TileMath<HD, NB, NW, HIDDEN> {
     // other piece of a cut item).
     DFX_D void plan_units(int64_t first, int count, int partner = -1, int seg = 0) const {
         (void)seg;
-        for (int idx = tid; idx < count * NW; idx += C::THREADS) {
+        // (the thread's number worked out here: what depends on it is then not computed ahead of the
+        // caller's chunk loop and, where registers are few, kept in scratch meanwhile)
+        for (int idx = thread_number_here(wave_s); idx < count * NW; idx += C::THREADS) {
             const int64_t pos = first + idx / NW;
             const int w = idx % NW;
             const int slot_in_ring = idx / NW;

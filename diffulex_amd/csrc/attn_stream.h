@@ -51,7 +51,7 @@ struct PlanHeader {
     uint32_t magic;      // kPlanMagic once both kernels have run; 0: unusable
     uint32_t signature;  // of the launch configuration the plan was made for
     int32_t n_active;    // workgroups that take part
-    int32_t mode;        // 0: equal linear ranges, 1: pairing partition
+    int32_t mode;        // 0: equal linear ranges, 1: pairing partition, 2: linear ranges cut at the plan's bounds table
     int32_t per_head;    // units per KV head
     int32_t total_units;
     int32_t capacity;    // unit descriptors the buffer has room for
@@ -72,12 +72,13 @@ struct WgWork {
 static_assert(sizeof(WgWork) == 64, "four 16-byte words");
 
 struct PlanLayout {
-    int64_t prefix_off, work_off, units_off, bands_off, bytes;
+    int64_t prefix_off, bounds_off, work_off, units_off, bands_off, bytes;
 };
 DFX_HD PlanLayout plan_layout(int num_seqs, int n_wg, int64_t capacity, int waves) {
     PlanLayout l;
     l.prefix_off = sizeof(PlanHeader);
-    l.work_off = (l.prefix_off + (static_cast<int64_t>(num_seqs) + 1) * 4 + 63) / 64 * 64;
+    l.bounds_off = (l.prefix_off + (static_cast<int64_t>(num_seqs) + 1) * 4 + 63) / 64 * 64;
+    l.work_off = (l.bounds_off + (static_cast<int64_t>(n_wg) + 1) * 4 + 63) / 64 * 64;
     l.units_off = (l.work_off + static_cast<int64_t>(n_wg) * sizeof(WgWork) + 63) / 64 * 64;
     l.bands_off = l.units_off + capacity * static_cast<int64_t>(sizeof(UnitDesc));
     l.bytes = l.bands_off + capacity * waves * static_cast<int64_t>(sizeof(BandDesc));
@@ -491,7 +492,7 @@ struct StreamAttn : TileMath<HD, NB, NW, HIDDEN> {
         w.partner = -1;
         w.ubase = 0;
         int64_t total = 0;
-        int n_active = 0;
+        int n_active = 0, plan_mode = 0;
         const UnitDesc* g_units = nullptr;
         const BandDesc* g_bands = nullptr;
         if (hdr != nullptr) {
@@ -508,6 +509,7 @@ struct StreamAttn : TileMath<HD, NB, NW, HIDDEN> {
                       u(h1[2]) == a.plan_capacity;
             if (planned) {
                 n_active = u(h0[2]);
+                plan_mode = u(h0[3]);
                 per_head = u(h1[0]);
                 total = u(h1[1]);
                 if (total == 0) return;
@@ -536,6 +538,14 @@ struct StreamAttn : TileMath<HD, NB, NW, HIDDEN> {
                                                          summary.max_tiles, a.n_wg);
         }
         split = make_wg_split(total, n_active);
+        if (planned && plan_mode == 2) {
+            // the plan has placed the cut points itself: its table, for the owners of a cut item's pieces,
+            // into the space the unit prefix takes when the kernel plans (visible behind the barriers
+            // of the first chunk; first read when a run ends)
+            const int32_t* g_bounds = reinterpret_cast<const int32_t*>(a.plan + plan_layout(a.num_seqs, a.n_wg, a.plan_capacity, NW).bounds_off);
+            for (int i = thread_number_here(wave_s); i <= n_active; i += C::THREADS) prefix[i] = g_bounds[i];
+            split.bounds = prefix;
+        }
         if (!planned && static_cast<int>(blockIdx.x) < n_active) {
             w.a0 = split.first(blockIdx.x);
             w.a1 = split.first(blockIdx.x + 1);

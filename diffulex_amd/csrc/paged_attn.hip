@@ -303,6 +303,7 @@ int run_paged_attn(const dfx_attn_params* p, void* workspace, int64_t workspace_
         pa.waves = plan_waves(plan);
         pa.signature = plan_signature(p, plan);
         pa.allow_pairing = (p->flags & DFX_ATTN_PAIRING) ? 1 : 0;
+        pa.equal_ranges = (p->flags & DFX_ATTN_EQUAL_RANGES) ? 1 : 0;
     }
 
     KArgs ka;

@@ -129,11 +129,16 @@ DFX_HD int wg_of_unit(int64_t u, int64_t total, int n_wg) {
 
 // The same cut points without a 64-bit division at every use: with total = q * n_wg + r,
 // floor(w * total / n_wg) = w * q + floor(w * r / n_wg), and w * r fits 32 bits (n_wg < 65536).
+// `bounds`, if not null: the cut points come from a table instead (bounds[w] = first unit of workgroup
+// w, bounds[n_wg] = total; strictly increasing), as a launch plan may place them (plan.h); q and r
+// still describe the total.
 struct WgSplit {
     int64_t q;
     uint32_t r;
     int n_wg;
+    const int32_t* bounds;
     DFX_HD int64_t first(int w) const {
+        if (bounds != nullptr) return bounds[w];
         return static_cast<int64_t>(w) * q + (static_cast<uint32_t>(w) * r) / static_cast<uint32_t>(n_wg);
     }
 };
@@ -143,6 +148,7 @@ DFX_HD WgSplit make_wg_split(int64_t total, int n_wg) {
     sp.q = total / n_wg;
     sp.r = static_cast<uint32_t>(total - sp.q * n_wg);
     sp.n_wg = n_wg;
+    sp.bounds = nullptr;
     return sp;
 }
 

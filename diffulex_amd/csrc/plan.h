@@ -5,6 +5,7 @@
 // Layout of the plan buffer:
 //   PlanHeader                                  64 bytes
 //   int32 prefix[num_seqs + 1]                  exclusive prefix of the sequences' units (per KV head)
+//   int32 bounds[n_wg + 1]                      mode 2: first unit of every workgroup's range
 //   WgWork work[n_wg]                           what every workgroup does (partition.h: linear ranges
 //                                               of the unit space, or the pairing partition), and the
 //                                               item of its first unit
@@ -27,7 +28,18 @@ struct PlanArgs {
     int waves;          // waves per attention workgroup
     uint32_t signature;
     int allow_pairing;
+    int equal_ranges;   // cut the unit space into equal ranges, as the attention kernels do without a plan
 };
+
+// Where the plan cuts the linear unit space (mode 2): ranges of equal COST, a unit costing 2 and
+// every sequence whose units begin in the range kPlanSeqCost more (a workgroup opens and closes an
+// item there: query rows, first scores alone, rows written -- time it cannot spend on tiles; equal
+// ranges of units leave the workgroups with many short items behind), and a cut point within
+// kPlanSnap units of such a beginning moved onto it (a piece of one or two tiles costs two
+// workgroups a partial result through memory for less work than that takes).
+constexpr int kPlanSeqCost = 3;
+constexpr int kPlanSnap = 2;
+constexpr int kPlanMinUnitsPerWg = 8;  // below this the ranges stay equal
 
 // Linear position of item y (0 <= y < items of the sequence) inside the sequence's units, and its tiles.
 DFX_HD void item_of_sequence(const SeqShape& sh, int rt, int& offset, int& tiles) {
@@ -123,6 +135,7 @@ __global__ void __launch_bounds__(512) paged_attn_plan_kernel(const KArgs a, con
     // ---- pairing partition, if it applies --------------------------------------------------------
     const int m = n_active;
     bool pairing = pa.allow_pairing && total > 0 && n_items <= m && m <= kMaxPairItems && total >= m;
+    bool placed = false;  // cut points placed by cost (mode 2)
     int critical = 0;
     if (pairing) {  // (uniform: every thread takes the same branch)
         int n_sort = 1;
@@ -223,6 +236,61 @@ __global__ void __launch_bounds__(512) paged_attn_plan_kernel(const KArgs a, con
         }
     } else {
         const WgSplit split = make_wg_split(total > 0 ? total : 1, n_active > 0 ? n_active : 1);
+        int32_t* g_bounds = reinterpret_cast<int32_t*>(pa.buf + lay.bounds_off);
+        int* bounds = reinterpret_cast<int*>(keys);  // [n_wg + 1] (the pairing partition's arrays are free here)
+        static_assert(kMaxPairItems + kMaxPairItems >= 1025, "room for the cut points of up to 1024 workgroups");
+        placed = !pa.equal_ranges && n_active > 1 && n_active <= 1024 && total >= static_cast<int64_t>(kPlanMinUnitsPerWg) * n_active &&
+                 total < (1ll << 30);
+        if (placed) {  // (uniform)
+            // the sequence of a KV head whose units contain unit rem of that head
+            auto seq_of = [&](int rem) {
+                int lo = 0, hi = a.num_seqs;
+                while (lo < hi) {
+                    const int mid = (lo + hi) >> 1;
+                    if (prefix[mid + 1] <= rem) lo = mid + 1;
+                    else hi = mid;
+                }
+                return lo;
+            };
+            auto cost_before = [&](int64_t x) {  // cost of units [0, x)
+                if (x >= total) return 2 * total + static_cast<int64_t>(kPlanSeqCost) * a.h_kv * a.num_seqs;
+                const int kvh = static_cast<int>(x / per_head);
+                const int rem = static_cast<int>(x - static_cast<int64_t>(kvh) * per_head);
+                return 2 * x + static_cast<int64_t>(kPlanSeqCost) * (static_cast<int64_t>(kvh) * a.num_seqs + seq_of(rem));
+            };
+            const int64_t cost_total = cost_before(total);
+            for (int k = tid; k <= n_active; k += blockDim.x) {
+                int64_t x = k == 0 ? 0 : total;
+                if (k > 0 && k < n_active) {
+                    const int64_t target = cost_total * k / n_active;
+                    int64_t lo = 0, hi = total;  // the first x with cost_before(x) >= target
+                    while (lo < hi) {
+                        const int64_t mid = (lo + hi) >> 1;
+                        if (cost_before(mid) < target) lo = mid + 1;
+                        else hi = mid;
+                    }
+                    x = lo;
+                    const int kvh = static_cast<int>(x / per_head);
+                    const int rem = static_cast<int>(x - static_cast<int64_t>(kvh) * per_head);
+                    const int sq = seq_of(rem);
+                    const int64_t below = static_cast<int64_t>(kvh) * per_head + prefix[sq];
+                    const int64_t above = static_cast<int64_t>(kvh) * per_head + prefix[sq + 1];
+                    if (x - below <= kPlanSnap && below > 0) x = below;
+                    else if (above - x <= kPlanSnap && above < total) x = above;
+                }
+                bounds[k] = static_cast<int>(x);
+            }
+            __syncthreads();
+            // every workgroup that takes part must own a unit (a cut item's pieces are counted by
+            // their owners' numbers): if not, equal ranges
+            int bad = 0;
+            for (int k = tid; k < n_active; k += blockDim.x) bad |= bounds[k] >= bounds[k + 1];
+            if (tid == 0) misc[32] = 0;
+            __syncthreads();
+            if (bad) misc[32] = 1;
+            __syncthreads();
+            placed = misc[32] == 0;
+        }
         for (int k = tid; k < pa.n_wg; k += blockDim.x) {
             WgWork w;
             w.a0 = w.a1 = w.b0 = w.b1 = 0;
@@ -231,19 +299,21 @@ __global__ void __launch_bounds__(512) paged_attn_plan_kernel(const KArgs a, con
             w.q0 = w.q_len = w.kvh = w.rt = 0;  // (the fill kernel enters them)
             w.pad[0] = w.pad[1] = 0;
             if (k < n_active && total > 0) {
-                w.a0 = split.first(k);
-                w.a1 = split.first(k + 1);
+                w.a0 = placed ? bounds[k] : split.first(k);
+                w.a1 = placed ? bounds[k + 1] : split.first(k + 1);
                 w.ubase = static_cast<int32_t>(w.a0);
             }
             work[k] = w;
         }
+        if (placed)
+            for (int k = tid; k <= n_active; k += blockDim.x) g_bounds[k] = bounds[k];
     }
     if (tid == 0) {
         PlanHeader h;
         h.magic = total <= pa.capacity ? kPlanMagic : 0u;  // too small a buffer: the kernels plan for themselves
         h.signature = pa.signature;
         h.n_active = n_active;
-        h.mode = pairing ? 1 : 0;
+        h.mode = pairing ? 1 : (placed ? 2 : 0);
         h.per_head = per_head;
         h.total_units = static_cast<int32_t>(total);
         h.capacity = static_cast<int32_t>(pa.capacity);

@@ -50,6 +50,8 @@ typedef enum dfx_index_type { DFX_INDEX_I32 = 0, DFX_INDEX_I64 = 1 } dfx_index_t
 #define DFX_ATTN_GENERIC_PATH 1 /* use the generic tile path even where the streaming path applies */
 #define DFX_ATTN_NO_PIPELINE 2  /* streaming path: the plain tile loop instead of the software-pipelined one */
 #define DFX_ATTN_PAIRING 4      /* dfx_paged_attn_plan: the pairing partition where it applies (see there) */
+#define DFX_ATTN_EQUAL_RANGES 8 /* dfx_paged_attn_plan: equal ranges of the unit space, as a launch without a plan cuts
+                                   them (the plan's own cut points are placed by cost; see there) */
 
 /* ABI version of the loaded library (== DFX_ABI_VERSION it was built with). */
 int dfx_abi_version(void);
@@ -236,7 +238,11 @@ int dfx_paged_attn(const dfx_attn_params* params, dfx_stream_t stream);
  * shapes, max_workgroups, flags and the strides of the caches and of k_new -- not on the base
  * pointers of q, k_new, v_new, out and the caches, nor on scale: the per-layer views of one cache
  * allocation share a plan.  It is built on `stream` with no host synchronisation (safe to record
- * into a graph).  DFX_ATTN_PAIRING in flags asks for the pairing partition where there are at most
+ * into a graph).  With at least 8 units per workgroup the plan places the cut points between the
+ * workgroups' ranges of the unit space by cost rather than by unit count (a range that begins many
+ * sequences gets fewer tiles) and onto a sequence's first unit where one is within two units;
+ * DFX_ATTN_EQUAL_RANGES in flags keeps the equal ranges a launch without a plan uses (the results of
+ * the two differ in the last bits: other pieces are merged).  DFX_ATTN_PAIRING in flags asks for the pairing partition where there are at most
  * as many (sequence, KV head, row tile) items as workgroups: every item gets a home workgroup and
  * only the excess of long items moves, which needs a third of the partial results that equal ranges
  * of the unit space need, at about the same speed.

@@ -140,7 +140,8 @@ def test_fp8_edge_cases(dev, case, mask, flags):
         got = _run(g, max_wg, flags=flags)
         assert max_abs_err(got, want) <= ATOL_FP8
     if flags == 0:
-        assert torch.equal(_run(g, 0, plan_cache={}), _run(g, 0))   # a planned launch gives the same bits
+        # a planned launch with the same cut points gives the same bits
+        assert torch.equal(_run(g, 0, plan_cache={}, flags=_lib.DFX_ATTN_EQUAL_RANGES), _run(g, 0))
 
 
 def test_fresh_k_and_v_with_different_strides(dev):
@@ -183,7 +184,7 @@ def test_fresh_v_sliced_out_of_the_projection(dev, name, over, flags):
     wl.v_new = v_view
     for max_wg in (0, 5):
         ref = _run(wl, max_wg, flags=flags) if max_wg == 0 else None
-        got = _run(wl, max_wg, flags=flags, plan_cache={})
+        got = _run(wl, max_wg, flags=flags | _lib.DFX_ATTN_EQUAL_RANGES, plan_cache={})   # (the cut points of a launch without a plan)
         if ref is not None:
             assert torch.equal(ref, want) and torch.equal(got, want)
         else:
@@ -818,26 +819,62 @@ def _read_plan(plan, num_seqs, n_wg):
     """Header and per-workgroup work of a plan buffer (layout: csrc/plan.h)."""
     raw = plan.cpu().numpy()
     hdr = raw[:64].view(np.int32)
-    work_off = (64 + (num_seqs + 1) * 4 + 63) // 64 * 64
+    bounds_off = (64 + (num_seqs + 1) * 4 + 63) // 64 * 64
+    work_off = (bounds_off + (n_wg + 1) * 4 + 63) // 64 * 64
     work = raw[work_off:work_off + n_wg * 64].reshape(n_wg, 64)   # WgWork: 64-byte records
     ranges = work[:, :32].copy().view(np.int64).reshape(n_wg, 4)
     partner = work[:, 32:36].copy().view(np.int32).reshape(n_wg)
+    bounds = raw[bounds_off:bounds_off + (n_wg + 1) * 4].copy().view(np.int32)
     return dict(magic=int(hdr[0]) & 0xffffffff, n_active=int(hdr[2]), mode=int(hdr[3]), per_head=int(hdr[4]),
-                total=int(hdr[5]), critical=int(hdr[7])), ranges, partner
+                total=int(hdr[5]), critical=int(hdr[7]), bounds=bounds), ranges, partner
 
 
 @pytest.mark.parametrize("name,over", PLAN_CASES)
 @pytest.mark.parametrize("max_wg", [0, 7])
 def test_planned_launch_with_equal_ranges_gives_the_same_bits(dev, name, over, max_wg):
-    """By default the plan describes the partition the kernels work out for themselves: reading it
-    must not change a bit."""
+    """With equal ranges the plan describes the partition the kernels work out for themselves:
+    reading it must not change a bit."""
     wl = make_workload(name, device=dev, **over)
     want = _run(wl, max_wg)
     cache = {}
     for _ in range(2):   # the second call reuses the plan
-        got = _run(wl, max_wg, plan_cache=cache)
+        got = _run(wl, max_wg, plan_cache=cache, flags=_lib.DFX_ATTN_EQUAL_RANGES)
         assert torch.equal(got, want)
     assert len(cache) == 1 and next(iter(cache.values())) is not None
+
+
+@pytest.mark.parametrize("name,over", PLAN_CASES + [("c3", dict(num_seqs=40, ctx=(64, 1500))),
+                                                    ("c3", dict(num_seqs=24, ctx=[70] * 12 + [2900] * 12))])
+@pytest.mark.parametrize("max_wg", [0, 7, 40])
+def test_planned_launch_with_cut_points_placed_by_cost(dev, name, over, max_wg):
+    """The default plan: ranges of equal cost, cut points moved onto a sequence's first unit where one is
+    near.  Other pieces are merged than without a plan, so the rows differ in the last bits only;
+    every launch with the plan gives the same bits; the ranges tile the unit space."""
+    wl = make_workload(name, device=dev, **over)
+    cache = {}
+    got = _run(wl, max_wg, plan_cache=cache)
+    tol = ATOL_FP8 if wl.kv_fp8 else ATOL_BF16
+    if wl.num_seqs <= 16:
+        assert max_abs_err(got, oracle_fp32(wl)) <= tol
+    assert max_abs_err(got, _run(wl, max_wg)) <= 1e-2
+    assert torch.equal(_run(wl, max_wg, plan_cache=cache), got)
+    plan = next(iter(cache.values()))
+    cus = torch.cuda.get_device_properties(dev).multi_processor_count
+    ok = False
+    for n_wg in ([max_wg, 2 * max_wg] if max_wg else [cus, 2 * cus]):   # (two workgroups per compute unit for the small shapes)
+        hdr, ranges, _ = _read_plan(plan, wl.num_seqs, n_wg)
+        assert hdr["magic"] == 0x44465850 and hdr["mode"] in (0, 2)
+        spans = [(int(r[0]), int(r[1])) for r in ranges[:hdr["n_active"]]]
+        if not (spans and spans[0][0] == 0 and spans[-1][1] == hdr["total"]):
+            continue
+        ok = True
+        assert all(x[1] == y[0] for x, y in zip(spans, spans[1:])), (hdr, spans)
+        if hdr["mode"] == 2:
+            assert all(b > a for a, b in spans), (hdr, spans)
+            assert [a for a, _ in spans] + [hdr["total"]] == hdr["bounds"][:hdr["n_active"] + 1].tolist()
+            assert hdr["total"] >= 8 * hdr["n_active"]
+        break
+    assert ok
 
 
 @pytest.mark.parametrize("name,over", PLAN_CASES)

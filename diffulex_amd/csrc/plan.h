@@ -33,12 +33,19 @@ struct PlanArgs {
 
 // Where the plan cuts the linear unit space (mode 2): ranges of equal COST, a unit costing 2 and
 // every sequence whose units begin in the range kPlanSeqCost more (a workgroup opens and closes an
-// item there: query rows, first scores alone, rows written -- time it cannot spend on tiles; equal
-// ranges of units leave the workgroups with many short items behind), and a cut point within
-// kPlanSnap units of such a beginning moved onto it (a piece of one or two tiles costs two
-// workgroups a partial result through memory for less work than that takes).
-constexpr int kPlanSeqCost = 3;
-constexpr int kPlanSnap = 2;
+// item there: query rows, first scores alone, rows written or a partial result through memory --
+// time it cannot spend on tiles; equal ranges of units leave the workgroups with several short
+// items behind), and a cut point within kPlanSnap units of such a beginning moved onto it (a piece
+// of a few tiles costs two workgroups a partial result through memory for less work than that
+// takes).  Both values are measured, not derived (MI355X, 64 sequences x 4 KV heads of 8-32 tiles
+// on 256 workgroups: 0 / 0: 67.6 µs, 3 / 2: 65.9, 6 / 3: 65.2, 8 / 4: 65.2-65.8, 8 / 6: 69.7, 8 / 0:
+// 73.5).  Only where a workgroup's range holds at most two items on average: with more, shorter
+// items every cut point is near a beginning, the ranges become whole numbers of items, and that
+// costs more than the cuts (800 items of 6 tiles: 77 µs against 70 with equal ranges; 400 items of
+// 12 tiles: 58 against 63).
+constexpr int kPlanSeqCost = 8;
+constexpr int kPlanSnap = 4;
+constexpr int kPlanMaxItemsPerWg = 2;
 constexpr int kPlanMinUnitsPerWg = 8;  // below this the ranges stay equal
 
 // Linear position of item y (0 <= y < items of the sequence) inside the sequence's units, and its tiles.
@@ -240,43 +247,36 @@ __global__ void __launch_bounds__(512) paged_attn_plan_kernel(const KArgs a, con
         int* bounds = reinterpret_cast<int*>(keys);  // [n_wg + 1] (the pairing partition's arrays are free here)
         static_assert(kMaxPairItems + kMaxPairItems >= 1025, "room for the cut points of up to 1024 workgroups");
         placed = !pa.equal_ranges && n_active > 1 && n_active <= 1024 && total >= static_cast<int64_t>(kPlanMinUnitsPerWg) * n_active &&
-                 total < (1ll << 30);
+                 n_items <= static_cast<int64_t>(kPlanMaxItemsPerWg) * n_active && total < (1ll << 30);
         if (placed) {  // (uniform)
-            // the sequence of a KV head whose units contain unit rem of that head
-            auto seq_of = [&](int rem) {
-                int lo = 0, hi = a.num_seqs;
-                while (lo < hi) {
-                    const int mid = (lo + hi) >> 1;
-                    if (prefix[mid + 1] <= rem) lo = mid + 1;
-                    else hi = mid;
-                }
-                return lo;
+            // Cost of the units before unit x: 2 x + kPlanSeqCost * (sequences that begin at or before x).
+            // Sequence j of the launch (KV head major) begins at unit start(j); the cost there:
+            const int n_seq_heads = a.h_kv * a.num_seqs;
+            auto start = [&](int j) {  // j == n_seq_heads: total
+                const int kvh = j / a.num_seqs;
+                return static_cast<int64_t>(kvh) * per_head + prefix[j - kvh * a.num_seqs];
             };
-            auto cost_before = [&](int64_t x) {  // cost of units [0, x)
-                if (x >= total) return 2 * total + static_cast<int64_t>(kPlanSeqCost) * a.h_kv * a.num_seqs;
-                const int kvh = static_cast<int>(x / per_head);
-                const int rem = static_cast<int>(x - static_cast<int64_t>(kvh) * per_head);
-                return 2 * x + static_cast<int64_t>(kPlanSeqCost) * (static_cast<int64_t>(kvh) * a.num_seqs + seq_of(rem));
-            };
-            const int64_t cost_total = cost_before(total);
+            auto cost_at = [&](int j) { return 2 * start(j) + static_cast<int64_t>(kPlanSeqCost) * j; };
+            const int64_t cost_total = cost_at(n_seq_heads);
             for (int k = tid; k <= n_active; k += blockDim.x) {
                 int64_t x = k == 0 ? 0 : total;
                 if (k > 0 && k < n_active) {
                     const int64_t target = cost_total * k / n_active;
-                    int64_t lo = 0, hi = total;  // the first x with cost_before(x) >= target
+                    int lo = 0, hi = n_seq_heads;  // the first sequence whose beginning costs at least the target
                     while (lo < hi) {
-                        const int64_t mid = (lo + hi) >> 1;
-                        if (cost_before(mid) < target) lo = mid + 1;
+                        const int mid = (lo + hi) >> 1;
+                        if (cost_at(mid) < target) lo = mid + 1;
                         else hi = mid;
                     }
-                    x = lo;
-                    const int kvh = static_cast<int>(x / per_head);
-                    const int rem = static_cast<int>(x - static_cast<int64_t>(kvh) * per_head);
-                    const int sq = seq_of(rem);
-                    const int64_t below = static_cast<int64_t>(kvh) * per_head + prefix[sq];
-                    const int64_t above = static_cast<int64_t>(kvh) * per_head + prefix[sq + 1];
-                    if (x - below <= kPlanSnap && below > 0) x = below;
-                    else if (above - x <= kPlanSnap && above < total) x = above;
+                    x = 0;
+                    if (lo > 0) {
+                        // inside the sequence before it the cost grows by 2 per unit: the first unit that reaches the target
+                        const int64_t below = start(lo - 1), above = start(lo);
+                        x = (target - static_cast<int64_t>(kPlanSeqCost) * (lo - 1) + 1) >> 1;
+                        x = x > above ? above : x;
+                        if (x - below <= kPlanSnap && below > 0) x = below;
+                        else if (above - x <= kPlanSnap && above < total) x = above;
+                    }
                 }
                 bounds[k] = static_cast<int>(x);
             }

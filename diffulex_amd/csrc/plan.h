@@ -78,6 +78,86 @@ DFX_D void bitonic_sort_desc(uint32_t* keys, int n) {
         }
 }
 
+// The cut points of one KV head by a sweep over its sequences (mode 2 as well; where it applies it
+// replaces the placement above).  Per workgroup, measured at the headline shape (timers in the
+// attention kernel, least squares over both partitions): 12.3 µs + 1.35 µs per unit + 4.1 µs per whole
+// item + 6.8 µs if its range begins inside an item + 8.5 µs if it ends inside one -- a cut costs
+// two workgroups as much as eleven tiles.  In half units: a unit 2, a whole item kSweepWhole, a range
+// that begins inside an item kSweepBegins, one that ends inside an item kSweepEnds.  With a capacity
+// per workgroup the sweep gives every workgroup in turn what fits: the rest of the item the one
+// before it cut, whole items while they fit, and a piece of the next item if a piece of at least
+// kSweepMinPiece units fits and leaves at least as much (5: shorter pieces measured worse, as in the
+// placement above; the other constants within a third of these measure the same, halved they lose
+// 3-20 %).  It succeeds if the last workgroup's share fits as well.  `out` (n_w + 1 cut points, in
+// units of the head), if not null, receives them.
+constexpr int kSweepWhole = 6, kSweepBegins = 10, kSweepEnds = 13, kSweepMinPiece = 5;
+DFX_D bool sweep_head(const int* __restrict__ prefix, int num_seqs, int n_w, int cap2, int* __restrict__ out, int out_stride) {
+    // (one lane, one dependent LDS read per item or workgroup: the item under the cursor is kept in
+    // registers -- lo, hi its first unit and the one behind its last -- and the one behind it is read ahead)
+    const int per_head = prefix[num_seqs];
+    int pos = 0, i = 0;
+    int lo = 0, hi = prefix[1], next = num_seqs > 1 ? prefix[2] : per_head;
+    auto advance = [&] {
+        ++i;
+        lo = hi;
+        hi = next;
+        next = i + 2 <= num_seqs ? prefix[i + 2] : per_head;
+    };
+    for (int w = 0; w + 1 < n_w; ++w) {
+        int used2 = 0;
+        while (i < num_seqs && hi <= pos) advance();  // (sequences without units, and items taken to their end)
+        if (pos < per_head) {
+            bool full = false;
+            if (lo < pos) {  // the rest of the item the workgroup before has cut
+                used2 = kSweepBegins;
+                const int rest = hi - pos;
+                if (used2 + 2 * rest > cap2) {  // cut once more
+                    int take = (cap2 - used2 - kSweepEnds) / 2;
+                    take = take < 1 ? 1 : (take > rest ? rest : take);
+                    pos += take;
+                    full = true;
+                } else {
+                    used2 += 2 * rest;
+                    pos = hi;
+                    advance();
+                }
+            }
+            if (!full) {
+                while (i < num_seqs) {
+                    const int len = hi - lo;
+                    if (len != 0) {
+                        if (used2 + 2 * len + kSweepWhole > cap2) break;
+                        used2 += 2 * len + kSweepWhole;
+                        pos = hi;
+                    }
+                    advance();
+                }
+                if (i < num_seqs) {
+                    const int len = hi - lo;
+                    const int room = (cap2 - used2 - kSweepEnds) / 2;
+                    if (room >= kSweepMinPiece) {
+                        if (len - room >= kSweepMinPiece) pos += room;
+                        else if (len - kSweepMinPiece >= kSweepMinPiece) pos += len - kSweepMinPiece;
+                    }
+                }
+            }
+        }
+        if (out != nullptr) out[w * out_stride] = pos;   // cut point w + 1
+    }
+    // the last workgroup takes what is left
+    int used2 = 0;
+    while (i < num_seqs && hi <= pos) advance();
+    if (pos < per_head) {
+        if (lo < pos) used2 = kSweepBegins - kSweepWhole;  // (the loop below counts the cut item as a whole one)
+        used2 += 2 * (per_head - pos);
+        while (i < num_seqs) {
+            used2 += hi > lo ? kSweepWhole : 0;
+            advance();
+        }
+    }
+    return used2 <= cap2;
+}
+
 // Phase one, one workgroup of 512 threads: the unit prefix, the partition and every workgroup's work.
 template <int RT>
 __global__ void __launch_bounds__(512) paged_attn_plan_kernel(const KArgs a, const PlanArgs pa) {
@@ -248,7 +328,55 @@ __global__ void __launch_bounds__(512) paged_attn_plan_kernel(const KArgs a, con
         static_assert(kMaxPairItems + kMaxPairItems >= 1025, "room for the cut points of up to 1024 workgroups");
         placed = !pa.equal_ranges && n_active > 1 && n_active <= 1024 && total >= static_cast<int64_t>(kPlanMinUnitsPerWg) * n_active &&
                  n_items <= static_cast<int64_t>(kPlanMaxItemsPerWg) * n_active && total < (1ll << 30);
-        if (placed) {  // (uniform)
+        // the sweep, where the workgroups divide evenly among the KV heads (whose sequences are the same):
+        // 64 capacities, from the mean load (no cuts) upwards in steps of 1 %, one per lane; the smallest
+        // that succeeds is swept once more for its cut points, which every KV head then uses
+        bool swept = false;
+        const int n_w = a.h_kv > 0 ? n_active / a.h_kv : 0;
+        if (placed && n_w >= 2 && n_w * a.h_kv == n_active && n_w <= 1023) {  // (uniform)
+            int nonempty = 0;
+            for (int sq = tid; sq < a.num_seqs; sq += blockDim.x) nonempty += prefix[sq + 1] > prefix[sq];
+#pragma unroll
+            for (int d = 32; d >= 1; d >>= 1) nonempty += __shfl_xor(nonempty, d);
+            if ((tid & 63) == 0) misc[40 + (tid >> 6)] = nonempty;
+            __syncthreads();
+            nonempty = 0;
+            for (int w = 0; w < static_cast<int>(blockDim.x >> 6); ++w) nonempty += misc[40 + w];
+            const int base2 = (2 * per_head + kSweepWhole * nonempty + n_w - 1) / n_w;
+            // every lane keeps the n_w - 1 inner cut points of its capacity (lane-minor, so that the lanes'
+            // stores do not collide) as long as 64 x (n_w - 1) numbers fit; otherwise the best capacity is swept again
+            const bool keep = 64 * (n_w - 1) <= kMaxSeqs + 1;
+            // (8 capacities per wave: lanes of one wave that walk at different speeds wait for each other)
+            if (tid < 64) misc[tid] = 0;
+            __syncthreads();
+            {
+                const int cand = (tid >> 6) * 8 + (tid & 63);
+                if ((tid & 63) < 8 && cand < 64) {
+                    const bool ok = sweep_head(prefix, a.num_seqs, n_w, base2 + base2 * cand / 100, keep ? iprefix + cand : nullptr, 64);
+                    misc[cand] = ok ? 1 : 0;
+                }
+            }
+            __syncthreads();
+            if (tid < 64) {
+                const uint64_t votes = __ballot(misc[tid] != 0);
+                const int best = votes != 0 ? __builtin_ctzll(votes) : 64;
+                if (tid == 0) {
+                    ubase[0] = best;
+                    if (best < 64 && !keep) sweep_head(prefix, a.num_seqs, n_w, base2 + base2 * best / 100, iprefix, 1);
+                }
+            }
+            __syncthreads();
+            swept = ubase[0] < 64;
+            if (swept) {
+                const int best = ubase[0];
+                for (int k = tid; k <= n_active; k += blockDim.x) {
+                    const int kvh = k / n_w, w = k - kvh * n_w;  // (k == n_active: the end of the last head)
+                    bounds[k] = kvh * per_head + (w == 0 ? 0 : iprefix[keep ? (w - 1) * 64 + best : w - 1]);
+                }
+            }
+            __syncthreads();
+        }
+        if (placed && !swept) {  // (uniform)
             // Cost of the units before unit x: 2 x + kPlanSeqCost * (sequences that begin at or before x).
             // Sequence j of the launch (KV head major) begins at unit start(j); the cost there:
             const int n_seq_heads = a.h_kv * a.num_seqs;
@@ -281,10 +409,13 @@ __global__ void __launch_bounds__(512) paged_attn_plan_kernel(const KArgs a, con
                 bounds[k] = static_cast<int>(x);
             }
             __syncthreads();
-            // every workgroup that takes part must own a unit (a cut item's pieces are counted by
-            // their owners' numbers): if not, equal ranges
+        }
+        if (placed) {
+            // every workgroup that takes part must own a unit (a cut item's pieces are counted by their
+            // owners' numbers), except that the sweep may leave workgroups without any where a sequence
+            // begins (no item reaches across such a point): if not, equal ranges
             int bad = 0;
-            for (int k = tid; k < n_active; k += blockDim.x) bad |= bounds[k] >= bounds[k + 1];
+            for (int k = tid; k < n_active; k += blockDim.x) bad |= swept ? bounds[k] > bounds[k + 1] : bounds[k] >= bounds[k + 1];
             if (tid == 0) misc[32] = 0;
             __syncthreads();
             if (bad) misc[32] = 1;

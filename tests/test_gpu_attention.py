@@ -870,7 +870,7 @@ def test_planned_launch_with_cut_points_placed_by_cost(dev, name, over, max_wg):
         ok = True
         assert all(x[1] == y[0] for x, y in zip(spans, spans[1:])), (hdr, spans)
         if hdr["mode"] == 2:
-            assert all(b > a for a, b in spans), (hdr, spans)
+            assert all(b >= a for a, b in spans), (hdr, spans)   # (the sweep may leave a workgroup without units)
             assert [a for a, _ in spans] + [hdr["total"]] == hdr["bounds"][:hdr["n_active"] + 1].tolist()
             assert hdr["total"] >= 8 * hdr["n_active"]
         break

@@ -238,9 +238,11 @@ int dfx_paged_attn(const dfx_attn_params* params, dfx_stream_t stream);
  * shapes, max_workgroups, flags and the strides of the caches and of k_new -- not on the base
  * pointers of q, k_new, v_new, out and the caches, nor on scale: the per-layer views of one cache
  * allocation share a plan.  It is built on `stream` with no host synchronisation (safe to record
- * into a graph).  With at least 8 units per workgroup the plan places the cut points between the
- * workgroups' ranges of the unit space by cost rather than by unit count (a range that begins many
- * sequences gets fewer tiles) and onto a sequence's first unit where one is within two units;
+ * into a graph).  With at least 8 units and at most two items per workgroup the plan places the cut
+ * points between the workgroups' ranges of the unit space by cost rather than by unit count (whole
+ * sequences where they fit, no pieces of a few tiles: a sweep with the smallest capacity per
+ * workgroup that works, which makes the plan kernel take about 50 us -- a plan is worth building
+ * for several launches, not for one);
  * DFX_ATTN_EQUAL_RANGES in flags keeps the equal ranges a launch without a plan uses (the results of
  * the two differ in the last bits: other pieces are merged).  DFX_ATTN_PAIRING in flags asks for the pairing partition where there are at most
  * as many (sequence, KV head, row tile) items as workgroups: every item gets a home workgroup and

@@ -92,68 +92,57 @@ DFX_D void bitonic_sort_desc(uint32_t* keys, int n) {
 // units of the head), if not null, receives them.
 constexpr int kSweepWhole = 6, kSweepBegins = 10, kSweepEnds = 13, kSweepMinPiece = 5;
 DFX_D bool sweep_head(const int* __restrict__ prefix, int num_seqs, int n_w, int cap2, int* __restrict__ out, int out_stride) {
-    // (one lane, one dependent LDS read per item or workgroup: the item under the cursor is kept in
-    // registers -- lo, hi its first unit and the one behind its last -- and the one behind it is read ahead)
+    // One lane walks; 64 lanes walk for 64 capacities, so the walk is one flat loop whose every turn
+    // either finishes the item under the cursor or closes a workgroup's range, written with selects
+    // rather than nested branches (lanes that disagree on a branch run both sides one after the
+    // other).  The item under the cursor is kept in registers (lo, hi: its first unit and the one
+    // behind its last) and the beginning of the one after next is read a turn ahead.
     const int per_head = prefix[num_seqs];
-    int pos = 0, i = 0;
+    int pos = 0, i = 0, w = 0;
     int lo = 0, hi = prefix[1], next = num_seqs > 1 ? prefix[2] : per_head;
+    int budget = cap2;
+    bool fresh = true;  // the workgroup has taken nothing yet
     auto advance = [&] {
         ++i;
         lo = hi;
         hi = next;
         next = i + 2 <= num_seqs ? prefix[i + 2] : per_head;
     };
-    for (int w = 0; w + 1 < n_w; ++w) {
-        int used2 = 0;
-        while (i < num_seqs && hi <= pos) advance();  // (sequences without units, and items taken to their end)
-        if (pos < per_head) {
-            bool full = false;
-            if (lo < pos) {  // the rest of the item the workgroup before has cut
-                used2 = kSweepBegins;
-                const int rest = hi - pos;
-                if (used2 + 2 * rest > cap2) {  // cut once more
-                    int take = (cap2 - used2 - kSweepEnds) / 2;
-                    take = take < 1 ? 1 : (take > rest ? rest : take);
-                    pos += take;
-                    full = true;
-                } else {
-                    used2 += 2 * rest;
-                    pos = hi;
-                    advance();
-                }
-            }
-            if (!full) {
-                while (i < num_seqs) {
-                    const int len = hi - lo;
-                    if (len != 0) {
-                        if (used2 + 2 * len + kSweepWhole > cap2) break;
-                        used2 += 2 * len + kSweepWhole;
-                        pos = hi;
-                    }
-                    advance();
-                }
-                if (i < num_seqs) {
-                    const int len = hi - lo;
-                    const int room = (cap2 - used2 - kSweepEnds) / 2;
-                    if (room >= kSweepMinPiece) {
-                        if (len - room >= kSweepMinPiece) pos += room;
-                        else if (len - kSweepMinPiece >= kSweepMinPiece) pos += len - kSweepMinPiece;
-                    }
-                }
-            }
+    while (w + 1 < n_w && i < num_seqs) {
+        const int rest = hi - pos;          // units of the item from the cursor on (0: a sequence without units)
+        const bool mid = lo < pos;          // the workgroup before has cut this item
+        budget -= (fresh && mid) ? kSweepBegins : 0;
+        const int need = rest > 0 ? 2 * rest + (mid ? 0 : kSweepWhole) : 0;
+        if (need <= budget) {               // the rest of the item fits
+            budget -= need;
+            pos = hi;
+            fresh = fresh && rest <= 0;
+            advance();
+            continue;
         }
-        if (out != nullptr) out[w * out_stride] = pos;   // cut point w + 1
+        // it does not: a piece of it, if a piece of at least kSweepMinPiece units fits and leaves as much
+        // (an item that was cut already is cut again wherever the capacity ends), and the range is closed
+        const int room = (budget - kSweepEnds) / 2;
+        const int again = room < 1 ? 1 : (room > rest ? rest : room);
+        const int first = room < kSweepMinPiece ? 0
+                          : (rest - room >= kSweepMinPiece ? room : (rest - kSweepMinPiece >= kSweepMinPiece ? rest - kSweepMinPiece : 0));
+        pos += (fresh && mid) ? again : first;
+        if (out != nullptr) out[w * out_stride] = pos;  // cut point w + 1
+        ++w;
+        budget = cap2;
+        fresh = true;
     }
+    if (out != nullptr)
+        for (; w + 1 < n_w; ++w) out[w * out_stride] = pos;  // (workgroups without units: every sequence is taken)
     // the last workgroup takes what is left
     int used2 = 0;
-    while (i < num_seqs && hi <= pos) advance();
-    if (pos < per_head) {
-        if (lo < pos) used2 = kSweepBegins - kSweepWhole;  // (the loop below counts the cut item as a whole one)
-        used2 += 2 * (per_head - pos);
-        while (i < num_seqs) {
-            used2 += hi > lo ? kSweepWhole : 0;
-            advance();
+    while (i < num_seqs) {
+        const int rest = hi - pos;
+        if (rest > 0) {
+            used2 += 2 * rest + (lo < pos ? kSweepBegins : kSweepWhole);
+            pos = hi;
         }
+        advance();
     }
     return used2 <= cap2;
 }

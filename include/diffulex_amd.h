@@ -241,7 +241,7 @@ int dfx_paged_attn(const dfx_attn_params* params, dfx_stream_t stream);
  * into a graph).  With at least 8 units and at most two items per workgroup the plan places the cut
  * points between the workgroups' ranges of the unit space by cost rather than by unit count (whole
  * sequences where they fit, no pieces of a few tiles: a sweep with the smallest capacity per
- * workgroup that works, which makes the plan kernel take about 50 us -- a plan is worth building
+ * workgroup that works, which makes the plan kernel take about 30 us -- a plan is worth building
  * for several launches, not for one);
  * DFX_ATTN_EQUAL_RANGES in flags keeps the equal ranges a launch without a plan uses (the results of
  * the two differ in the last bits: other pieces are merged).  DFX_ATTN_PAIRING in flags asks for the pairing partition where there are at most

@@ -78,75 +78,6 @@ DFX_D void bitonic_sort_desc(uint32_t* keys, int n) {
         }
 }
 
-// The cut points of one KV head by a sweep over its sequences (mode 2 as well; where it applies it
-// replaces the placement above).  Per workgroup, measured at the headline shape (timers in the
-// attention kernel, least squares over both partitions): 12.3 µs + 1.35 µs per unit + 4.1 µs per whole
-// item + 6.8 µs if its range begins inside an item + 8.5 µs if it ends inside one -- a cut costs
-// two workgroups as much as eleven tiles.  In half units: a unit 2, a whole item kSweepWhole, a range
-// that begins inside an item kSweepBegins, one that ends inside an item kSweepEnds.  With a capacity
-// per workgroup the sweep gives every workgroup in turn what fits: the rest of the item the one
-// before it cut, whole items while they fit, and a piece of the next item if a piece of at least
-// kSweepMinPiece units fits and leaves at least as much (5: shorter pieces measured worse, as in the
-// placement above; the other constants within a third of these measure the same, halved they lose
-// 3-20 %).  It succeeds if the last workgroup's share fits as well.  `out` (n_w + 1 cut points, in
-// units of the head), if not null, receives them.
-constexpr int kSweepWhole = 6, kSweepBegins = 10, kSweepEnds = 13, kSweepMinPiece = 5;
-DFX_D bool sweep_head(const int* __restrict__ prefix, int num_seqs, int n_w, int cap2, int* __restrict__ out, int out_stride) {
-    // One lane walks; 64 lanes walk for 64 capacities, so the walk is one flat loop whose every turn
-    // either finishes the item under the cursor or closes a workgroup's range, written with selects
-    // rather than nested branches (lanes that disagree on a branch run both sides one after the
-    // other).  The item under the cursor is kept in registers (lo, hi: its first unit and the one
-    // behind its last) and the beginning of the one after next is read a turn ahead.
-    const int per_head = prefix[num_seqs];
-    int pos = 0, i = 0, w = 0;
-    int lo = 0, hi = prefix[1], next = num_seqs > 1 ? prefix[2] : per_head;
-    int budget = cap2;
-    bool fresh = true;  // the workgroup has taken nothing yet
-    auto advance = [&] {
-        ++i;
-        lo = hi;
-        hi = next;
-        next = i + 2 <= num_seqs ? prefix[i + 2] : per_head;
-    };
-    while (w + 1 < n_w && i < num_seqs) {
-        const int rest = hi - pos;          // units of the item from the cursor on (0: a sequence without units)
-        const bool mid = lo < pos;          // the workgroup before has cut this item
-        budget -= (fresh && mid) ? kSweepBegins : 0;
-        const int need = rest > 0 ? 2 * rest + (mid ? 0 : kSweepWhole) : 0;
-        if (need <= budget) {               // the rest of the item fits
-            budget -= need;
-            pos = hi;
-            fresh = fresh && rest <= 0;
-            advance();
-            continue;
-        }
-        // it does not: a piece of it, if a piece of at least kSweepMinPiece units fits and leaves as much
-        // (an item that was cut already is cut again wherever the capacity ends), and the range is closed
-        const int room = (budget - kSweepEnds) / 2;
-        const int again = room < 1 ? 1 : (room > rest ? rest : room);
-        const int first = room < kSweepMinPiece ? 0
-                          : (rest - room >= kSweepMinPiece ? room : (rest - kSweepMinPiece >= kSweepMinPiece ? rest - kSweepMinPiece : 0));
-        pos += (fresh && mid) ? again : first;
-        if (out != nullptr) out[w * out_stride] = pos;  // cut point w + 1
-        ++w;
-        budget = cap2;
-        fresh = true;
-    }
-    if (out != nullptr)
-        for (; w + 1 < n_w; ++w) out[w * out_stride] = pos;  // (workgroups without units: every sequence is taken)
-    // the last workgroup takes what is left
-    int used2 = 0;
-    while (i < num_seqs) {
-        const int rest = hi - pos;
-        if (rest > 0) {
-            used2 += 2 * rest + (lo < pos ? kSweepBegins : kSweepWhole);
-            pos = hi;
-        }
-        advance();
-    }
-    return used2 <= cap2;
-}
-
 // Phase one, one workgroup of 512 threads: the unit prefix, the partition and every workgroup's work.
 template <int RT>
 __global__ void __launch_bounds__(512) paged_attn_plan_kernel(const KArgs a, const PlanArgs pa) {

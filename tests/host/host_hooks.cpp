@@ -134,4 +134,23 @@ int hook_combine_slots(const int* ctx, const int* q_len, const int* new_len, int
     }
     return n;
 }
+
+// The capacity sweep of a launch plan over one KV head (partition.h): n_w + 1 cut points into out
+// (out[0] = 0, out[n_w] = the head's units); returns whether the last workgroup's share fits.
+int hook_sweep_head(const int* prefix, int num_seqs, int n_w, int cap2, int* out) {
+    using namespace dfx;
+    out[0] = 0;
+    const bool ok = sweep_head(prefix, num_seqs, n_w, cap2, out + 1, 1);
+    out[n_w] = prefix[num_seqs];
+    return ok ? 1 : 0;
+}
+
+// owners_of_units with a table of cut points (a plan's bounds): the first and last workgroup whose
+// range meets units [first_unit, last_unit], walking from `me`.
+void hook_owners_with_bounds(const int* bounds, int n_wg, int me, long long first_unit, long long last_unit, int* wa, int* wb) {
+    using namespace dfx;
+    WgSplit sp = make_wg_split(bounds[n_wg], n_wg);
+    sp.bounds = bounds;
+    owners_of_units(sp, me, first_unit, last_unit, *wa, *wb);
+}
 }

@@ -33,4 +33,8 @@ def load():
     lib.hook_enumerate_units.argtypes = [i32, i32, i32, i32, i32, i32, i32, vp, i32]
     lib.hook_combine_slots.restype = i32
     lib.hook_combine_slots.argtypes = [vp, vp, vp, i32, i32, i32, i32, i32, i32, i32, i32, vp, i32]
+    lib.hook_sweep_head.restype = i32
+    lib.hook_sweep_head.argtypes = [vp, i32, i32, i32, vp]
+    lib.hook_owners_with_bounds.restype = None
+    lib.hook_owners_with_bounds.argtypes = [vp, i32, i32, i64, i64, vp, vp]
     return lib

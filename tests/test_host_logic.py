@@ -377,3 +377,93 @@ def test_pairwise_merge_protocol_model(p):
         assert len(written) == 1, "the rows are written exactly once"
         assert written[0] == frozenset(range(p)), "every piece reaches the root"
         assert all(v == 0 for v in counters.values()), "every counter is left at zero"
+
+
+# ---- the launch plan's capacity sweep (partition.h: sweep_head) and owners looked up in a table of cut points ----
+SWEEP_WHOLE, SWEEP_BEGINS, SWEEP_ENDS, SWEEP_MIN_PIECE = 6, 10, 13, 5
+
+
+def _sweep(lib, lengths, n_w, cap2):
+    prefix = np.concatenate([[0], np.cumsum(lengths)]).astype(np.int32)
+    out = np.full(n_w + 1, -1, dtype=np.int32)
+    ok = lib.hook_sweep_head(prefix.ctypes.data, len(lengths), n_w, int(cap2), out.ctypes.data)
+    return prefix, out, bool(ok)
+
+
+def _range_cost(prefix, a, e):
+    """Cost of range [a, e) in half units, by the rule the sweep states."""
+    if e <= a:
+        return 0
+    cost = 2 * (e - a)
+    for i in range(len(prefix) - 1):
+        lo, hi = int(prefix[i]), int(prefix[i + 1])
+        if hi <= lo or hi <= a or lo >= e:
+            continue
+        if lo < a:
+            cost += SWEEP_BEGINS
+        elif hi > e:
+            cost += SWEEP_ENDS
+        else:
+            cost += SWEEP_WHOLE
+    return cost
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_plan_sweep_tiles_the_head_and_keeps_its_promises(seed):
+    lib = hosthooks.load()
+    rng = np.random.default_rng(seed)
+    n_seq = int(rng.integers(1, 90))
+    lengths = rng.integers(0 if seed % 3 == 0 else 1, int(rng.integers(4, 60)), size=n_seq)
+    if lengths.sum() == 0:
+        lengths[0] = 7
+    n_w = int(rng.integers(2, 80))
+    base2 = (2 * int(lengths.sum()) + SWEEP_WHOLE * int((lengths > 0).sum()) + n_w - 1) // n_w
+    feasible_before = False
+    starts = set(np.concatenate([[0], np.cumsum(lengths)]).tolist())
+    for t in range(0, 64, 3):
+        cap2 = base2 + base2 * t // 100
+        prefix, b, ok = _sweep(lib, lengths, n_w, cap2)
+        per_head = int(prefix[-1])
+        assert b[0] == 0 and b[-1] == per_head and np.all(np.diff(b) >= 0), (b, cap2)
+        assert not (feasible_before and not ok), "a larger capacity cannot fail where a smaller one worked"
+        feasible_before = feasible_before or ok
+        for w in range(n_w):
+            a, e = int(b[w]), int(b[w + 1])
+            if e == a:
+                assert a in starts or a == per_head, "a workgroup without units only where a sequence begins"
+                continue
+            if ok or w + 1 < n_w:
+                # (an item cut for the second time takes at least one unit whatever the capacity)
+                assert _range_cost(prefix, a, e) <= cap2 + SWEEP_BEGINS + SWEEP_ENDS + 2, (w, a, e, cap2)
+        # a first cut of an item leaves at least SWEEP_MIN_PIECE units on either side
+        for w in range(1, n_w):
+            x = int(b[w])
+            if x in starts or x == int(b[w - 1]):
+                continue
+            i = int(np.searchsorted(prefix, x, side="right") - 1)
+            lo, hi = int(prefix[i]), int(prefix[i + 1])
+            if int(b[w - 1]) <= lo:       # the range that ends here began at or before the item: its first cut
+                assert x - lo >= SWEEP_MIN_PIECE and hi - x >= SWEEP_MIN_PIECE, (w, x, lo, hi)
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_owners_of_a_cut_item_from_a_table_of_cut_points(seed):
+    """The attention kernels find the workgroups that hold pieces of a cut item by walking the plan's
+    table of cut points; workgroups without units (the sweep leaves them where a sequence begins)
+    must never be counted among them."""
+    lib = hosthooks.load()
+    rng = np.random.default_rng(100 + seed)
+    lengths = rng.integers(1, 40, size=int(rng.integers(3, 50)))
+    n_w = int(rng.integers(3, 60))
+    base2 = (2 * int(lengths.sum()) + SWEEP_WHOLE * len(lengths) + n_w - 1) // n_w
+    prefix, b, ok = _sweep(lib, lengths, n_w, base2 + base2 * int(rng.integers(20, 80)) // 100)
+    bounds = b.astype(np.int32)
+    for i in range(len(lengths)):
+        first, last = int(prefix[i]), int(prefix[i + 1]) - 1
+        owners = [w for w in range(n_w) if bounds[w] < bounds[w + 1] and bounds[w] <= last and bounds[w + 1] > first]
+        assert owners == list(range(owners[0], owners[-1] + 1)), "pieces of an item are held by consecutive workgroups"
+        for me in owners:
+            wa, wb = C.c_int(-1), C.c_int(-1)
+            lib.hook_owners_with_bounds(bounds.ctypes.data, n_w, me, first, last, C.byref(wa), C.byref(wb))
+            assert (wa.value, wb.value) == (owners[0], owners[-1]), (i, me, owners)
+

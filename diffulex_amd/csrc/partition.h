@@ -163,16 +163,17 @@ DFX_HD void owners_of_units(const WgSplit& sp, int me, int64_t first_unit, int64
 
 // The cut points of one KV head by a sweep over its sequences (plan.h: mode 2 of a launch plan).
 // Per workgroup, measured at the headline shape (timers in the attention kernel, least squares over
-// equal ranges and ranges placed by cost): 12.3 µs + 1.35 µs per unit + 4.1 µs per whole
-// item + 6.8 µs if its range begins inside an item + 8.5 µs if it ends inside one -- a cut costs
-// two workgroups as much as eleven tiles.  In half units: a unit 2, a whole item kSweepWhole, a range
+// the workgroups of a launch): 12.8 µs + 1.31 µs per unit + 5.0 µs per whole item + 6.7 µs if its
+// range begins inside an item + 10.0 µs if it ends inside one (rms error 1.0 µs) -- a cut costs
+// two workgroups as much as thirteen tiles.  In half units: a unit 2, a whole item kSweepWhole, a range
 // that begins inside an item kSweepBegins, one that ends inside an item kSweepEnds.  With a capacity
 // per workgroup the sweep gives every workgroup in turn what fits: the rest of the item the one
 // before it cut, whole items while they fit, and a piece of the next item if a piece of at least
-// kSweepMinPiece units fits and leaves at least as much (5: shorter pieces measured worse; the other constants within a third of these measure the same, halved they lose
-// 3-20 %).  It succeeds if the last workgroup's share fits as well.  `out` (n_w + 1 cut points, in
-// units of the head), if not null, receives them.
-constexpr int kSweepWhole = 6, kSweepBegins = 10, kSweepEnds = 13, kSweepMinPiece = 5;
+// kSweepMinPiece units fits and leaves at least as much (5: shorter pieces measured worse; the
+// other constants within a third of these measure the same to 1 %, halved they lose 3-20 %).  It
+// succeeds if the last workgroup's share fits as well.  `out`, if not null, receives the n_w - 1
+// inner cut points (in units of the head), out_stride numbers apart.
+constexpr int kSweepWhole = 8, kSweepBegins = 10, kSweepEnds = 15, kSweepMinPiece = 5;
 DFX_HD bool sweep_head(const int* __restrict__ prefix, int num_seqs, int n_w, int cap2, int* __restrict__ out, int out_stride) {
     // One lane walks; 64 lanes walk for 64 capacities, so the walk is one flat loop whose every turn
     // either finishes the item under the cursor or closes a workgroup's range, written with selects

@@ -380,7 +380,7 @@ def test_pairwise_merge_protocol_model(p):
 
 
 # ---- the launch plan's capacity sweep (partition.h: sweep_head) and owners looked up in a table of cut points ----
-SWEEP_WHOLE, SWEEP_BEGINS, SWEEP_ENDS, SWEEP_MIN_PIECE = 6, 10, 13, 5
+SWEEP_WHOLE, SWEEP_BEGINS, SWEEP_ENDS, SWEEP_MIN_PIECE = 8, 10, 15, 5
 
 
 def _sweep(lib, lengths, n_w, cap2):

@@ -253,7 +253,7 @@ __global__ void __launch_bounds__(512) paged_attn_plan_kernel(const KArgs a, con
         // that succeeds is swept once more for its cut points, which every KV head then uses
         bool swept = false;
         const int n_w = a.h_kv > 0 ? n_active / a.h_kv : 0;
-        if (placed && n_w >= 2 && n_w * a.h_kv == n_active && n_w <= 1023) {  // (uniform)
+        if (placed && blockDim.x == 512 && n_w >= 2 && n_w * a.h_kv == n_active && n_w <= 1023) {  // (uniform)
             int nonempty = 0;
             for (int sq = tid; sq < a.num_seqs; sq += blockDim.x) nonempty += prefix[sq + 1] > prefix[sq];
 #pragma unroll
@@ -266,19 +266,19 @@ __global__ void __launch_bounds__(512) paged_attn_plan_kernel(const KArgs a, con
             // every lane keeps the n_w - 1 inner cut points of its capacity (lane-minor, so that the lanes'
             // stores do not collide) as long as 64 x (n_w - 1) numbers fit; otherwise the best capacity is swept again
             const bool keep = 64 * (n_w - 1) <= kMaxSeqs + 1;
-            // (8 capacities per wave: lanes of one wave that walk at different speeds wait for each other)
-            if (tid < 64) misc[tid] = 0;
-            __syncthreads();
+            // (8 capacities per wave: lanes of one wave that walk at different speeds wait for each other;
+            // the kernel runs with 8 waves, and every one of the 64 flags is written)
+            int* fits = ubase + 64;  // [64]
             {
                 const int cand = (tid >> 6) * 8 + (tid & 63);
                 if ((tid & 63) < 8 && cand < 64) {
                     const bool ok = sweep_head(prefix, a.num_seqs, n_w, base2 + base2 * cand / 100, keep ? iprefix + cand : nullptr, 64);
-                    misc[cand] = ok ? 1 : 0;
+                    fits[cand] = ok ? 1 : 0;
                 }
             }
             __syncthreads();
             if (tid < 64) {
-                const uint64_t votes = __ballot(misc[tid] != 0);
+                const uint64_t votes = __ballot(fits[tid] != 0);
                 const int best = votes != 0 ? __builtin_ctzll(votes) : 64;
                 if (tid == 0) {
                     ubase[0] = best;

@@ -139,6 +139,13 @@ DFX_D void async_load16(const void* base, uint32_t voff, uint32_t lds_wave_base)
                  : "memory", "m0");
 }
 
+// The float at p (wave-uniform, not written during the launch), read into a scalar register.
+DFX_D float scalar_load(const float* p) {
+    float x;
+    asm volatile("s_load_dword %0, %1, 0x0\n\ts_waitcnt lgkmcnt(0)" : "=s"(x) : "s"(p) : "memory");
+    return x;
+}
+
 template <int N>
 DFX_D void wait_async_loads() {
     asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
@@ -351,6 +358,57 @@ struct StreamAttn : TileMath<HD, NB, NW, HIDDEN> {
         }
     }
 
+    // FP8, pipelined kernel.  Its step works on the K tile of one unit and the V tile of the unit
+    // before, so the widened K tiles and the widened V tiles are kept apart, two of each, and a
+    // unit's two halves are widened a step apart (K first).  Fresh rows are copied as they are: the
+    // kernel folds the scales that tell them from cached rows into its softmax constants.
+    DFX_D uint8_t* wide_k(int rel) const { return lds + C::WIDE_OFF + (rel & 1) * L::MAT_BYTES; }
+    DFX_D uint8_t* wide_v(int rel) const { return lds + C::WIDE_OFF + 2 * L::MAT_BYTES + (rel & 1) * L::MAT_BYTES; }
+    // CTX_ONLY: the caller knows the band to be one of cached rows.
+    template <bool IS_V, bool CTX_ONLY = false>
+    DFX_D void widen_matrix(int rel) const {
+        int tag = 1;
+        if constexpr (!CTX_ONLY) tag = uniform(bands[rel * NW + wave_s].is_ctx);
+        uint8_t* dst = IS_V ? wide_v(rel) : wide_k(rel);
+        // (the lane's number worked out here: see thread_number_here())
+        const int ln = thread_number_here(0);
+        const int cc = ln % C::CPR;
+        if (CTX_ONLY || tag > 0) {
+            const uint8_t* raw = lds + C::STAGES_OFF + (static_cast<unsigned>(rel) % C::kStages) * C::STAGE_BYTES +
+                                 (IS_V ? C::MAT_BYTES : 0) + wave_s * (C::IPW * 1024) + ln * 16;
+#pragma unroll
+            for (int j = 0; j < C::IPW; ++j) {
+                const int row = wave_s * C::ROWS_PER_WAVE + j * C::RPI + ln / C::CPR;
+                const u32x4 codes = *reinterpret_cast<const u32x4*>(raw + j * 1024);
+                u32x4 lo, hi;
+                widen16(codes, lo, hi);
+                *reinterpret_cast<u32x4*>(dst + L::chunk_offset(row, 2 * cc)) = lo;
+                *reinterpret_cast<u32x4*>(dst + L::chunk_offset(row, 2 * cc + 1)) = hi;
+            }
+        } else {
+            const BandDesc b = bands[rel * NW + wave_s];
+            const int last = uniform(b.last);
+            const int64_t off = (static_cast<int64_t>(uniform(static_cast<int>(b.off >> 32))) << 32) |
+                                static_cast<uint32_t>(uniform(static_cast<int>(b.off)));
+            const uint8_t* base = IS_V ? reinterpret_cast<const uint8_t*>(a.v_new) + off + static_cast<int64_t>(-1 - tag) * a.v_fresh_delta
+                                       : reinterpret_cast<const uint8_t*>(a.k_new) + off;
+            const int64_t stride = (IS_V ? a.vn_st : a.kn_st) * 2;
+#pragma unroll
+            for (int j = 0; j < C::IPW; ++j) {
+                const int r = j * C::RPI + ln / C::CPR;
+                const int row = wave_s * C::ROWS_PER_WAVE + r;
+                const int64_t voff = static_cast<int64_t>(min(r, last)) * stride + cc * 32;
+                const u32x4 x0 = *reinterpret_cast<const u32x4*>(base + voff);
+                const u32x4 x1 = *reinterpret_cast<const u32x4*>(base + voff + 16);
+                // Wait here, inside the branch: a wait the compiler places where the two branches
+                // meet again would drain the asynchronous loads in every step.
+                __builtin_amdgcn_s_waitcnt(0x0f70);
+                *reinterpret_cast<u32x4*>(dst + L::chunk_offset(row, 2 * cc)) = x0;
+                *reinterpret_cast<u32x4*>(dst + L::chunk_offset(row, 2 * cc + 1)) = x1;
+            }
+        }
+    }
+
     // Make the compiler wait for the query loads here, once per item.  Left to itself it puts the
     // wait before their first use inside the tile loop, where it also drains the asynchronous tile
     // loads issued since, in every iteration.
@@ -396,6 +454,13 @@ struct StreamAttn : TileMath<HD, NB, NW, HIDDEN> {
         this->kvh = uniform(d.kvh);
         this->q0 = uniform(d.q0);
         this->sh.q_len = uniform(d.q_len);
+        if (KVB == 1) {
+            // read through the scalar cache into scalar registers: as vector loads the compiler keeps them
+            // in vector registers, spills those, and waits for every tile load in flight at each reload
+            k_mul = scalar_load(a.k_scale + this->kvh);
+            this->out_mul = scalar_load(a.v_scale + this->kvh);
+            v_inv = __builtin_bit_cast(float, uniform(__builtin_bit_cast(int, 1.0f / this->out_mul)));
+        }
         this->reset_accumulators();
     }
     // First key position the lane's query row does not see under the block-causal mask (fresh tiles
@@ -405,7 +470,11 @@ struct StreamAttn : TileMath<HD, NB, NW, HIDDEN> {
         const int q_len = uniform(d.q_len);
         const int r = this->row_of(uniform(d.rt), 0);
         const int i = r < a.group * q_len ? r % q_len : 0;
-        return (i / a.dbs + 1) * a.dbs;
+        // (the divisor made opaque here: its reciprocal, worked out once ahead of the tile loop, would be
+        // kept in scratch, and the reload waits for every tile load in flight)
+        int dbs = a.dbs;
+        asm volatile("" : "+s"(dbs));
+        return (i / dbs + 1) * dbs;
     }
     // Both at once, waiting for every outstanding load of the wave.
     DFX_D void begin_item_hidden(const UnitDesc& d) {
@@ -443,22 +512,23 @@ struct StreamAttn : TileMath<HD, NB, NW, HIDDEN> {
     }
 
     // Step r of the pipelined loop (softmax and O^T of unit r, S^T of unit r + 1, tile loads of unit
-    // r + 3) is "plain" if it needs none of the loop's case distinctions: unit r + 1 follows in the
-    // same run and needs no mask, and unit r + 3 is in the table with every wave's band a full band
-    // of cached rows.  Writes into the flags of every unit r the number of consecutive plain steps
+    // r + 3; r + 5 with a ring of codes) is "plain" if it needs none of the loop's case distinctions:
+    // unit r + 1 follows in the same run and needs no mask, and the unit to fetch is in the table with
+    // every wave's band a full band of cached rows.  Writes into the flags of every unit r the number of consecutive plain steps
     // from step r on (kUnitPlainShift).  One wave, one lane per unit; the table is complete
     // (barrier) and nobody else writes flags now; readers come behind a later barrier.
+    static constexpr int kPlainAhead = KVB == 1 ? C::kStages + 1 : C::kStages - 1;  // step r fetches unit r + kPlainAhead
     DFX_D void mark_plain_steps(int n_units) const {
         static_assert(C::kPlanUnits <= 64, "a lane per unit of the table");
         if (wave_s != NW - 1) return;
         const int r = thread_number_here(0);
         bool plain = false;
         int flags = 0;
-        if (r + 3 < n_units) {
+        if (r + kPlainAhead < n_units) {
             bool full = true;
 #pragma unroll
             for (int w = 0; w < NW; ++w) {
-                const BandDesc& b = bands[(r + 3) * NW + w];
+                const BandDesc& b = bands[(r + kPlainAhead) * NW + w];
                 full = full && b.is_ctx > 0 && b.last >= C::ROWS_PER_WAVE - 1;
             }
             flags = units[r].flags;
@@ -466,6 +536,8 @@ struct StreamAttn : TileMath<HD, NB, NW, HIDDEN> {
             const bool masked = nxt.base + C::TN > nxt.limit || unit_holes(nxt.flags) != 0 ||
                                 (!(nxt.flags & kUnitCtx) && a.mask_mode == DFX_MASK_BLOCK_CAUSAL);
             plain = full && !(flags & kUnitLast) && !masked;
+            // codes: the step also widens K of unit r + 2 and V of unit r + 1, and a plain one only knows cached rows
+            if (KVB == 1) plain = plain && (flags & nxt.flags & units[r + 2].flags & kUnitCtx) != 0;
         }
         const uint64_t not_plain = ~(__ballot(plain) >> r);  // bit j: step r + j is not plain (bits past 63 - r: set)
         if (plain) units[r].flags = flags | (__builtin_ctzll(not_plain) << kUnitPlainShift);
@@ -932,6 +1004,237 @@ paged_attn_pipe_kernel(const KArgs a) {
             if (next_opens) wait_async_loads<0>();  // the next item's query rows (and the tiles requested before them)
             at.finish_run(rel - 1, split);
             if (next_opens) at.adopt_item(at.units[run_end]);
+        }
+    }, on_work);
+}
+
+// The FP8 kernel with the pipelined tile step: the ring holds the codes as stored (4 stages of
+// 16 KB), and the blocks of attn_pipe_gen.h read two widened K tiles and two widened V tiles.  In
+// step r (softmax and O^T of unit r, S^T of unit r + 1) every wave widens its own rows of K of
+// unit r + 2 and of V of unit r + 1 -- the tiles the step before has just released -- and then
+// fetches unit r + 5 into the stage that frees.  Steps and units correspond one to one across the
+// items of a chunk, so the widening runs on through the ends of runs.  A wave only reads codes it
+// has loaded itself: the ring needs no barrier, and the step's one barrier orders the widened tiles.
+// The scales: cached K rows count k_scale (folded into the softmax constant of that tile), cached V
+// rows v_scale (O^T is kept in units of it: a fresh tile's exponentials are raised by 1 / v_scale
+// through their exponent, and its row sums, gathered apart, are multiplied back).
+template <int NW>
+__global__ void __launch_bounds__(64 * NW, 1) __attribute__((amdgpu_num_vgpr(32)))
+paged_attn_pipe_fp8_kernel(const KArgs a) {
+    extern __shared__ __attribute__((aligned(256))) uint8_t smem[];
+    constexpr int HD = 128;
+    using C = StreamCfg<HD, 1, NW, false, 1>;
+    using SA = StreamAttn<HD, 1, NW, false, 1, true>;
+    static_assert(C::kStages == 4 && C::LOADS_PER_UNIT == 2, "ring depth and wait counts below");
+    SA at(a, smem);
+    pipe_reserve();
+    {
+        const uint32_t o = static_cast<uint32_t>(at.lane / C::CPR) * static_cast<uint32_t>(a.c_st) + (at.lane % C::CPR) * 16;
+        pipe_set_load_offsets(o, o);
+    }
+    store_fresh_rows<HD, true, 1>(a);
+    const bool busy = at.wave < a.busy_waves;
+    constexpr int kHoleRows = C::ROWS_PER_WAVE;
+    static_assert(kHoleRows == 8, "mask blocks of attn_pipe_gen.h");
+    bool requested_early = false;
+    auto on_work = [&](const WgWork& w) {
+        UnitDesc d;
+        d.q0 = w.q0;
+        d.q_len = w.q_len;
+        d.kvh = w.kvh;
+        d.rt = w.rt;
+        at.request_queries(d);
+        requested_early = true;
+    };
+    auto as_scalar = [](float x) { return __builtin_bit_cast(float, uniform(__builtin_bit_cast(int, x))); };
+    // The current item's constants, in scalar registers from the moment the item is adopted (worked out
+    // where they are used, the compiler keeps their inputs in vector registers, and those in scratch):
+    // the log2-domain scale of a tile of cached rows, and what raises a fresh tile's exponentials by
+    // 1 / v_scale.
+    float c_ctx = 0.0f, fresh_shift = 0.0f;
+    auto adopt = [&](const UnitDesc& d) {
+        at.adopt_item(d);
+        c_ctx = as_scalar(a.c * at.k_mul);
+        fresh_shift = as_scalar(__builtin_amdgcn_logf(at.v_inv));
+    };
+    at.for_each_chunk([&](int n_units) {
+        const WgSplit& split = at.split;
+        const bool opens = (uniform(at.units[0].flags) & kUnitFirst) != 0;
+        if (opens && !requested_early) at.request_queries(at.units[0]);
+        requested_early = false;
+        at.mark_plain_steps(n_units);  // (while the query rows are on their way; first read behind a barrier)
+        if (opens) {
+            wait_async_loads<0>();
+            adopt(at.units[0]);
+        }
+        // ring fill, and the tiles the first step reads
+        int issued = 0;
+        for (; issued < C::kStages && issued < n_units; ++issued) at.issue_unit(issued);
+        at.wait_younger(max(issued - 2, 0));  // units 0 and 1 have landed
+        at.template widen_matrix<false>(0);
+        at.template widen_matrix<true>(0);
+        if (n_units > 1) at.template widen_matrix<false>(1);
+        if (issued < n_units) at.issue_unit(issued++);  // into the stage of unit 0
+
+        auto mask = [&](int r, bool set_a, float& mx_lane) {
+            const TileInfo t = at.tile_info_of(r);
+            const bool bc = !t.is_ctx && a.mask_mode == DFX_MASK_BLOCK_CAUSAL;
+            if (!(t.base + C::TN > t.limit || t.holes != 0 || bc)) return;
+            int lim = t.limit;
+            if (bc) lim = min(lim, at.visible_limit(at.units[r]));
+            const int thr = lim - t.base - 4 * at.half;
+            const uint32_t holes = static_cast<uint32_t>(t.holes);
+            if (set_a) pipe_mask_a_8(thr, holes, mx_lane);
+            else pipe_mask_b_8(thr, holes, mx_lane);
+        };
+        const bool compute_first = at.wave < NW / 2;
+
+        int rel = 0;
+        while (rel < n_units) {
+            const UnitDesc d = at.units[rel];
+            const int run_end = min(rel + uniform(d.run), n_units);
+            auto scale_of = [&](int r) { return (uniform(at.units[r].flags) & kUnitCtx) ? c_ctx : a.c; };
+
+            float mx_lane = 0.0f;
+            float neg_m = 0.0f;
+            auto prepare = [&](float c) {
+                const float m_tile = wave_xor32_max(mx_lane) * c;
+                float& m_run = at.m_run[0];
+                if (__any(m_tile > m_run + kRescaleThreshold)) {
+                    const float m_new = fmaxf(m_run, m_tile);
+                    if (__any(m_run != -INFINITY)) {
+                        const float alpha = (m_new == -INFINITY) ? 1.0f : fast_exp2(m_run - m_new);
+                        at.l_run[0] *= alpha;
+                        pipe_rescale_outputs(alpha);
+                    }
+                    m_run = m_new;
+                }
+                neg_m = (m_run == -INFINITY) ? 0.0f : -m_run;
+            };
+            // every wave has widened K of the run's first unit (at the latest a step ago; the chunk's
+            // first two units just now)
+            __builtin_amdgcn_s_waitcnt(0xc07f);
+            __builtin_amdgcn_s_barrier();
+            if (busy) {
+                pipe_first_scores(at.lds_address(at.wide_k(rel)) + at.k_lane, mx_lane);
+                mask(rel, true, mx_lane);
+                if (compute_first) prepare(scale_of(rel));
+            }
+            const bool next_opens = run_end < n_units;
+            // for the plain steps behind the run's first step: how many, and where the first of them fetches
+            const int plain_word = at.units[min(rel + 1, n_units - 1)].flags;
+            const uint64_t off_first = static_cast<uint64_t>(at.bands[min(rel + C::kStages + 2, n_units - 1) * NW + at.wave].off);
+            auto step = [&](int r, bool cur_is_a) {
+                const bool has_next = r + 1 < run_end;
+                // every wave has widened K of unit r + 1 and V of unit r and is done with step r - 1
+                __builtin_amdgcn_s_waitcnt(0xc07f);
+                __builtin_amdgcn_s_barrier();
+                auto refill = [&] {
+                    if (r + 2 < n_units) {
+                        at.wait_younger(issued - r - 3);
+                        at.template widen_matrix<false>(r + 2);
+                    }
+                    if (r + 1 < n_units) at.template widen_matrix<true>(r + 1);
+                    if (issued < n_units && issued < r + 2 + C::kStages) at.issue_unit(issued++);
+                };
+                const int flags = uniform(at.units[r].flags);
+                const bool cur_fresh = !(flags & kUnitCtx);
+                const float c_cur = cur_fresh ? a.c : c_ctx;
+                if (!compute_first || !busy) {
+                    refill();
+                    if (!has_next && next_opens) at.request_queries(at.units[run_end]);
+                    if (busy) prepare(c_cur);
+                } else if (!has_next && next_opens) {
+                    at.request_queries(at.units[run_end]);
+                }
+                if (busy) {
+                    const uint32_t v_cur = at.lds_address(at.wide_v(r)) + at.v_lane;
+                    const float l_before = at.l_run[0];
+                    float l_step = cur_fresh ? 0.0f : l_before;
+                    const float nm = cur_fresh ? neg_m + fresh_shift : neg_m;
+                    if (has_next) {
+                        const uint32_t k_next = at.lds_address(at.wide_k(r + 1)) + at.k_lane;
+                        if (cur_is_a) {
+                            pipe_step_ab_x(k_next, v_cur, c_cur, nm, l_step);
+                            pipe_step_ab_y(c_cur, nm, l_step, mx_lane);
+                        } else {
+                            pipe_step_ba_x(k_next, v_cur, c_cur, nm, l_step);
+                            pipe_step_ba_y(c_cur, nm, l_step, mx_lane);
+                        }
+                        mask(r + 1, !cur_is_a, mx_lane);
+                    } else {
+                        if (cur_is_a) {
+                            pipe_last_a_x(v_cur, c_cur, nm, l_step);
+                            pipe_last_a_y(c_cur, nm, l_step);
+                        } else {
+                            pipe_last_b_x(v_cur, c_cur, nm, l_step);
+                            pipe_last_b_y(c_cur, nm, l_step);
+                        }
+                    }
+                    at.l_run[0] = cur_fresh ? fmaf(l_step, at.out_mul, l_before) : l_step;
+                    if (compute_first) {
+                        refill();
+                        if (has_next) prepare(scale_of(r + 1));
+                    }
+                }
+            };
+            // A plain step (mark_plain_steps()): units r, r + 1 and r + 2 are tiles of cached rows, nothing to
+            // mask, and the unit to fetch is a full band of cached rows at `off`.
+            auto plain_step = [&](int r, bool cur_is_a, int64_t off) {
+                __builtin_amdgcn_s_waitcnt(0xc07f);
+                __builtin_amdgcn_s_barrier();
+                auto refill = [&] {
+                    wait_async_loads<2 * C::LOADS_PER_UNIT>();  // unit r + 2 has landed
+                    at.template widen_matrix<false, true>(r + 2);
+                    at.template widen_matrix<true, true>(r + 1);
+                    pipe_issue_band_fp8(a.k_cache + off, a.v_cache + off,
+                                        uniform(static_cast<int>(at.stages_lds + (static_cast<unsigned>(issued) % C::kStages) * C::STAGE_BYTES +
+                                                                 at.wave * (C::IPW * 1024))));
+                };
+                if (!compute_first || !busy) {
+                    refill();
+                    if (busy) prepare(c_ctx);
+                }
+                if (busy) {
+                    const uint32_t v_cur = at.lds_address(at.wide_v(r)) + at.v_lane;
+                    const uint32_t k_next = at.lds_address(at.wide_k(r + 1)) + at.k_lane;
+                    if (cur_is_a) {
+                        pipe_step_ab_x(k_next, v_cur, c_ctx, neg_m, at.l_run[0]);
+                        pipe_step_ab_y(c_ctx, neg_m, at.l_run[0], mx_lane);
+                    } else {
+                        pipe_step_ba_x(k_next, v_cur, c_ctx, neg_m, at.l_run[0]);
+                        pipe_step_ba_y(c_ctx, neg_m, at.l_run[0], mx_lane);
+                    }
+                    if (compute_first) {
+                        refill();
+                        prepare(c_ctx);
+                    }
+                }
+                ++issued;
+            };
+            auto band_offset = [&](int unit) { return static_cast<uint64_t>(at.bands[unit * NW + at.wave].off); };
+            auto uniform_offset = [&](uint64_t off) {
+                return (static_cast<int64_t>(uniform(static_cast<int>(off >> 32))) << 32) | static_cast<uint32_t>(uniform(static_cast<int>(off)));
+            };
+            bool first_step = true;
+            while (rel < run_end) {
+                step(rel++, true);
+                // in steady state the step about to run fetches unit rel + kStages + 1
+                if (first_step && rel < run_end && issued == rel + C::kStages + 1) {
+                    uint64_t off = off_first;
+                    for (int pairs = (uniform(plain_word) >> kUnitPlainShift) >> 1; pairs > 0; --pairs) {
+                        const uint64_t off_next = band_offset(issued + 1);
+                        plain_step(rel++, false, uniform_offset(off));
+                        off = band_offset(min(issued + 1, n_units - 1));
+                        plain_step(rel++, true, uniform_offset(off_next));
+                    }
+                }
+                first_step = false;
+                if (rel < run_end) step(rel++, false);
+            }
+            if (next_opens) wait_async_loads<0>();
+            at.finish_run(rel - 1, split);
+            if (next_opens) adopt(at.units[run_end]);
         }
     }, on_work);
 }

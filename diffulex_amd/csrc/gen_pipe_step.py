@@ -361,6 +361,12 @@ namespace dfx {
                         comment="The wave's four direct-to-LDS loads of a tile whose 8 rows of the wave are all cached rows (K rows at\n"
                                 "k_rows, V rows at v_rows, both wave-uniform; lds_dst: the wave's place in the K tile of the ring stage):\n"
                                 "no vector instruction, the offsets are those of pipe_set_load_offsets."))
+    issue8 = [f"s_add_u32 m0, %[d], 0", f"global_load_lds_dwordx4 {vr(LOAD_OFF)}, %[kb] nt",
+              f"s_add_u32 m0, %[d], {MAT_BYTES // 2}", f"global_load_lds_dwordx4 {vr(LOAD_OFF)}, %[vb] nt"]
+    parts.append(asm_fn("pipe_issue_band_fp8", "const void* k_rows, const void* v_rows, uint32_t lds_dst", join(issue8),
+                        ins=['[kb] "s"(k_rows)', '[vb] "s"(v_rows)', '[d] "s"(lds_dst)'], clobbers=["memory", "m0", "scc"],
+                        comment="The same for a cache of one-byte codes: a wave's 8 rows of a tile are one load each for K and V (the\n"
+                                "first offset of pipe_set_load_offsets), and the V codes of a stage follow its K codes."))
     for d in range(NDB):
         outs = [f'"=v"(x[{e}])' for e in range(16)]
         body = join(f"v_accvgpr_read_b32 %{e}, {ar(O_BASE + 16 * d + e)}" for e in range(16))

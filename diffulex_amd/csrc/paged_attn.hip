@@ -33,7 +33,7 @@ struct Plan {
     bool stream;   // streaming tile path (else generic)
     bool distinct; // the cache is in the "distinct" layout (generic path)
     bool compact;  // streaming path, two workgroups per compute unit
-    bool pipelined;  // streaming path, bf16 KV, 4-stage ring: software-pipelined tile step
+    bool pipelined;  // streaming path, 8 waves, 4-stage ring: software-pipelined tile step
     int64_t slot_floats;
 };
 
@@ -74,7 +74,7 @@ int make_plan(const dfx_attn_params* p, Plan& plan) {
     plan.compact = plan.stream && !plan.fp8 && plan.nb == 1 && p->num_seqs <= kCompactMaxSeqs;
     // (8 waves only: with 4 waves a wave has twice the tile loads to address, and the 32 registers
     // the pipelined kernel leaves the compiler no longer hold that without spilling in the loop)
-    plan.pipelined = plan.stream && !plan.fp8 && !plan.compact && plan.hd == 128 && plan.nb == 2 &&
+    plan.pipelined = plan.stream && !plan.compact && plan.hd == 128 && plan.nb == 2 &&
                      !(p->flags & DFX_ATTN_NO_PIPELINE);
     if (p->max_workgroups > 0) {
         plan.n_wg = p->max_workgroups;
@@ -133,6 +133,12 @@ int launch(const KArgs& ka, const Plan& plan, hipStream_t st, const PlanArgs* pa
         fill_lds = C::STAGES_OFF;
         threads = 64 * FNW;
         slot = kSlotBase + 3;
+        if constexpr (HD == 128 && FNW == 8) {
+            if (plan.pipelined) {
+                main_k = paged_attn_pipe_fp8_kernel<FNW>;
+                slot = 28;
+            }
+        }
     } else if constexpr (PATH == 2) {
         // 4 waves for up to 128 rows (then two workgroups per compute unit where the batch allows),
         // 8 waves (two per SIMD) for up to 256

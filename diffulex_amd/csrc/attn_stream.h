@@ -1031,7 +1031,12 @@ paged_attn_pipe_fp8_kernel(const KArgs a) {
     {
         const uint32_t o = static_cast<uint32_t>(at.lane / C::CPR) * static_cast<uint32_t>(a.c_st) + (at.lane % C::CPR) * 16;
         pipe_set_load_offsets(o, o);
+        const int row = at.wave * C::ROWS_PER_WAVE + at.lane / C::CPR, cc = at.lane % C::CPR;
+        const uint32_t wide = at.lds_address(at.wide_k(0));
+        pipe_set_widen_addresses(at.stages_lds + at.wave * (C::IPW * 1024) + at.lane * 16,
+                                 wide + SA::L::chunk_offset(row, 2 * cc), wide + SA::L::chunk_offset(row, 2 * cc + 1));
     }
+    static_assert(C::IPW == 1, "pipe_widen: one load of codes per wave and matrix");
     store_fresh_rows<HD, true, 1>(a);
     const bool busy = at.wave < a.busy_waves;
     constexpr int kHoleRows = C::ROWS_PER_WAVE;
@@ -1185,8 +1190,9 @@ paged_attn_pipe_fp8_kernel(const KArgs a) {
                 __builtin_amdgcn_s_barrier();
                 auto refill = [&] {
                     wait_async_loads<2 * C::LOADS_PER_UNIT>();  // unit r + 2 has landed
-                    at.template widen_matrix<false, true>(r + 2);
-                    at.template widen_matrix<true, true>(r + 1);
+                    pipe_widen((static_cast<unsigned>(r + 2) % C::kStages) * C::STAGE_BYTES,
+                               (static_cast<unsigned>(r + 1) % C::kStages) * C::STAGE_BYTES + C::MAT_BYTES,
+                               (r & 1) * SA::L::MAT_BYTES, (2 + ((r + 1) & 1)) * SA::L::MAT_BYTES);
                     pipe_issue_band_fp8(a.k_cache + off, a.v_cache + off,
                                         uniform(static_cast<int>(at.stages_lds + (static_cast<unsigned>(issued) % C::kStages) * C::STAGE_BYTES +
                                                                  at.wave * (C::IPW * 1024))));

@@ -24,6 +24,7 @@ Register map (head_dim 128; one 32-row query block per wave; 128 + 128 registers
     v[112:127] operand ring: four 4-register buffers (K operands in phase X, V^T in phase Y)
     v[32:42]   temporaries: exp2 pair, K operand address, 8 V^T operand addresses
     v[43:44]   the lane's byte offsets inside a band of cached rows (tile loads, pipe_issue_band)
+    v[45:47]   cache of one-byte codes: the lane's LDS addresses for pipe_widen
     v[0:31], a[0:31]  the compiler's
 The two score sets swap roles every step (steps AB and BA), so nothing is ever moved.  P (the
 bf16 pairs, the B operand of the second product) overwrites the current score set as it is
@@ -58,6 +59,7 @@ T_EXP = [TMP + 0, TMP + 1]  # exp2 arguments / results of the pair in flight
 T_ADDR = TMP + 2            # K operand address of the slab being read (phase X); scratch elsewhere
 T_VADDR = TMP + 3           # 8 V^T operand addresses (phase Y)
 LOAD_OFF = 43               # two registers: byte offsets of the lane's chunk in its two rows of a band of cached rows
+WIDEN_ADDR = 45             # three registers: LDS addresses for pipe_widen (cache of one-byte codes)
 MAT_BYTES = 64 * ROWB       # K tile; the V tile of a ring stage follows it
 NEG_INF = "0xff800000"
 MFMA_TO_VALU = ["s_nop 15", "s_nop 1"]  # 18 wait states: the longest the ISA asks for
@@ -367,6 +369,36 @@ namespace dfx {
                         ins=['[kb] "s"(k_rows)', '[vb] "s"(v_rows)', '[d] "s"(lds_dst)'], clobbers=["memory", "m0", "scc"],
                         comment="The same for a cache of one-byte codes: a wave's 8 rows of a tile are one load each for K and V (the\n"
                                 "first offset of pipe_set_load_offsets), and the V codes of a stage follow its K codes."))
+    parts.append(asm_fn("pipe_set_widen_addresses", "uint32_t raw, uint32_t lo, uint32_t hi",
+                        join(f"v_mov_b32 {vr(WIDEN_ADDR + j)}, %{j}" for j in range(3)), ins=['"v"(raw)', '"v"(lo)', '"v"(hi)'],
+                        comment="Once per kernel (cache of one-byte codes): LDS addresses of the 16 codes the lane widens in stage 0 of the\n"
+                                "ring (K; V follows at pipe_widen's offsets) and of the two 16-byte chunks they become in widened tile 0."))
+    w = Block()
+    ta, tb2 = TMP, TMP + 1
+    w.valu(f"v_add_u32 {vr(ta)}, %[rk], {vr(WIDEN_ADDR)}", {ta})
+    w.valu(f"v_add_u32 {vr(tb2)}, %[rv], {vr(WIDEN_ADDR)}", {tb2})
+    w.other(f"ds_read_b128 {vr(RING, 4)}, {vr(ta)}")
+    w.other(f"ds_read_b128 {vr(RING + 4, 4)}, {vr(tb2)}")
+    for j, (sel, which) in enumerate((("wk", 1), ("wk", 2), ("wv", 1), ("wv", 2))):
+        w.valu(f"v_add_u32 {vr(TMP + 2 + j)}, %[{sel}], {vr(WIDEN_ADDR + which)}", {TMP + 2 + j})
+    def widen(src, dst):  # 4 registers of codes -> 8 registers of bf16 pairs; dst may end on src's last registers
+        for q in range(4):
+            w.valu(f"v_cvt_scalef32_pk_bf16_fp8 {vr(dst + 2 * q)}, {vr(src + q)}, 1.0", {dst + 2 * q})
+            w.valu(f"v_cvt_scalef32_pk_bf16_fp8 {vr(dst + 2 * q + 1)}, {vr(src + q)}, 1.0 op_sel:[1,0,0]", {dst + 2 * q + 1})
+    w.other("s_waitcnt lgkmcnt(1)")
+    widen(RING, RING + 8)
+    w.other(f"ds_write_b128 {vr(TMP + 2)}, {vr(RING + 8, 4)}")
+    w.other(f"ds_write_b128 {vr(TMP + 3)}, {vr(RING + 12, 4)}")
+    w.other("s_waitcnt lgkmcnt(2)")
+    widen(RING + 4, RING)   # (register RING + 4 + q is read by the instructions that write RING + 2q, 2q + 1 <= RING + 4 + q: in order)
+    w.other(f"ds_write_b128 {vr(TMP + 4)}, {vr(RING, 4)}")
+    w.other(f"ds_write_b128 {vr(TMP + 5)}, {vr(RING + 4, 4)}")
+    parts.append(asm_fn("pipe_widen", "uint32_t raw_k, uint32_t raw_v, uint32_t wide_k, uint32_t wide_v", w.text(),
+                        ins=['[rk] "s"(raw_k)', '[rv] "s"(raw_v)', '[wk] "s"(wide_k)', '[wv] "s"(wide_v)'], clobbers=["memory"],
+                        comment="Widens the lane's 16 K codes at raw_k and 16 V codes at raw_v (byte offsets from the address given for\n"
+                                "stage 0) into the widened tiles at wide_k and wide_v (byte offsets from widened tile 0): both reads first,\n"
+                                "one instruction per pair of codes (exact), in the operand ring's registers, which are free between the\n"
+                                "blocks of two steps.  The writes are waited for by whatever waits for LDS next (lgkmcnt)."))
     for d in range(NDB):
         outs = [f'"=v"(x[{e}])' for e in range(16)]
         body = join(f"v_accvgpr_read_b32 %{e}, {ar(O_BASE + 16 * d + e)}" for e in range(16))

@@ -536,7 +536,7 @@ def main():
     gbs = nbytes / (ms * 1e-3) / 1e9
     tflops = nflops / (ms * 1e-3) / 1e12
     traffic, traffic_source = measured_traffic(args.workload, nbytes)
-    kernel = ("paged_attn_stream_fp8_kernel<128, 8>" if wl.kv_fp8 else
+    kernel = ("paged_attn_pipe_fp8_kernel<8>" if wl.kv_fp8 else
               "paged_attn_pipe_kernel<8>" if args.workload == "c3" else "paged_attn_stream_kernel")
     result = {
         "metric": "attn query-tokens/sec + achieved HBM GB/s (% of peak), Dream-7B shape, 1 GPU",

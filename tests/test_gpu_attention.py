@@ -122,6 +122,7 @@ FP8_EDGE_CASES = [
     dict(num_seqs=2, h_q=8, h_kv=1, hd=128, page=32, ctx=[100, 200], q_len=64, dbs=64),
     dict(num_seqs=3, h_q=6, h_kv=3, hd=128, page=24, ctx=[23, 24, 100], q_len=32, dbs=32),
     dict(num_seqs=70, h_q=4, h_kv=1, hd=128, page=64, ctx=(0, 200), q_len=32, dbs=32),   # more units than one plan holds
+    dict(num_seqs=40, h_q=14, h_kv=2, hd=128, page=64, ctx=(0, 1500), q_len=32, dbs=32),  # the same with 8 waves: long runs of plain steps across plans
     # head_dim 64: 4 waves with one (up to 128 rows) or two (up to 256 rows) query blocks each, several row tiles
     dict(num_seqs=4, h_q=8, h_kv=2, hd=64, page=32, ctx=[0, 63, 64, 500], q_len=32, dbs=32),
     dict(num_seqs=3, h_q=14, h_kv=2, hd=64, page=256, ctx=[255, 700, 1300], q_len=32, dbs=32),
@@ -129,7 +130,7 @@ FP8_EDGE_CASES = [
 ]
 
 
-@pytest.mark.parametrize("flags", PATHS)
+@pytest.mark.parametrize("flags", PATHS + [_lib.DFX_ATTN_NO_PIPELINE])
 @pytest.mark.parametrize("case", FP8_EDGE_CASES)
 @pytest.mark.parametrize("mask", [MASK_FULL, MASK_BLOCK_CAUSAL])
 def test_fp8_edge_cases(dev, case, mask, flags):

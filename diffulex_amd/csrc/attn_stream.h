@@ -852,10 +852,14 @@ paged_attn_pipe_kernel(const KArgs a) {
         // half of the workgroup behind its matrix work, at the end of a step, and by the upper half
         // in front of it: while one wave of a SIMD does that, the other has the matrix unit.
         const bool compute_first = at.wave < NW / 2;
+        // Under the block-causal mask: the fresh key position up to which every query row of the current
+        // run's row tile sees everything (set where a run begins).  A fresh tile that ends at or below it
+        // needs no mask; in a prefill those are all of a row tile's tiles but the last few.
+        int bc_clear = 0;
         // Mask of the score set that holds unit r, if that tile needs one; updates the lane maximum.
         auto mask = [&](int r, bool set_a, float& mx_lane) {
             const TileInfo t = at.tile_info_of(r);
-            const bool bc = !t.is_ctx && a.mask_mode == DFX_MASK_BLOCK_CAUSAL;
+            const bool bc = !t.is_ctx && a.mask_mode == DFX_MASK_BLOCK_CAUSAL && t.base + C::TN > bc_clear;
             if (!(t.base + C::TN > t.limit || t.holes != 0 || bc)) return;
             int lim = t.limit;
             if (bc) lim = min(lim, at.visible_limit(at.units[r]));
@@ -876,6 +880,18 @@ paged_attn_pipe_kernel(const KArgs a) {
             const UnitDesc d = at.units[rel];
             const int run_end = min(rel + uniform(d.run), n_units);
             // (an item that opens inside the chunk was adopted when the run before it ended)
+            if (a.mask_mode == DFX_MASK_BLOCK_CAUSAL) {
+                // the row tile's rows are (head of the group, query position) pairs, position minor: within
+                // one head the first row has the lowest position, across heads position 0 is among them
+                const int q_len = uniform(d.q_len);
+                const int r_lo = uniform(d.rt) * C::RT;
+                const int r_hi = min(r_lo + C::RT, a.group * q_len) - 1;
+                const int g_lo = r_lo / q_len;
+                const int first_pos = g_lo == r_hi / q_len ? r_lo - g_lo * q_len : 0;
+                int dbs = a.dbs;
+                asm volatile("" : "+s"(dbs));
+                bc_clear = uniform((first_pos / dbs + 1) * dbs);
+            }
 
             // S^T of the run's first tile (into score set A), with nothing to overlap it with
             if (admit(rel, rel)) at.issue_unit(issued++);

@@ -476,6 +476,19 @@ struct StreamAttn : TileMath<HD, NB, NW, HIDDEN> {
         asm volatile("" : "+s"(dbs));
         return (i / dbs + 1) * dbs;
     }
+    // Under the block-causal mask: the fresh key position up to which every query row of row tile rt of
+    // an item with q_len query positions sees everything.  The tile's rows are (head of the group, query
+    // position) pairs, position minor: within one head the first row has the lowest position, across
+    // heads position 0 is among them.
+    DFX_D int clear_limit(int rt, int q_len) const {
+        const int r_lo = rt * C::RT;
+        const int r_hi = min(r_lo + C::RT, a.group * q_len) - 1;
+        const int g_lo = r_lo / q_len;
+        const int first_pos = g_lo == r_hi / q_len ? r_lo - g_lo * q_len : 0;
+        int dbs = a.dbs;
+        asm volatile("" : "+s"(dbs));
+        return (first_pos / dbs + 1) * dbs;
+    }
     // Both at once, waiting for every outstanding load of the wave.
     DFX_D void begin_item_hidden(const UnitDesc& d) {
         request_queries(d);
@@ -518,7 +531,8 @@ struct StreamAttn : TileMath<HD, NB, NW, HIDDEN> {
     // from step r on (kUnitPlainShift).  One wave, one lane per unit; the table is complete
     // (barrier) and nobody else writes flags now; readers come behind a later barrier.
     static constexpr int kPlainAhead = KVB == 1 ? C::kStages + 1 : C::kStages - 1;  // step r fetches unit r + kPlainAhead
-    DFX_D void mark_plain_steps(int n_units) const {
+    // fresh_bands: the kernel's plain steps fetch bands of fresh rows (a launch without a cache) instead of cached ones.
+    DFX_D void mark_plain_steps(int n_units, bool fresh_bands = false) const {
         static_assert(C::kPlanUnits <= 64, "a lane per unit of the table");
         if (wave_s != NW - 1) return;
         const int r = thread_number_here(0);
@@ -529,12 +543,13 @@ struct StreamAttn : TileMath<HD, NB, NW, HIDDEN> {
 #pragma unroll
             for (int w = 0; w < NW; ++w) {
                 const BandDesc& b = bands[(r + kPlainAhead) * NW + w];
-                full = full && b.is_ctx > 0 && b.last >= C::ROWS_PER_WAVE - 1;
+                full = full && (b.is_ctx > 0) != fresh_bands && b.last >= C::ROWS_PER_WAVE - 1;
             }
             flags = units[r].flags;
             const UnitDesc& nxt = units[r + 1];
-            const bool masked = nxt.base + C::TN > nxt.limit || unit_holes(nxt.flags) != 0 ||
-                                (!(nxt.flags & kUnitCtx) && a.mask_mode == DFX_MASK_BLOCK_CAUSAL);
+            bool masked = nxt.base + C::TN > nxt.limit || unit_holes(nxt.flags) != 0;
+            if (!(nxt.flags & kUnitCtx) && a.mask_mode == DFX_MASK_BLOCK_CAUSAL)
+                masked = masked || nxt.base + C::TN > clear_limit(nxt.rt, nxt.q_len);
             plain = full && !(flags & kUnitLast) && !masked;
             // codes: the step also widens K of unit r + 2 and V of unit r + 1, and a plain one only knows cached rows
             if (KVB == 1) plain = plain && (flags & nxt.flags & units[r + 2].flags & kUnitCtx) != 0;
@@ -781,7 +796,11 @@ __global__ void __launch_bounds__(64 * NW, 1) paged_attn_stream_fp8_kernel(const
 //
 // amdgpu_num_vgpr(32): the compiler allocates v0..v31 and a0..a31 only; the registers above hold
 // the matrix state of the generated blocks, which the compiler never sees.
-template <int NW>
+//
+// PREFILL: the variant for launches without a cache whose k_new and v_new have one layout.  Every tile
+// is one of fresh rows there, and its plain steps fetch full bands of those the way the other variant's
+// fetch bands of cached rows (which keeps its fresh tiles, one or two per item, on the general step).
+template <int NW, bool PREFILL = false>
 __global__ void __launch_bounds__(64 * NW, 1) __attribute__((amdgpu_num_vgpr(32)))
 paged_attn_pipe_kernel(const KArgs a) {
     extern __shared__ __attribute__((aligned(256))) uint8_t smem[];
@@ -799,6 +818,13 @@ paged_attn_pipe_kernel(const KArgs a) {
             o[j] = static_cast<uint32_t>(r) * static_cast<uint32_t>(a.c_st * 2) + chunk * 16;
         }
         pipe_set_load_offsets(o[0], o[1]);
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int r = j * C::RPI + at.lane / C::CPR;
+            const int chunk = (at.lane % C::CPR) ^ C::swizzle(at.wave * C::ROWS_PER_WAVE + r);
+            o[j] = static_cast<uint32_t>(r) * static_cast<uint32_t>(a.kn_st * 2) + chunk * 16;
+        }
+        if constexpr (PREFILL) pipe_set_fresh_offsets(o[0], o[1]);
     }
     store_fresh_rows<HD, false, 1>(a);
     const bool busy = at.wave < a.busy_waves;  // waves whose 32 rows exist in no item of this launch only fetch
@@ -827,7 +853,7 @@ paged_attn_pipe_kernel(const KArgs a) {
         // behind the barrier of the first run's first step; they only add bits to the flags that
         // nobody looks at before.  (Not behind the ring fill: a spilled register reloaded here would
         // wait for every tile of it.)
-        at.mark_plain_steps(n_units);
+        at.mark_plain_steps(n_units, PREFILL);
         __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the marks are written before this wave reaches that barrier
         if (opens) {
             wait_async_loads<0>();
@@ -880,18 +906,7 @@ paged_attn_pipe_kernel(const KArgs a) {
             const UnitDesc d = at.units[rel];
             const int run_end = min(rel + uniform(d.run), n_units);
             // (an item that opens inside the chunk was adopted when the run before it ended)
-            if (a.mask_mode == DFX_MASK_BLOCK_CAUSAL) {
-                // the row tile's rows are (head of the group, query position) pairs, position minor: within
-                // one head the first row has the lowest position, across heads position 0 is among them
-                const int q_len = uniform(d.q_len);
-                const int r_lo = uniform(d.rt) * C::RT;
-                const int r_hi = min(r_lo + C::RT, a.group * q_len) - 1;
-                const int g_lo = r_lo / q_len;
-                const int first_pos = g_lo == r_hi / q_len ? r_lo - g_lo * q_len : 0;
-                int dbs = a.dbs;
-                asm volatile("" : "+s"(dbs));
-                bc_clear = uniform((first_pos / dbs + 1) * dbs);
-            }
+            if (a.mask_mode == DFX_MASK_BLOCK_CAUSAL) bc_clear = uniform(at.clear_limit(uniform(d.rt), uniform(d.q_len)));
 
             // S^T of the run's first tile (into score set A), with nothing to overlap it with
             if (admit(rel, rel)) at.issue_unit(issued++);
@@ -900,7 +915,8 @@ paged_attn_pipe_kernel(const KArgs a) {
             // of the unit the first of them fetches (in steady state, which is checked there, step
             // rel + 1 fetches unit rel + 1 + kStages - 1, whatever the first step had to fetch).
             const int plain_word = at.units[min(rel + 1, n_units - 1)].flags;
-            const uint64_t off_first = static_cast<uint64_t>(at.bands[min(rel + C::kStages, n_units - 1) * NW + at.wave].off);
+            auto band_offset = [&](int unit) { return static_cast<uint64_t>(at.bands[unit * NW + at.wave].off); };
+            const uint64_t off_first = band_offset(min(rel + C::kStages, n_units - 1));
             float mx_lane = 0.0f;  // the lane's maximum over the score set that is consumed next
             float neg_m = 0.0f;    // minus the running maximum the exponentials of the next step refer to
             // Raise the running maximum (and rescale O^T and the row sum) if the tile about to be
@@ -969,12 +985,16 @@ paged_attn_pipe_kernel(const KArgs a) {
             // A plain step (mark_plain_steps()): the same work with the decisions taken out; `off` is
             // the offset of this wave's band of the unit to fetch.
             auto plain_step = [&](int r, bool cur_is_a, int64_t off) {
+                auto issue_band = [&](int dst) {
+                    if constexpr (PREFILL) pipe_issue_band_fresh(reinterpret_cast<const uint8_t*>(a.k_new) + off, reinterpret_cast<const uint8_t*>(a.v_new) + off, dst);
+                    else pipe_issue_band(a.k_cache + off, a.v_cache + off, dst);
+                };
                 wait_async_loads<C::LOADS_PER_UNIT>();  // unit r + 1 has landed; unit r + 2 may be on its way
                 __builtin_amdgcn_s_barrier();
                 const int dst = uniform(static_cast<int>(at.stages_lds + (static_cast<unsigned>(issued) % C::kStages) * C::STAGE_BYTES +
                                                          at.wave * (C::IPW * 1024)));
                 if (!compute_first || !busy) {
-                    pipe_issue_band(a.k_cache + off, a.v_cache + off, dst);
+                    issue_band(dst);
                     if (busy) prepare();
                 }
                 if (busy) {
@@ -988,13 +1008,12 @@ paged_attn_pipe_kernel(const KArgs a) {
                         pipe_step_ba_y(a.c, neg_m, at.l_run[0], mx_lane);
                     }
                     if (compute_first) {
-                        pipe_issue_band(a.k_cache + off, a.v_cache + off, dst);
+                        issue_band(dst);
                         prepare();
                     }
                 }
                 ++issued;
             };
-            auto band_offset = [&](int unit) { return static_cast<uint64_t>(at.bands[unit * NW + at.wave].off); };
             auto uniform_offset = [&](uint64_t off) {
                 return (static_cast<int64_t>(uniform(static_cast<int>(off >> 32))) << 32) | static_cast<uint32_t>(uniform(static_cast<int>(off)));
             };

@@ -24,7 +24,8 @@ Register map (head_dim 128; one 32-row query block per wave; 128 + 128 registers
     v[112:127] operand ring: four 4-register buffers (K operands in phase X, V^T in phase Y)
     v[32:42]   temporaries: exp2 pair, K operand address, 8 V^T operand addresses
     v[43:44]   the lane's byte offsets inside a band of cached rows (tile loads, pipe_issue_band)
-    v[45:47]   cache of one-byte codes: the lane's LDS addresses for pipe_widen
+    v[45:47]   cache of one-byte codes: the lane's LDS addresses for pipe_widen;
+               two-byte elements: v[45:46] the lane's byte offsets inside a band of fresh rows (pipe_issue_band_fresh)
     v[0:31], a[0:31]  the compiler's
 The two score sets swap roles every step (steps AB and BA), so nothing is ever moved.  P (the
 bf16 pairs, the B operand of the second product) overwrites the current score set as it is
@@ -60,6 +61,7 @@ T_ADDR = TMP + 2            # K operand address of the slab being read (phase X)
 T_VADDR = TMP + 3           # 8 V^T operand addresses (phase Y)
 LOAD_OFF = 43               # two registers: byte offsets of the lane's chunk in its two rows of a band of cached rows
 WIDEN_ADDR = 45             # three registers: LDS addresses for pipe_widen (cache of one-byte codes)
+FRESH_OFF = 45              # two registers: LOAD_OFF for a band of fresh rows (two-byte cache elements: no pipe_widen there)
 MAT_BYTES = 64 * ROWB       # K tile; the V tile of a ring stage follows it
 NEG_INF = "0xff800000"
 MFMA_TO_VALU = ["s_nop 15", "s_nop 1"]  # 18 wait states: the longest the ISA asks for
@@ -363,6 +365,14 @@ namespace dfx {
                         comment="The wave's four direct-to-LDS loads of a tile whose 8 rows of the wave are all cached rows (K rows at\n"
                                 "k_rows, V rows at v_rows, both wave-uniform; lds_dst: the wave's place in the K tile of the ring stage):\n"
                                 "no vector instruction, the offsets are those of pipe_set_load_offsets."))
+    parts.append(asm_fn("pipe_set_fresh_offsets", "uint32_t o0, uint32_t o1",
+                        join(f"v_mov_b32 {vr(FRESH_OFF + j)}, %{j}" for j in range(2)), ins=['"v"(o0)', '"v"(o1)'],
+                        comment="Once per kernel (two-byte cache elements): the same offsets for a band of fresh rows, whose rows lie a\n"
+                                "token of k_new apart (and of v_new: only used where the two have one layout)."))
+    parts.append(asm_fn("pipe_issue_band_fresh", "const void* k_rows, const void* v_rows, uint32_t lds_dst",
+                        join(issue).replace(vr(LOAD_OFF + 1), vr(FRESH_OFF + 1)).replace(vr(LOAD_OFF), vr(FRESH_OFF)),
+                        ins=['[kb] "s"(k_rows)', '[vb] "s"(v_rows)', '[d] "s"(lds_dst)'], clobbers=["memory", "m0", "scc"],
+                        comment="pipe_issue_band() for a full band of fresh rows (offsets of pipe_set_fresh_offsets)."))
     issue8 = [f"s_add_u32 m0, %[d], 0", f"global_load_lds_dwordx4 {vr(LOAD_OFF)}, %[kb] nt",
               f"s_add_u32 m0, %[d], {MAT_BYTES // 2}", f"global_load_lds_dwordx4 {vr(LOAD_OFF)}, %[vb] nt"]
     parts.append(asm_fn("pipe_issue_band_fp8", "const void* k_rows, const void* v_rows, uint32_t lds_dst", join(issue8),

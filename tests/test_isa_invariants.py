@@ -78,7 +78,8 @@ def test_tile_loop_has_no_spills_and_no_compiler_waits(isa, kernel, max_waits):
     assert ops["global_load_lds_dwordx4"] in (2, 4, 8)   # a wave's share of the 64 * head_dim * elt * 2 bytes of a tile
 
 
-PIPE_KERNELS = ["_ZN3dfx22paged_attn_pipe_kernelILi8E", "_ZN3dfx26paged_attn_pipe_fp8_kernelILi8E"]
+PIPE_KERNELS = ["_ZN3dfx22paged_attn_pipe_kernelILi8ELb0E", "_ZN3dfx22paged_attn_pipe_kernelILi8ELb1E",
+                "_ZN3dfx26paged_attn_pipe_fp8_kernelILi8E"]
 
 
 @pytest.mark.parametrize("kernel", PIPE_KERNELS)

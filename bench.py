@@ -291,7 +291,7 @@ def bench_prefill(args, dev):
                                f"block-causal mask, {dbs}-token blocks, no cache", "spin_up_launches": n_spin},
         "roofline": {"bound": "mfma", "achieved": tflops, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": tflops / MFMA_BF16_PEAK_TFLOPS, "traffic": None, "algorithmic_flops": nflops,
-                     "kernel": "paged_attn_stream_kernel<128, 1, 8, false>, duration = timed region / steps"},
+                     "kernel": "paged_attn_pipe_kernel<8, true>, duration = timed region / steps"},
     }))
 
 
@@ -423,7 +423,7 @@ def bench_layer(args, dev):
                    "tensor_sets_rotated": n_sets, "spin_up_launches": n_spin},
         "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS,
                      "traffic": None, "algorithmic_bytes": nbytes,
-                     "kernel": "rope_kv_store_kernel + paged_attn_pipe_kernel<8> (+ plan kernels once per graph), "
+                     "kernel": "rope_kv_store_kernel + paged_attn_pipe_kernel<8, false> (+ plan kernels once per graph), "
                                "duration = graph replay / layers"},
     }))
 
@@ -537,7 +537,7 @@ def main():
     tflops = nflops / (ms * 1e-3) / 1e12
     traffic, traffic_source = measured_traffic(args.workload, nbytes)
     kernel = ("paged_attn_pipe_fp8_kernel<8>" if wl.kv_fp8 else
-              "paged_attn_pipe_kernel<8>" if args.workload == "c3" else "paged_attn_stream_kernel")
+              "paged_attn_pipe_kernel<8, false>" if args.workload == "c3" else "paged_attn_stream_kernel")
     result = {
         "metric": "attn query-tokens/sec + achieved HBM GB/s (% of peak), Dream-7B shape, 1 GPU",
         "value": wl.total_q_tokens / (ms * 1e-3), "unit": "query-tokens/s",

@@ -112,7 +112,9 @@ struct StreamCfg : Shape<HD, NB, NW> {
     static constexpr int IPW = MAT_BYTES / 1024 / NW;  // loads per wave per matrix per tile
     static constexpr int LOADS_PER_UNIT = 2 * IPW;
     static constexpr int ROWS_PER_WAVE = IPW * RPI;        // 16 (4 waves) or 8 (8 waves)
-    static constexpr int kPlanUnits = COMPACT ? 32 : 512 / NW;  // units planned (and then streamed) at a time
+    // units described (and then streamed) at a time: the tile loop drains and refills its ring at the end of
+    // every table (≈ 5 µs), so as many as the LDS of a compute unit has room for beside the tiles
+    static constexpr int kPlanUnits = COMPACT ? 32 : (NW == 8 ? 88 : 128);
     static constexpr int PREFIX_BYTES = COMPACT ? (kCompactMaxSeqs + 1) * 4 : S::PREFIX_BYTES;
     static constexpr int UNIT_TABLE_BYTES = kPlanUnits * static_cast<int>(sizeof(UnitDesc));
     static constexpr int BAND_TABLE_BYTES = kPlanUnits * NW * static_cast<int>(sizeof(BandDesc));
@@ -533,31 +535,39 @@ struct StreamAttn : TileMath<HD, NB, NW, HIDDEN> {
     static constexpr int kPlainAhead = KVB == 1 ? C::kStages + 1 : C::kStages - 1;  // step r fetches unit r + kPlainAhead
     // fresh_bands: the kernel's plain steps fetch bands of fresh rows (a launch without a cache) instead of cached ones.
     DFX_D void mark_plain_steps(int n_units, bool fresh_bands = false) const {
-        static_assert(C::kPlanUnits <= 64, "a lane per unit of the table");
         if (wave_s != NW - 1) return;
-        const int r = thread_number_here(0);
-        bool plain = false;
-        int flags = 0;
-        if (r + kPlainAhead < n_units) {
-            bool full = true;
+        const int lane_here = thread_number_here(0);
+        // 64 units at a time, the last ones first: a stretch that reaches the end of its 64 goes on with
+        // the count of the unit behind it
+        int next_count = 0;
+        for (int first = ((n_units - 1) / 64) * 64; first >= 0; first -= 64) {
+            const int r = first + lane_here;
+            bool plain = false;
+            int flags = 0;
+            if (r + kPlainAhead < n_units) {
+                bool full = true;
 #pragma unroll
-            for (int w = 0; w < NW; ++w) {
-                const BandDesc& b = bands[(r + kPlainAhead) * NW + w];
-                full = full && (b.is_ctx > 0) != fresh_bands && b.last >= C::ROWS_PER_WAVE - 1;
+                for (int w = 0; w < NW; ++w) {
+                    const BandDesc& b = bands[(r + kPlainAhead) * NW + w];
+                    full = full && (b.is_ctx > 0) != fresh_bands && b.last >= C::ROWS_PER_WAVE - 1;
+                }
+                flags = units[r].flags;
+                const UnitDesc& nxt = units[r + 1];
+                bool masked = nxt.base + C::TN > nxt.limit || unit_holes(nxt.flags) != 0;
+                if (!(nxt.flags & kUnitCtx) && a.mask_mode == DFX_MASK_BLOCK_CAUSAL)
+                    masked = masked || nxt.base + C::TN > clear_limit(nxt.rt, nxt.q_len);
+                plain = full && !(flags & kUnitLast) && !masked;
+                // codes: the step also widens K of unit r + 2 and V of unit r + 1, and a plain one only knows cached rows
+                if (KVB == 1) plain = plain && (flags & nxt.flags & units[r + 2].flags & kUnitCtx) != 0;
             }
-            flags = units[r].flags;
-            const UnitDesc& nxt = units[r + 1];
-            bool masked = nxt.base + C::TN > nxt.limit || unit_holes(nxt.flags) != 0;
-            if (!(nxt.flags & kUnitCtx) && a.mask_mode == DFX_MASK_BLOCK_CAUSAL)
-                masked = masked || nxt.base + C::TN > clear_limit(nxt.rt, nxt.q_len);
-            plain = full && !(flags & kUnitLast) && !masked;
-            // codes: the step also widens K of unit r + 2 and V of unit r + 1, and a plain one only knows cached rows
-            if (KVB == 1) plain = plain && (flags & nxt.flags & units[r + 2].flags & kUnitCtx) != 0;
+            const uint64_t votes = __ballot(plain);
+            const uint64_t not_plain = ~(votes >> lane_here);  // bit j: step r + j is not plain (bits past 63 - lane: set)
+            int count = __builtin_ctzll(not_plain);
+            if (count == 64 - lane_here) count += next_count;  // (the stretch runs into the next 64)
+            if (plain) units[r].flags = flags | (count << kUnitPlainShift);  // (at most kPlanUnits: the flags' top bits are free)
+            next_count = (votes & 1) ? uniform(count) : 0;     // lane 0 holds the first unit of these 64
         }
-        const uint64_t not_plain = ~(__ballot(plain) >> r);  // bit j: step r + j is not plain (bits past 63 - r: set)
-        if (plain) units[r].flags = flags | (__builtin_ctzll(not_plain) << kUnitPlainShift);
     }
-
     // ---- the workgroup's work -----------------------------------------------------------------
     // Calls body(n_units) for every chunk of the workgroup's units, with the chunk's descriptors in
     // the LDS tables and begin / end set to the range of the unit space the chunk belongs to.  The

@@ -255,6 +255,7 @@ DFX_HD int pair_critical_length(int l, int s) {
 
 // Tiles the long item of a pair donates so that its owner meets M (0: the pair is not cut).
 DFX_HD int pair_donation(int l, int s, int M) {
+    (void)s;
     if (l <= M) return 0;
     int d = l + kPairCostMerge - M;       // owner: l - d + merge <= M
     if (d > l - 1) d = l - 1;             // the owner keeps at least the item's last tile

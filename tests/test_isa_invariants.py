@@ -33,7 +33,8 @@ def isa(tmp_path_factory):
 
 
 def _tile_loop(isa_text, mangled_prefix):
-    """Instructions of the innermost loop that contains every matrix instruction of the kernel."""
+    """Instructions of the innermost loop that contains every matrix instruction of the kernel and its
+    tile loads (a jump from a peeled iteration into the middle of the loop looks like a smaller one)."""
     m = re.search(r"^(%s\w*):" % re.escape(mangled_prefix), isa_text, re.M)
     assert m, mangled_prefix
     body = [l.strip() for l in isa_text[m.start():isa_text.index("s_endpgm", m.start())].split("\n")]
@@ -44,7 +45,8 @@ def _tile_loop(isa_text, mangled_prefix):
         mm = re.search(r"s_c?branch\S*\s+(\.LBB\d+_\d+)", l)
         if mm and mm.group(1) in labels:
             t = labels[mm.group(1)]
-            if t < mfma[0] and i > mfma[-1] and (best is None or i - t < best[1] - best[0]):
+            if t < mfma[0] and i > mfma[-1] and (best is None or i - t < best[1] - best[0]) and \
+                    any(x.startswith("global_load_lds") for x in body[t:i]):
                 best = (t, i)
     assert best, "no loop around the matrix instructions"
     return [l for l in body[best[0]:best[1] + 1] if l and not l.startswith((";", "."))]

@@ -556,6 +556,7 @@ def test_store_fused_into_the_attention_launch(dev, name, over, flags):
     ("c3", dict(num_seqs=4, ctx=[700, 256, 1000, 90], page=32)),
     ("c3", dict(num_seqs=3, ctx=[700, 513, 1000])),                    # page 256: whole tiles vanish
     ("c5", dict(num_seqs=3, ctx=[700, 513, 1000])),
+    ("c5", dict(num_seqs=3, ctx=[700, 513, 1000], page=32)),           # FP8: bands of a tile missing, masked per band
     ("c4", dict(num_seqs=2, ctx=[300, 95], page=48)),
 ])
 def test_pages_with_negative_table_entries_are_skipped(dev, name, over, flags):

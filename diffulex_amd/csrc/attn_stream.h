@@ -807,7 +807,7 @@ __global__ void __launch_bounds__(64 * NW, 1) paged_attn_stream_fp8_kernel(const
 // amdgpu_num_vgpr(32): the compiler allocates v0..v31 and a0..a31 only; the registers above hold
 // the matrix state of the generated blocks, which the compiler never sees.
 //
-// PREFILL: the variant for launches without a cache whose k_new and v_new have one layout.  Every tile
+// PREFILL: the variant for launches without a cache.  Every tile
 // is one of fresh rows there, and its plain steps fetch full bands of those the way the other variant's
 // fetch bands of cached rows (which keeps its fresh tiles, one or two per item, on the general step).
 template <int NW, bool PREFILL = false>
@@ -834,7 +834,17 @@ paged_attn_pipe_kernel(const KArgs a) {
             const int chunk = (at.lane % C::CPR) ^ C::swizzle(at.wave * C::ROWS_PER_WAVE + r);
             o[j] = static_cast<uint32_t>(r) * static_cast<uint32_t>(a.kn_st * 2) + chunk * 16;
         }
-        if constexpr (PREFILL) pipe_set_fresh_offsets(o[0], o[1]);
+        if constexpr (PREFILL) {
+            pipe_set_fresh_offsets(o[0], o[1]);
+            // (no cache: the registers of the cached rows' offsets take those of the fresh V rows)
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const int r = j * C::RPI + at.lane / C::CPR;
+                const int chunk = (at.lane % C::CPR) ^ C::swizzle(at.wave * C::ROWS_PER_WAVE + r);
+                o[j] = static_cast<uint32_t>(r) * static_cast<uint32_t>(a.vn_st * 2) + chunk * 16;
+            }
+            pipe_set_load_offsets(o[0], o[1]);
+        }
     }
     store_fresh_rows<HD, false, 1>(a);
     const bool busy = at.wave < a.busy_waves;  // waves whose 32 rows exist in no item of this launch only fetch
@@ -926,7 +936,11 @@ paged_attn_pipe_kernel(const KArgs a) {
             // rel + 1 fetches unit rel + 1 + kStages - 1, whatever the first step had to fetch).
             const int plain_word = at.units[min(rel + 1, n_units - 1)].flags;
             auto band_offset = [&](int unit) { return static_cast<uint64_t>(at.bands[unit * NW + at.wave].off); };
+            // (fresh rows: the index of the band's first row, from which the V offset follows where v_new has
+            // another token stride than k_new; cached rows have one offset for both)
+            auto band_row = [&](int unit) { return PREFILL ? -1 - at.bands[unit * NW + at.wave].is_ctx : 0; };
             const uint64_t off_first = band_offset(min(rel + C::kStages, n_units - 1));
+            const int row_first = band_row(min(rel + C::kStages, n_units - 1));
             float mx_lane = 0.0f;  // the lane's maximum over the score set that is consumed next
             float neg_m = 0.0f;    // minus the running maximum the exponentials of the next step refer to
             // Raise the running maximum (and rescale O^T and the row sum) if the tile about to be
@@ -994,9 +1008,10 @@ paged_attn_pipe_kernel(const KArgs a) {
             };
             // A plain step (mark_plain_steps()): the same work with the decisions taken out; `off` is
             // the offset of this wave's band of the unit to fetch.
-            auto plain_step = [&](int r, bool cur_is_a, int64_t off) {
+            auto plain_step = [&](int r, bool cur_is_a, int64_t off, int row) {
                 auto issue_band = [&](int dst) {
-                    if constexpr (PREFILL) pipe_issue_band_fresh(reinterpret_cast<const uint8_t*>(a.k_new) + off, reinterpret_cast<const uint8_t*>(a.v_new) + off, dst);
+                    if constexpr (PREFILL) pipe_issue_band_fresh(reinterpret_cast<const uint8_t*>(a.k_new) + off,
+                                                                 reinterpret_cast<const uint8_t*>(a.v_new) + off + static_cast<int64_t>(row) * a.v_fresh_delta, dst);
                     else pipe_issue_band(a.k_cache + off, a.v_cache + off, dst);
                 };
                 wait_async_loads<C::LOADS_PER_UNIT>();  // unit r + 1 has landed; unit r + 2 may be on its way
@@ -1036,11 +1051,14 @@ paged_attn_pipe_kernel(const KArgs a) {
                 step(rel++, true);
                 if (first_step && rel < run_end && issued == rel + C::kStages - 1) {
                     uint64_t off = off_first;
+                    int row = row_first;
                     for (int pairs = (uniform(plain_word) >> kUnitPlainShift) >> 1; pairs > 0; --pairs) {
                         const uint64_t off_next = band_offset(issued + 1);  // (in the table: the second step of the pair is plain)
-                        plain_step(rel++, false, uniform_offset(off));
+                        const int row_next = band_row(issued + 1);
+                        plain_step(rel++, false, uniform_offset(off), uniform(row));
                         off = band_offset(min(issued + 1, n_units - 1));  // used if another pair follows
-                        plain_step(rel++, true, uniform_offset(off_next));
+                        row = band_row(min(issued + 1, n_units - 1));
+                        plain_step(rel++, true, uniform_offset(off_next), uniform(row_next));
                     }
                 }
                 first_step = false;

@@ -367,12 +367,17 @@ namespace dfx {
                                 "no vector instruction, the offsets are those of pipe_set_load_offsets."))
     parts.append(asm_fn("pipe_set_fresh_offsets", "uint32_t o0, uint32_t o1",
                         join(f"v_mov_b32 {vr(FRESH_OFF + j)}, %{j}" for j in range(2)), ins=['"v"(o0)', '"v"(o1)'],
-                        comment="Once per kernel (two-byte cache elements): the same offsets for a band of fresh rows, whose rows lie a\n"
-                                "token of k_new apart (and of v_new: only used where the two have one layout)."))
+                        comment="Once per kernel (two-byte cache elements): the same offsets for the K rows of a band of fresh rows,\n"
+                                "which lie a token of k_new apart."))
+    issue_fresh = []
+    for j in range(2):  # K rows with the offsets of pipe_set_fresh_offsets, V rows with those of pipe_set_load_offsets
+        issue_fresh += [f"s_add_u32 m0, %[d], {j * 1024}", f"global_load_lds_dwordx4 {vr(FRESH_OFF + j)}, %[kb] nt",
+                        f"s_add_u32 m0, %[d], {MAT_BYTES + j * 1024}", f"global_load_lds_dwordx4 {vr(LOAD_OFF + j)}, %[vb] nt"]
     parts.append(asm_fn("pipe_issue_band_fresh", "const void* k_rows, const void* v_rows, uint32_t lds_dst",
-                        join(issue).replace(vr(LOAD_OFF + 1), vr(FRESH_OFF + 1)).replace(vr(LOAD_OFF), vr(FRESH_OFF)),
+                        join(issue_fresh),
                         ins=['[kb] "s"(k_rows)', '[vb] "s"(v_rows)', '[d] "s"(lds_dst)'], clobbers=["memory", "m0", "scc"],
-                        comment="pipe_issue_band() for a full band of fresh rows (offsets of pipe_set_fresh_offsets)."))
+                        comment="pipe_issue_band() for a full band of fresh rows in a launch without a cache: the K rows lie a token of\n"
+                                "k_new apart (pipe_set_fresh_offsets), the V rows a token of v_new (pipe_set_load_offsets, free there)."))
     issue8 = [f"s_add_u32 m0, %[d], 0", f"global_load_lds_dwordx4 {vr(LOAD_OFF)}, %[kb] nt",
               f"s_add_u32 m0, %[d], {MAT_BYTES // 2}", f"global_load_lds_dwordx4 {vr(LOAD_OFF)}, %[vb] nt"]
     parts.append(asm_fn("pipe_issue_band_fp8", "const void* k_rows, const void* v_rows, uint32_t lds_dst", join(issue8),

@@ -158,8 +158,8 @@ int launch(const KArgs& ka, const Plan& plan, hipStream_t st, const PlanArgs* pa
                 if (plan.pipelined) {
                     main_k = paged_attn_pipe_kernel<NW>;
                     slot = kSlotBase + 2;
-                    // no cache, one layout for k_new and v_new: the variant whose plain steps fetch fresh rows
-                    if (ka.k_cache == nullptr && ka.v_fresh_delta == 0) {
+                    // no cache: the variant whose plain steps fetch fresh rows
+                    if (ka.k_cache == nullptr) {
                         main_k = paged_attn_pipe_kernel<NW, true>;
                         slot = 29;
                     }

@@ -712,6 +712,33 @@ def test_block_causal_prefill_without_a_cache(dev):
         assert max_abs_err(got, want) <= ATOL_BF16
 
 
+@pytest.mark.parametrize("mask", [MASK_FULL, MASK_BLOCK_CAUSAL])
+def test_prefill_with_v_sliced_out_of_the_projection(dev, mask):
+    """A prefill as a decoder layer issues it: K rotated into a buffer of its own, V still a column slice of the
+    fused QKV projection (another token stride, the same head stride).  Long enough for the plain steps of the
+    kernel variant without a cache; the same bits as with a contiguous V, within tolerance of the oracle."""
+    from oracle import attention as oat
+    B, L, hq, hkv, hd = 2, 1280, 14, 2, 128
+    g = torch.Generator().manual_seed(23)
+    q = torch.randn(B * L, hq, hd, generator=g).to(torch.bfloat16)
+    k = torch.randn(B * L, hkv, hd, generator=g).to(torch.bfloat16)
+    v = torch.randn(B * L, hkv, hd, generator=g).to(torch.bfloat16)
+    cu = torch.arange(0, B * L + 1, L, dtype=torch.int32)
+    want = oat.paged_attention_fp32(q, k, v, None, None, None, None, cu, cu, hd ** -0.5, mask_mode=mask, dbs=32)
+    qkv = torch.zeros(B * L, (hq + 2 * hkv) * hd, dtype=torch.bfloat16, device=dev)
+    v_view = qkv[:, (hq + hkv) * hd:].view(B * L, hkv, hd)
+    v_view.copy_(v)
+    assert v_view.stride(0) != k.stride(0) and v_view.stride(1) == k.stride(1)
+    kw = dict(block_tables=None, context_lens=None, cu_seqlens_q=cu.to(dev), cu_seqlens_new=cu.to(dev), max_seqlen_q=L,
+              mask_mode=mask, diffusion_block_size=32)
+    for max_wg in (0, 3):
+        ref = dfx.paged_attention(q.to(dev), k.to(dev), v.to(dev), None, None, hd ** -0.5, max_workgroups=max_wg, **kw)
+        got = dfx.paged_attention(q.to(dev), k.to(dev), v_view, None, None, hd ** -0.5, max_workgroups=max_wg, **kw)
+        torch.cuda.synchronize()
+        assert torch.equal(got, ref)
+        assert max_abs_err(got, want) <= ATOL_BF16
+
+
 # the shapes of the reference's prefill kernel tests (tests/python/kernel/test_dllm_flash_attn_prefill_kernel.py
 # :162-310): (sequences, query heads, KV heads, head_dim, length, block attention, diffusion block size)
 REF_PREFILL_CASES = [

@@ -537,7 +537,7 @@ def main():
     tflops = nflops / (ms * 1e-3) / 1e12
     traffic, traffic_source = measured_traffic(args.workload, nbytes)
     kernel = ("paged_attn_pipe_fp8_kernel<8>" if wl.kv_fp8 else
-              "paged_attn_pipe_kernel<8, false>" if args.workload == "c3" else "paged_attn_stream_kernel")
+              "paged_attn_pipe_kernel<8, false>")
     result = {
         "metric": "attn query-tokens/sec + achieved HBM GB/s (% of peak), Dream-7B shape, 1 GPU",
         "value": wl.total_q_tokens / (ms * 1e-3), "unit": "query-tokens/s",

@@ -73,12 +73,13 @@ int make_plan(const dfx_attn_params* p, Plan& plan) {
                   p->kn_stride_head == p->vn_stride_head;
     // head_dim 128, 65..128 rows: the 8-wave pipelined kernels (their waves without rows only fetch) are
     // faster than 4 waves with a compiler-scheduled step, with or without a second workgroup on the
-    // compute unit (C4 -7 %, 112 or 128 rows at the C3 shape -18 %).  33..64 rows: the same (-17 % at the
-    // C3 shape) while a workgroup has few items to open and close; with four short items each the two
-    // workgroups per compute unit are 22 % ahead, and a launch cannot see lengths.  32 rows: +7 %.
+    // compute unit (C4 -7 %, 112 or 128 rows at the C3 shape -18 %).  Fewer rows: the same (64 or 48 rows
+    // at the C3 shape -17 %, 32 rows -1 to -15 %) while a workgroup has few items to open and close; with
+    // four short items each the two workgroups per compute unit are ahead (64 rows: by 22 %, 32 rows: by
+    // 7 %), and a launch cannot see lengths.
     if (plan.stream && plan.hd == 128 && !(p->flags & DFX_ATTN_NO_PIPELINE)) {
         const int64_t items = static_cast<int64_t>(p->num_seqs) * p->num_kv_heads;
-        if (rows > 64 || (rows > 32 && items <= 2 * static_cast<int64_t>(device_cu_count()))) plan.nb = 2;
+        if (rows > 64 || items <= 2 * static_cast<int64_t>(device_cu_count())) plan.nb = 2;
     }
     plan.compact = plan.stream && !plan.fp8 && plan.nb == 1 && p->num_seqs <= kCompactMaxSeqs;
     // (8 waves only: with 4 waves a wave has twice the tile loads to address, and the 32 registers

@@ -91,7 +91,7 @@ def algorithmic_flops(wl) -> int:
     return 4 * wl.num_q_heads * wl.head_dim * pairs
 
 
-def cpu_baseline(name: str, budget_s: float = 15.0):
+def cpu_baseline(name: str, budget_s: float = 15.0, **override):
     """The reference's PyTorch path on the host cores, on a bounded batch slice."""
     from diffulex_amd.workloads import make_workload
     from oracle import attention as oat
@@ -100,7 +100,7 @@ def cpu_baseline(name: str, budget_s: float = 15.0):
     torch.set_num_threads(cores)
     from diffulex_amd.workloads import SPECS
     n_seqs = min(SPECS[name]["num_seqs"], 16 if name == "c5" else 64)
-    wl = make_workload(name, num_seqs=n_seqs)
+    wl = make_workload(name, num_seqs=n_seqs, **override)
 
     def run():
         return oat.paged_attention_sdpa(wl.q, wl.k_new, wl.v_new, wl.k_cache, wl.v_cache, wl.block_tables,
@@ -428,6 +428,75 @@ def bench_layer(args, dev):
     }))
 
 
+def bench_d2f_small(args, dev):
+    """Small D2F batches the way the reference's D2F runner issues them: eagerly (it captures no graph,
+    strategy/d2f/engine/model_runner.py:291-297), one ``Attention.forward`` per layer through the Python
+    operators (store of the blocks to cache, then the varlen decode), a new metadata object per decoding
+    step.  LLaDA-8B heads (the C4 shape), batches of 1, 4 and 8 sequences of three in-flight blocks.  GPU
+    time by events and the host's wall time to issue the calls are reported side by side: whichever is
+    larger is what a step costs."""
+    import diffulex_amd as dfx
+    from diffulex_amd.workloads import make_workload
+    layers_per_step = 32   # LLaDA-8B
+    rows = []
+    for b in (1, 4, 8):
+        wl = make_workload("c4", device=dev, num_seqs=b)
+        T, hq, hkv, hd = wl.q.shape[0], wl.num_q_heads, wl.num_kv_heads, wl.head_dim
+        n_sets = 4
+        layers = []
+        for _ in range(n_sets):
+            att = dfx.Attention(hq, hd, wl.scale, hkv)
+            att.k_cache, att.v_cache = wl.k_cache.clone(), wl.v_cache.clone()
+            layers.append((att, wl.q.reshape(T, -1).clone(), wl.k_new.reshape(T, -1).clone(), wl.v_new.reshape(T, -1).clone()))
+        state = {}
+
+        def new_decode_step():
+            state["md"] = dfx.PagedAttnMetaData(
+                is_prefill=False, cu_seqlens_q=wl.cu_seqlens_q, cu_seqlens_k=wl.cu_seqlens_k, max_seqlen_q=wl.q_len,
+                slot_mapping=wl.slot_mapping, context_lens=wl.context_lens, block_tables=wl.block_tables,
+                page_block_size=wl.page_size, diffusion_block_size=wl.diffusion_block_size, decode_mode="varlen",
+                need_kv_cache_store=True, seq_lens_ts=wl.seq_lens_new, decode_mask="block_causal")
+        dfx.set_fetch_fn_for_attn_metadata(lambda: state["md"])
+
+        def layer(i):
+            if i % layers_per_step == 0:
+                new_decode_step()
+            att, q, k, v = layers[i % n_sets]
+            return att(q, k, v)
+
+        with torch.inference_mode():   # as the reference's run_model
+            spin_up(layer)
+            for i in range(args.warmup):
+                layer(i)
+            steps = max(layers_per_step, args.steps // layers_per_step * layers_per_step)
+            ms, issue_ms = timed(layer, steps)
+        nbytes = algorithmic_bytes(wl) + 2 * T * hkv * hd * 2   # + the block stored into the cache
+        rows.append({"num_seqs": b, "gpu_ms_per_layer": ms, "host_wall_ms_per_layer": issue_ms,
+                     "bound": "host" if issue_ms > ms else "gpu", "algorithmic_bytes": nbytes,
+                     "gbs": nbytes / (max(ms, issue_ms) * 1e-3) / 1e9,
+                     "ctx": [int(c) for c in wl.context_lens.tolist()]})
+        del layers, wl
+        torch.cuda.empty_cache()
+    worst = rows[-1]
+    step_ms = max(worst["gpu_ms_per_layer"], worst["host_wall_ms_per_layer"])
+    print(json.dumps({
+        "metric": "eager D2F decode layer (KV store + paged attention through the Python operators), small batches, "
+                  "query-tokens/sec, 1 GPU",
+        "value": worst["num_seqs"] * 96 / (step_ms * 1e-3), "unit": "query-tokens/s", "n_gpus": 1, "steps": steps,
+        "warmup": args.warmup, "ms_per_step": step_ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "d2f-small: LLaDA-8B heads (32/32, head_dim 128), 3 in-flight 32-token blocks per sequence, "
+                               "block-causal, contexts in [1024, 4096], 256-token pages, batches of 1, 4 and 8; eager "
+                               "Attention.forward per layer under torch.inference_mode(), a new metadata object (and plan) "
+                               f"every {layers_per_step} layers; value and ms_per_step are the batch of 8, the larger of "
+                               "GPU time and host issue time",
+                   "batches": rows, "host_wall_ms_per_step": worst["host_wall_ms_per_layer"]},
+        "roofline": {"bound": "hbm", "achieved": worst["gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": worst["gbs"] / HBM_PEAK_GBS, "traffic": None, "algorithmic_bytes": worst["algorithmic_bytes"],
+                     "kernel": "paged_attn_pipe_kernel<8, false> (+ kv store), duration = max(GPU events, host issue) / layers"},
+    }))
+
+
 SPIN_UP_SECONDS = 0.25
 
 
@@ -451,7 +520,10 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=1000)
     ap.add_argument("--warmup", type=int, default=100)
-    ap.add_argument("--workload", default="c3", choices=["c3", "c4", "c5", "c1", "c2", "rope", "prefill", "layer", "store-distinct"])
+    ap.add_argument("--workload", default="c3", choices=["c3", "c4", "c5", "c1", "c2", "rope", "prefill", "layer", "store-distinct", "d2f-small"])
+    ap.add_argument("--page", type=int, default=0,
+                    help="tokens per KV-cache page for the attention workloads (default: the workload's 256; the "
+                         "reference's default kvcache_block_size is 32, diffulex/config.py:41)")
     ap.add_argument("--copies", type=int, default=4, help="independent KV-cache copies rotated between steps")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -493,7 +565,10 @@ def main():
     if args.workload == "store-distinct":
         bench_store_distinct(args, dev)
         return
-    wl = make_workload(args.workload, device=dev)
+    if args.workload == "d2f-small":
+        bench_d2f_small(args, dev)
+        return
+    wl = make_workload(args.workload, device=dev, **({"page": args.page} if args.page > 0 else {}))
     # every tensor a launch touches exists `copies` times; step i uses set i % copies
     sets = [(wl.q, wl.k_new, wl.v_new, torch.empty_like(wl.q), wl.k_cache, wl.v_cache)]
     for _ in range(args.copies - 1):
@@ -535,7 +610,7 @@ def main():
     nbytes, nflops = algorithmic_bytes(wl), algorithmic_flops(wl)
     gbs = nbytes / (ms * 1e-3) / 1e9
     tflops = nflops / (ms * 1e-3) / 1e12
-    traffic, traffic_source = measured_traffic(args.workload, nbytes)
+    traffic, traffic_source = measured_traffic(args.workload, nbytes) if args.page <= 0 else (None, None)
     kernel = ("paged_attn_pipe_fp8_kernel<8>" if wl.kv_fp8 else
               "paged_attn_pipe_kernel<8, false>")
     result = {
@@ -568,7 +643,7 @@ def main():
         },
     }
     if not args.no_cpu:
-        result["cpu_baseline"] = cpu_baseline(args.workload)
+        result["cpu_baseline"] = cpu_baseline(args.workload, **({"page": args.page} if args.page > 0 else {}))
     print(json.dumps(result))
 
 

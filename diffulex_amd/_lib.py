@@ -10,7 +10,7 @@ from pathlib import Path
 
 LIB_PATH = Path(__file__).resolve().parent / "libdiffulex_amd.so"
 
-DFX_ABI_VERSION = 6
+DFX_ABI_VERSION = 7
 DFX_OK = 0
 DFX_KV_BF16, DFX_KV_FP8_E4M3 = 0, 1
 DFX_MASK_FULL, DFX_MASK_BLOCK_CAUSAL = 0, 1
@@ -51,7 +51,7 @@ class AttnParams(C.Structure):
         ("max_workgroups", C.c_int32), ("flags", C.c_int32), ("scale", C.c_float),
         ("store_slot_mapping", C.c_void_p), ("store_slot_index_type", C.c_int32),
         ("plan", C.c_void_p), ("plan_bytes", C.c_int64), ("num_new_tokens", C.c_int64),
-        ("cache_layout", C.c_int32), ("reserved1", C.c_int32), ("kc_stride", C.c_int64 * 5), ("vc_stride", C.c_int64 * 4),
+        ("cache_layout", C.c_int32), ("num_q_tokens", C.c_int32), ("kc_stride", C.c_int64 * 5), ("vc_stride", C.c_int64 * 4),
     ]
 
 

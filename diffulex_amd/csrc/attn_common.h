@@ -46,6 +46,7 @@ struct KArgs {
     const void* store_slots;  // fused KV-cache store: slot per fresh row, or null
     int store_slots_i64;
     int64_t n_new;            // rows of k_new / v_new (and of the slot mapping)
+    int32_t n_q;              // rows of q / out: no row at or beyond it is read or written, whatever the offsets say
     int64_t v_fresh_delta;    // streaming paths: (token stride of v_new - token stride of k_new) in bytes
     const uint8_t* plan;      // launch plan built by the plan kernels, or null
     uint32_t plan_signature;  // of this launch's configuration: a plan made for another one is ignored
@@ -219,9 +220,10 @@ struct AttnState {
 #pragma unroll
         for (int qb = 0; qb < NB; ++qb) {
             const int r = row_of(rt, qb);
-            const bool valid = r < a.group * sh.q_len;
+            bool valid = r < a.group * sh.q_len;
             const int g = valid ? r / sh.q_len : 0;
             const int i = valid ? r - g * sh.q_len : 0;
+            valid = valid && i < a.n_q - q0;
             vis_limit[qb] = (i / a.dbs + 1) * a.dbs;
             const uint16_t* qp = a.q + (q0 + i) * a.q_st + (kvh * a.group + g) * a.q_sh + half * 8;
 #pragma unroll
@@ -332,9 +334,10 @@ struct AttnState {
 #pragma unroll
         for (int qb = 0; qb < NB; ++qb) {
             const int r = row_of(rt, qb);
-            const bool valid = r < a.group * sh.q_len;
+            bool valid = r < a.group * sh.q_len;
             const int g = valid ? r / sh.q_len : 0;
             const int i = valid ? r - g * sh.q_len : 0;
+            valid = valid && i < a.n_q - q0;  // (a plan made before the offsets were rewritten in place may say otherwise)
             // a row none of whose keys is visible (every page of its context a hole, no fresh rows)
             // has a zero sum: it gets zeros, not 0 * inf
             const float inv = l_tot[qb] > 0.0f ? out_mul / l_tot[qb] : 0.0f;

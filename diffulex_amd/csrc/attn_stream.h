@@ -448,8 +448,11 @@ struct StreamAttn : TileMath<HD, NB, NW, HIDDEN> {
         const bool valid = r < a.group * q_len;
         const int g = valid ? r / q_len : 0;
         const int i = valid ? r - g * q_len : 0;
-        // (lanes without a row read row 0 of the item: finite data whose results are never stored)
-        pipe_issue_queries(a.q + (uniform(d.q0) + i) * a.q_st + (uniform(d.kvh) * a.group + g) * a.q_sh + half * 8);
+        // (lanes without a row read row 0 of the item: finite data whose results are never stored; a row
+        // beyond the rows q has -- offsets rewritten in place after the plan was made -- reads row 0 of q)
+        int row = uniform(d.q0) + i;
+        row = row < a.n_q ? row : 0;
+        pipe_issue_queries(a.q + row * a.q_st + (uniform(d.kvh) * a.group + g) * a.q_sh + half * 8);
     }
     DFX_D void adopt_item(const UnitDesc& d) {
         this->s = uniform(d.s);

@@ -236,7 +236,7 @@ int check_args(const dfx_attn_params* p, Plan& plan, bool& empty) {
     if (has_cache && (!p->block_tables || p->page_size <= 0 || p->max_pages_per_seq < 0 || p->n_pages < 0))
         return DFX_ERR_INVALID_ARG;
     if (plan.fp8 && (!p->k_scale || !p->v_scale)) return DFX_ERR_INVALID_ARG;
-    if (p->num_new_tokens < 0) return DFX_ERR_INVALID_ARG;
+    if (p->num_new_tokens < 0 || p->num_q_tokens < 0) return DFX_ERR_INVALID_ARG;
     if (p->store_slot_mapping != nullptr) {
         if (!has_cache || p->num_new_tokens <= 0) return DFX_ERR_INVALID_ARG;  // the store needs the row count
         if (p->store_slot_index_type != DFX_INDEX_I32 && p->store_slot_index_type != DFX_INDEX_I64)
@@ -286,6 +286,7 @@ uint32_t plan_signature(const dfx_attn_params* p, const Plan& plan) {
     mix(p->cache_stride_head); mix(p->block_table_stride); mix(p->n_pages); mix(p->k_cache != nullptr);
     mix(reinterpret_cast<uintptr_t>(p->block_tables)); mix(reinterpret_cast<uintptr_t>(p->context_lens));
     mix(reinterpret_cast<uintptr_t>(p->cu_seqlens_q)); mix(reinterpret_cast<uintptr_t>(p->cu_seqlens_new));
+    mix(static_cast<uint32_t>(p->flags)); mix(plan.pipelined);
     const uint32_t sig = static_cast<uint32_t>(h ^ (h >> 32));
     return sig == 0 ? 1u : sig;
 }
@@ -379,6 +380,7 @@ int run_paged_attn(const dfx_attn_params* p, void* workspace, int64_t workspace_
     }
     ka.c = p->scale * kLog2e;
     ka.n_new = p->num_new_tokens > 0 ? p->num_new_tokens : INT64_MAX;
+    ka.n_q = p->num_q_tokens > 0 ? p->num_q_tokens : INT32_MAX;
     ka.v_fresh_delta = (p->vn_stride_token - p->kn_stride_token) * 2;
     ka.plan = nullptr;
     ka.plan_capacity = 0;

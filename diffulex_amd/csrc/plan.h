@@ -281,14 +281,15 @@ __global__ void __launch_bounds__(512) paged_attn_plan_kernel(const KArgs a, con
                 const uint64_t votes = __ballot(fits[tid] != 0);
                 const int best = votes != 0 ? __builtin_ctzll(votes) : 64;
                 if (tid == 0) {
-                    ubase[0] = best;
+                    // (kept in misc: the cut points written below reach into ubase[0] when n_active == 1024)
+                    misc[48] = best;
                     if (best < 64 && !keep) sweep_head(prefix, a.num_seqs, n_w, base2 + base2 * best / 100, iprefix, 1);
                 }
             }
             __syncthreads();
-            swept = ubase[0] < 64;
+            swept = misc[48] < 64;
             if (swept) {
-                const int best = ubase[0];
+                const int best = misc[48];
                 for (int k = tid; k <= n_active; k += blockDim.x) {
                     const int kvh = k / n_w, w = k - kvh * n_w;  // (k == n_active: the end of the last head)
                     bounds[k] = kvh * per_head + (w == 0 ? 0 : iprefix[keep ? (w - 1) * 64 + best : w - 1]);

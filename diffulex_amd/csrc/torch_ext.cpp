@@ -149,6 +149,7 @@ dfx_attn_params attn_params(DFX_ATTN_ARGS) {
     p.num_kv_heads = static_cast<int32_t>(h_kv);
     p.head_dim = static_cast<int32_t>(hd);
     p.num_new_tokens = k.size(0);
+    p.num_q_tokens = static_cast<int32_t>(q.size(0));
     p.max_seqlen_q = static_cast<int32_t>(max_seqlen_q);
     p.diffusion_block_size = static_cast<int32_t>(dbs);
     p.mask_mode = static_cast<int32_t>(mask_mode);

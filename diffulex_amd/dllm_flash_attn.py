@@ -74,7 +74,8 @@ def paged_attention(q, k, v, k_cache, v_cache, scale, *, block_tables, context_l
     the workgroups, page address of every tile) is built on the first call and reused by later
     calls with the same dict -- the attention layers of one decoding step, whose lengths and block
     tables are the same.  In-place updates of those tensors and graph captures are noticed (they
-    change the cache key); a caller that rewrites them behind PyTorch's back drops the dict.
+    change the cache key); a caller that rewrites them behind PyTorch's back, or rewrites tensors made
+    under ``torch.inference_mode()`` (which carry no version counter) in place, drops the dict.
     ``cache_layout="distinct"``: k_cache [pages, H_kv, hd / 8, page, 8], v_cache [pages, H_kv, hd,
     page] (what ``store_kvcache_distinct_layout`` writes); bf16, generic tile path, no fused store."""
     ops = _lib.ops()
@@ -104,12 +105,9 @@ def paged_attention(q, k, v, k_cache, v_cache, scale, *, block_tables, context_l
             store_slot_mapping)
     plan = None
     if plan_cache is not None and has_cache and not distinct:
-        # A plan is only as good as the lengths and tables it was made from: the key carries the
-        # tensors' version counters (any in-place update makes a new key) and the graph capture the
-        # call is recorded into (a plan built outside that capture is not part of its graph).
-        meta = (block_tables, context_lens, cu_seqlens_q, cu_seqlens_new)
-        key = (H_q, H_kv, hd, fp8, tail[1:], k.stride(0), k.stride(1), k_cache.stride()[:3], num_seqs,
-               tuple((t.data_ptr(), t._version) for t in meta), int(ops.stream_capture_id()))
+        # A plan is only as good as the lengths and tables it was made from: see plan_key().
+        key = plan_key(q, k, k_cache, fp8, tail, (block_tables, context_lens, cu_seqlens_q, cu_seqlens_new),
+                       int(ops.stream_capture_id()))
         plan = plan_cache.get(key, False)
         if plan is False:
             plan = plan_cache[key] = _build_plan(ops, head, tail, H_q // H_kv, int(max_seqlen_q), num_seqs,
@@ -118,7 +116,9 @@ def paged_attention(q, k, v, k_cache, v_cache, scale, *, block_tables, context_l
         if static_scratch:
             ops.paged_attention(*head, plan, *tail, None, True)
             return out
-        shape_key = (num_seqs, H_q, H_kv, hd, tail[1:], has_cache, fp8, k.stride() == v.stride(),
+        # (what dfx_paged_attn_workspace_bytes looks at: the shapes, the flags, whether k and v share
+        # their head stride -- which decides the tile path -- and the device's compute-unit count)
+        shape_key = (q.device.index, num_seqs, H_q, H_kv, hd, tail[1:], has_cache, fp8, k.stride(1) == v.stride(1),
                      k_cache.shape[1] if has_cache and not distinct else 0)
         need = _workspace_need.get(shape_key)
         if need is None:
@@ -130,6 +130,24 @@ def paged_attention(q, k, v, k_cache, v_cache, scale, *, block_tables, context_l
             raise _lib.DfxError(str(e).split("\n")[0]) from None
         raise
     return out
+
+
+def _content_token(t: torch.Tensor):
+    """What tells two states of a metadata tensor apart, as far as PyTorch can tell: its address and
+    its version counter, which every in-place update through PyTorch bumps.  Tensors created under
+    ``torch.inference_mode()`` (the reference's runners build their metadata there:
+    strategy/block_diffusion/engine/model_runner.py:206, strategy/d2f/engine/model_runner.py:291)
+    track no version and reading it raises; for them the address alone stands, and the plan lives as
+    long as the dict it is kept in -- the metadata object of one decoding step."""
+    return (t.data_ptr(), -1 if t.is_inference() else t._version)
+
+
+def plan_key(q, k, k_cache, fp8, tail, meta, capture_id):
+    """Cache key of a launch plan: everything ``dfx_paged_attn_plan`` depends on (shapes, strides, the
+    metadata tensors and their contents as far as ``_content_token`` sees them) and the graph capture
+    the call is recorded into (a plan built outside that capture is not part of its graph)."""
+    return (q.shape[1], k.shape[1], q.shape[2], bool(fp8), tail[1:], k.stride(0), k.stride(1), k_cache.stride()[:3],
+            meta[2].numel() - 1, tuple(_content_token(t) for t in meta), int(capture_id))
 
 
 def _build_plan(ops, head, tail, group, max_seqlen_q, num_seqs, max_pages, page_size, t_new):

@@ -19,7 +19,7 @@
 extern "C" {
 #endif
 
-#define DFX_ABI_VERSION 6
+#define DFX_ABI_VERSION 7
 
 typedef void* dfx_stream_t; /* a hipStream_t; NULL is the default stream */
 
@@ -209,13 +209,18 @@ typedef struct dfx_attn_params {
      * (diffulex/attention/attn_impl.py:66-69); here it runs on the generic tile path.  No fused store,
      * no FP8, no plan with it. */
     int32_t cache_layout;
-    int32_t reserved1;
+    /* Rows of q and out.  No row at or beyond it is read or written, whatever cu_seqlens_q (or a plan
+     * built from an earlier state of it) says.  0: unknown, the offsets are trusted. */
+    int32_t num_q_tokens;
     int64_t kc_stride[5];
     int64_t vc_stride[4];
 } dfx_attn_params;
 
-/* Bytes of scratch dfx_paged_attn needs for these shapes (depends on the sizes
- * and max_workgroups only, never on device data). Negative: dfx_status.
+/* Bytes of scratch dfx_paged_attn needs for these shapes.  It depends on the sizes (num_seqs, heads,
+ * head_dim, max_seqlen_q), on max_workgroups (0: the current device's compute-unit count, doubled
+ * for the small shapes that run two workgroups per compute unit), on flags, on kv_dtype and on
+ * whether k_new and v_new share their head stride (which selects the tile path) -- never on device
+ * data.  Negative: dfx_status.
  * The workspace starts with DFX_WORKSPACE_COUNTER_BYTES of arrival counters, which
  * the kernel expects to be zero and resets before it ends: zero-fill that area of a
  * new workspace once (hipMemsetAsync, or a fill kernel under graph capture).  Calls
@@ -237,7 +242,11 @@ int dfx_paged_attn(const dfx_attn_params* params, dfx_stream_t stream);
  * A plan depends on the lengths (context_lens, cu_seqlens_q, cu_seqlens_new), the block tables, the
  * shapes, max_workgroups, flags and the strides of the caches and of k_new -- not on the base
  * pointers of q, k_new, v_new, out and the caches, nor on scale: the per-layer views of one cache
- * allocation share a plan.  It is built on `stream` with no host synchronisation (safe to record
+ * allocation share a plan.  The kernels recognise a plan made for other shapes, strides, flags or
+ * metadata ADDRESSES and ignore it; they cannot see that the CONTENTS of the metadata arrays were
+ * rewritten in place since: after such an update the caller builds the plan again (a stale plan
+ * gives wrong rows, never an access outside the tensors as sized by n_pages, num_new_tokens and
+ * num_q_tokens).  It is built on `stream` with no host synchronisation (safe to record
  * into a graph).  With at least 8 units and at most two items per workgroup the plan places the cut
  * points between the workgroups' ranges of the unit space by cost rather than by unit count (whole
  * sequences where they fit, no pieces of a few tiles: a sweep with the smallest capacity per

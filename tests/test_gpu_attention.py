@@ -382,15 +382,71 @@ def test_result_bits_do_not_depend_on_which_piece_merges(dev):
 
 
 def test_full_size_c4_and_c5_on_sampled_sequences(dev):
-    for name, seqs, tol in (("c4", [0, 31], ATOL_BF16), ("c5", [3, 100], ATOL_FP8)):
+    """Full C4 and C5, without a plan and with the default plan (the launch bench.py times), each against
+    the oracle on sampled sequences."""
+    for name, seqs, tol in (("c4", [0, 13, 31], ATOL_BF16), ("c5", [3, 64, 100], ATOL_FP8)):
         wl = make_workload(name, device=dev)
-        out = _run(wl)
-        assert torch.isfinite(out.float()).all()
+        want = oracle_fp32(wl, seqs=seqs)
         cu = wl.cu_seqlens_q.tolist()
-        for s, w in zip(seqs, oracle_fp32(wl, seqs=seqs)):
-            assert max_abs_err(out[cu[s]:cu[s + 1]], w) <= tol
-        del wl, out
+        cache = {}
+        for kw in ({}, dict(plan_cache=cache), dict(plan_cache=cache)):
+            out = _run(wl, **kw)
+            assert torch.isfinite(out.float()).all()
+            for s, w in zip(seqs, want):
+                assert max_abs_err(out[cu[s]:cu[s + 1]], w) <= tol, (name, s, bool(kw))
+        assert len(cache) == 1 and next(iter(cache.values())) is not None
+        del wl, out, cache
         torch.cuda.empty_cache()
+
+
+def test_the_planned_launch_the_benchmark_times_against_the_oracle(dev):
+    """Full C3 with the default plan (cut points from the capacity sweep: plan mode 2), the launch the
+    headline figure is measured on: against the oracle on sampled sequences, and the same bits from
+    every launch that reads the plan."""
+    wl = make_workload("c3", device=dev)
+    cache = {}
+    got = _run(wl, plan_cache=cache)
+    plan = next(iter(cache.values()))
+    n_wg = torch.cuda.get_device_properties(dev).multi_processor_count
+    hdr, ranges, _ = _read_plan(plan, wl.num_seqs, n_wg)
+    assert hdr["magic"] == 0x44465850 and hdr["mode"] == 2 and hdr["n_active"] == n_wg
+    seqs = [0, 9, 17, 31, 44, 63]
+    cu = wl.cu_seqlens_q.tolist()
+    for s, want in zip(seqs, oracle_fp32(wl, seqs=seqs)):
+        assert max_abs_err(got[cu[s]:cu[s + 1]], want) <= ATOL_BF16, f"sequence {s}"
+    for _ in range(3):
+        assert torch.equal(_run(wl, plan_cache=cache), got)
+
+
+def test_decode_under_inference_mode_eager_and_captured(dev):
+    """The reference's runners build the step's metadata and run the model under
+    torch.inference_mode() (strategy/block_diffusion/engine/model_runner.py:206,
+    strategy/d2f/engine/model_runner.py:291): such tensors carry no version counter.  The plan cache
+    must work on them, eagerly and inside a capture."""
+    with torch.inference_mode():
+        wl = make_workload("c3", num_seqs=6, ctx=(300, 900), seed=43).to(dev)
+        assert wl.context_lens.is_inference()
+        att = dfx.Attention(wl.num_q_heads, wl.head_dim, wl.scale, wl.num_kv_heads)
+        att.k_cache, att.v_cache = wl.k_cache, wl.v_cache
+        md = metadata_for(wl, "static")
+        dfx.set_fetch_fn_for_attn_metadata(lambda: md)
+        t = wl.q.shape[0]
+        q, k, v = (x.reshape(t, -1).clone() for x in (wl.q, wl.k_new, wl.v_new))
+        want = oracle_fp32(wl)
+        eager = att(q, k, v)
+        again = att(q, k, v)          # the second layer of the step: same metadata object, same plan
+        torch.cuda.synchronize()
+        assert len(md.dfx_plan_cache) == 1
+        assert torch.equal(eager, again)
+        assert max_abs_err(eager.view(t, wl.num_q_heads, wl.head_dim), want) <= ATOL_BF16
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            o_static = att(q, k, v)
+        assert len(md.dfx_plan_cache) == 2   # a plan of its own inside the capture
+        for _ in range(2):
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(o_static, eager)
 
 
 def test_static_decode_in_a_captured_graph(dev):
@@ -885,6 +941,11 @@ def test_planned_launch_with_cut_points_placed_by_cost(dev, name, over, max_wg):
     tol = ATOL_FP8 if wl.kv_fp8 else ATOL_BF16
     if wl.num_seqs <= 16:
         assert max_abs_err(got, oracle_fp32(wl)) <= tol
+    else:   # the oracle on a sample: first, last and two sequences in between
+        seqs = sorted({0, wl.num_seqs // 3, 2 * wl.num_seqs // 3, wl.num_seqs - 1})
+        cu = wl.cu_seqlens_q.tolist()
+        for s, want in zip(seqs, oracle_fp32(wl, seqs=seqs)):
+            assert max_abs_err(got[cu[s]:cu[s + 1]], want) <= tol, f"sequence {s}"
     assert max_abs_err(got, _run(wl, max_wg)) <= 1e-2
     assert torch.equal(_run(wl, max_wg, plan_cache=cache), got)
     plan = next(iter(cache.values()))
@@ -941,6 +1002,54 @@ def test_pairing_plan_covers_every_unit_once_at_c3(dev):
     cu = wl.cu_seqlens_q.tolist()
     for s, want in zip([0, 63], oracle_fp32(wl, seqs=[0, 63])):
         assert max_abs_err(got[cu[s]:cu[s + 1]], want) <= ATOL_BF16
+
+
+def test_plan_with_1024_workgroups(dev):
+    """The largest grid the plan places cut points for: its table of 1025 cut points fills the
+    plan kernel's array to the last word."""
+    wl = make_workload("c3", device=dev, num_seqs=128, ctx=(2048, 8192), seed=12)
+    cache = {}
+    got = _run(wl, 1024, plan_cache=cache)
+    hdr, ranges, _ = _read_plan(next(iter(cache.values())), wl.num_seqs, 1024)
+    assert hdr["magic"] == 0x44465850 and hdr["mode"] == 2 and hdr["n_active"] == 1024
+    spans = [(int(r[0]), int(r[1])) for r in ranges]
+    assert spans[0][0] == 0 and spans[-1][1] == hdr["total"]
+    assert all(x[1] == y[0] for x, y in zip(spans, spans[1:])) and all(b >= a for a, b in spans)
+    assert [a for a, _ in spans] + [hdr["total"]] == hdr["bounds"][:1025].tolist()
+    assert torch.equal(_run(wl, 1024, plan_cache=cache), got)
+    seqs = [0, 77, 127]
+    cu = wl.cu_seqlens_q.tolist()
+    for s, want in zip(seqs, oracle_fp32(wl, seqs=seqs)):
+        assert max_abs_err(got[cu[s]:cu[s + 1]], want) <= ATOL_BF16
+
+
+def test_stale_plan_after_offsets_shrank_in_place_stays_inside_the_tensors(dev):
+    """A C-ABI caller that rewrites cu_seqlens in place and reuses the plan gets wrong rows (its
+    contract), but nothing outside q / out is touched: rows the plan names beyond num_q_tokens are
+    neither read nor written."""
+    wl = make_workload("c3", device=dev, num_seqs=6, ctx=(300, 900), seed=5)
+    cache = {}
+    _run(wl, plan_cache=cache)
+    plan = next(iter(cache.values()))
+    t_small = 4 * wl.q_len                                   # the batch shrinks to 4 sequences' rows ...
+    cu_small = wl.cu_seqlens_q.clone()
+    cu_small[5:] = t_small                                   # ... in a tensor of the same size (the last two have none)
+    wl.cu_seqlens_q.copy_(cu_small)                          # in place: same address, the plan's signature still matches
+    guard = torch.full((wl.q.shape[0], wl.num_q_heads, wl.head_dim), 7.0, dtype=torch.bfloat16, device=dev)
+    out = guard[:t_small]
+    key = next(iter(cache))
+    stale = {key: plan}
+    import diffulex_amd.dllm_flash_attn as dfa
+    orig = dfa.plan_key
+    dfa.plan_key = lambda *a, **k: key                       # (what a caller that bypasses PyTorch's version counters sees)
+    try:
+        dfx.paged_attention(wl.q[:t_small], wl.k_new, wl.v_new, wl.k_cache, wl.v_cache, wl.scale, out=out,
+                            block_tables=wl.block_tables, context_lens=wl.context_lens, cu_seqlens_q=wl.cu_seqlens_q,
+                            cu_seqlens_new=wl.cu_seqlens_q, max_seqlen_q=wl.q_len, plan_cache=stale)
+        torch.cuda.synchronize()
+    finally:
+        dfa.plan_key = orig
+    assert bool((guard[t_small:] == 7.0).all()), "rows beyond num_q_tokens were written"
 
 
 def test_plan_made_for_another_configuration_is_ignored(dev):

@@ -467,3 +467,32 @@ def test_owners_of_a_cut_item_from_a_table_of_cut_points(seed):
             lib.hook_owners_with_bounds(bounds.ctypes.data, n_w, me, first, last, C.byref(wa), C.byref(wb))
             assert (wa.value, wb.value) == (owners[0], owners[-1]), (i, me, owners)
 
+
+
+def test_plan_cache_key_works_on_inference_tensors_and_sees_in_place_updates():
+    """The reference's runners create the step's metadata under torch.inference_mode()
+    (strategy/block_diffusion/engine/model_runner.py:206, strategy/d2f/engine/model_runner.py:291);
+    such tensors have no version counter and asking for it raises.  The key must not."""
+    from diffulex_amd.dllm_flash_attn import plan_key, _content_token
+    q = torch.zeros(64, 28, 128, dtype=torch.bfloat16)
+    k = torch.zeros(64, 4, 128, dtype=torch.bfloat16)
+    kc = torch.zeros(4, 256, 4, 128, dtype=torch.bfloat16)
+    tail = (0.1, 32, 0, 32, 0, 0, 0)
+
+    def meta():
+        return (torch.zeros(2, 8, dtype=torch.int32), torch.zeros(2, dtype=torch.int32),
+                torch.zeros(3, dtype=torch.int32), torch.zeros(3, dtype=torch.int32))
+    with torch.inference_mode():
+        m = meta()
+        assert all(t.is_inference() for t in m)
+        with pytest.raises(RuntimeError):
+            m[0]._version
+        key = plan_key(q, k, kc, False, tail, m, 0)
+        assert key == plan_key(q, k, kc, False, tail, m, 0)          # the layers of one step share the plan
+        assert key != plan_key(q, k, kc, False, tail, m, 5)          # a capture gets a plan of its own
+        assert key != plan_key(q, k, kc, False, tail, meta(), 0)     # the next step's tensors
+        assert _content_token(m[1]) == (m[1].data_ptr(), -1)
+    m = meta()
+    key = plan_key(q, k, kc, False, tail, m, 0)
+    m[1].add_(1)   # ordinary tensors: an in-place update makes a new key
+    assert key != plan_key(q, k, kc, False, tail, m, 0)

@@ -19,6 +19,7 @@ DFX_ATTN_GENERIC_PATH = 1
 DFX_ATTN_NO_PIPELINE = 2
 DFX_ATTN_PAIRING = 4
 DFX_ATTN_EQUAL_RANGES = 8
+DFX_ATTN_BATCH_ORDER = 16
 DFX_ERR_SCRATCH_LIMIT = -5
 DFX_STATIC_SCRATCH_BYTES = 40 << 20
 DFX_WORKSPACE_COUNTER_BYTES = 1 << 18

@@ -56,7 +56,8 @@ struct PlanHeader {
     int32_t total_units;
     int32_t capacity;    // unit descriptors the buffer has room for
     int32_t critical;    // pairing: the critical length M (tiles), for diagnostics
-    int32_t pad[8];
+    int32_t reordered;   // 1: the unit space lists the sequences in the order of the plan's order table
+    int32_t pad[7];
 };
 static_assert(sizeof(PlanHeader) == 64, "header is one 64-byte line");
 
@@ -72,14 +73,15 @@ struct WgWork {
 static_assert(sizeof(WgWork) == 64, "four 16-byte words");
 
 struct PlanLayout {
-    int64_t prefix_off, bounds_off, work_off, units_off, bands_off, bytes;
+    int64_t prefix_off, bounds_off, work_off, order_off, units_off, bands_off, bytes;
 };
 DFX_HD PlanLayout plan_layout(int num_seqs, int n_wg, int64_t capacity, int waves) {
     PlanLayout l;
     l.prefix_off = sizeof(PlanHeader);
     l.bounds_off = (l.prefix_off + (static_cast<int64_t>(num_seqs) + 1) * 4 + 63) / 64 * 64;
     l.work_off = (l.bounds_off + (static_cast<int64_t>(n_wg) + 1) * 4 + 63) / 64 * 64;
-    l.units_off = (l.work_off + static_cast<int64_t>(n_wg) * sizeof(WgWork) + 63) / 64 * 64;
+    l.order_off = (l.work_off + static_cast<int64_t>(n_wg) * sizeof(WgWork) + 63) / 64 * 64;
+    l.units_off = (l.order_off + static_cast<int64_t>(num_seqs) * 4 + 63) / 64 * 64;
     l.bands_off = l.units_off + capacity * static_cast<int64_t>(sizeof(UnitDesc));
     l.bytes = l.bands_off + capacity * waves * static_cast<int64_t>(sizeof(BandDesc));
     return l;
@@ -177,6 +179,9 @@ struct StreamAttn : TileMath<HD, NB, NW, HIDDEN> {
     int64_t begin, end;
     int64_t rel_base;  // what UnitDesc::item_rel is relative to: the first unit of the workgroup's work
     int per_head;
+    // plan kernels only: the sequence at every position of the unit space (prefix[] is over positions), or
+    // null where the sequences follow each other in their own order
+    const int32_t* order = nullptr;
     float k_mul, v_inv;  // FP8: the current item's K scale and the reciprocal of its V scale
 
     DFX_D StreamAttn(const KArgs& args, uint8_t* smem)
@@ -203,15 +208,15 @@ struct StreamAttn : TileMath<HD, NB, NW, HIDDEN> {
             const int slot_in_ring = idx / NW;
             const int kv_head = static_cast<int>(pos / per_head);
             const int rem = static_cast<int>(pos - static_cast<int64_t>(kv_head) * per_head);
-            int lo = 0, hi = a.num_seqs;  // the sequence with prefix[s] <= rem < prefix[s + 1]
+            int lo = 0, hi = a.num_seqs;  // the position with prefix[p] <= rem < prefix[p + 1]
             while (lo < hi) {
                 const int mid = (lo + hi) >> 1;
                 if (prefix[mid + 1] <= rem) lo = mid + 1;
                 else hi = mid;
             }
-            const int sq = lo;
+            const int sq = order != nullptr ? order[lo] : lo;
             const SeqShape shp = load_seq_shape(a, sq, C::RT);
-            const int u = rem - prefix[sq];
+            const int u = rem - prefix[lo];
             int rt, tile, item_tiles;
             locate_unit(shp, u, rt, tile, item_tiles);
             const bool is_ctx = tile < shp.n_ctx_tiles;

@@ -130,6 +130,7 @@ int launch(const KArgs& ka, const Plan& plan, hipStream_t st, const PlanArgs* pa
     void (*plan_k)(const KArgs, const PlanArgs) = nullptr;
     void (*fill_k)(const KArgs, const PlanArgs) = nullptr;
     int lds, threads = kThreads, fill_lds = 0, slot;
+    int plan_slot = 30;  // (the plan kernel exists for row tiles of 128 and of 256 rows)
     constexpr int NW = 4 * NB;  // streaming paths: one 32-row query block per wave
     constexpr int kSlotBase = (HD == 128 ? 0 : 8) + (NB == 1 ? 0 : 4);
     if constexpr (PATH == 3) {
@@ -139,6 +140,7 @@ int launch(const KArgs& ka, const Plan& plan, hipStream_t st, const PlanArgs* pa
         using C = StreamCfg<HD, FNB, FNW, false, 1>;
         lds = C::LDS_BYTES;
         plan_k = paged_attn_plan_kernel<C::RT>;
+            plan_slot = C::RT == 256 ? 31 : 30;
         fill_k = paged_attn_plan_fill_kernel<HD, FNB, FNW, false, 1>;
         fill_lds = C::STAGES_OFF;
         threads = 64 * FNW;
@@ -157,6 +159,7 @@ int launch(const KArgs& ka, const Plan& plan, hipStream_t st, const PlanArgs* pa
             main_k = paged_attn_stream_kernel<HD, 1, 4, true>;
             lds = C::LDS_BYTES;
             plan_k = paged_attn_plan_kernel<C::RT>;
+            plan_slot = C::RT == 256 ? 31 : 30;
             fill_k = paged_attn_plan_fill_kernel<HD, 1, 4, true, 2>;
             fill_lds = C::STAGES_OFF;
             slot = kSlotBase + 1;
@@ -177,6 +180,7 @@ int launch(const KArgs& ka, const Plan& plan, hipStream_t st, const PlanArgs* pa
             }
             lds = C::LDS_BYTES;
             plan_k = paged_attn_plan_kernel<C::RT>;
+            plan_slot = C::RT == 256 ? 31 : 30;
             fill_k = paged_attn_plan_fill_kernel<HD, 1, NW, false, 2>;
             fill_lds = C::STAGES_OFF;
         }
@@ -192,8 +196,8 @@ int launch(const KArgs& ka, const Plan& plan, hipStream_t st, const PlanArgs* pa
     }
     if (pa != nullptr) {
         if (plan_k == nullptr) return DFX_ERR_UNSUPPORTED;
-        constexpr int kPlanLds = (2 * (kMaxSeqs + 1) + 2 * kMaxPairItems + 64) * 4;
-        hipLaunchKernelGGL(plan_k, dim3(1), dim3(512), kPlanLds, st, ka, *pa);
+        if (!ensure_lds_limit(reinterpret_cast<const void*>(plan_k), plan_slot, kPlanKernelLdsBytes)) return DFX_ERR_LAUNCH;
+        hipLaunchKernelGGL(plan_k, dim3(1), dim3(512), kPlanKernelLdsBytes, st, ka, *pa);
         hipLaunchKernelGGL(fill_k, dim3(plan.n_wg), dim3(threads), fill_lds, st, ka, *pa);
         return hipGetLastError() == hipSuccess ? DFX_OK : DFX_ERR_LAUNCH;
     }
@@ -326,6 +330,7 @@ int run_paged_attn(const dfx_attn_params* p, void* workspace, int64_t workspace_
         pa.signature = plan_signature(p, plan);
         pa.allow_pairing = (p->flags & DFX_ATTN_PAIRING) ? 1 : 0;
         pa.equal_ranges = (p->flags & DFX_ATTN_EQUAL_RANGES) ? 1 : 0;
+        pa.batch_order = (p->flags & DFX_ATTN_BATCH_ORDER) ? 1 : 0;
     }
 
     KArgs ka;

@@ -9,6 +9,8 @@
 //   WgWork work[n_wg]                           what every workgroup does (partition.h: linear ranges
 //                                               of the unit space, or the pairing partition), and the
 //                                               item of its first unit
+//   int32 order[num_seqs]                       header.reordered: the sequence at every position of the
+//                                               unit space (prefix[] then runs over positions)
 //   UnitDesc units[capacity]                    one per unit, in each workgroup's processing order
 //   BandDesc bands[capacity * NW]               one per unit and wave
 // Two kernels fill it: paged_attn_plan_kernel (one workgroup: prefix, partition) and
@@ -29,6 +31,7 @@ struct PlanArgs {
     uint32_t signature;
     int allow_pairing;
     int equal_ranges;   // cut the unit space into equal ranges, as the attention kernels do without a plan
+    int batch_order;    // keep the sequences in the batch's order in the unit space
 };
 
 // Where the plan cuts the linear unit space (mode 2): ranges of equal COST, a unit costing 2 and
@@ -47,6 +50,12 @@ constexpr int kPlanSeqCost = 8;
 constexpr int kPlanSnap = 4;
 constexpr int kPlanMaxItemsPerWg = 2;
 constexpr int kPlanMinUnitsPerWg = 8;  // below this the ranges stay equal
+// LDS of paged_attn_plan_kernel, in ints: unit prefix and item prefix over the sequences, the sort keys
+// and unit bases of the pairing partition (the cut points of the other partitions), scratch, then the
+// unit prefix over the positions of the second order of the sequences, that order, and the cut points the
+// sweep's candidates leave behind.
+constexpr int kPlanCutsRoom = 8192;
+constexpr int kPlanKernelLdsBytes = (2 * (kMaxSeqs + 1) + 2 * kMaxPairItems + 64 + (kMaxPairItems + 64) + kMaxPairItems + kPlanCutsRoom) * 4;
 
 // Linear position of item y (0 <= y < items of the sequence) inside the sequence's units, and its tiles.
 DFX_HD void item_of_sequence(const SeqShape& sh, int rt, int& offset, int& tiles) {
@@ -87,6 +96,9 @@ __global__ void __launch_bounds__(512) paged_attn_plan_kernel(const KArgs a, con
     uint32_t* keys = reinterpret_cast<uint32_t*>(iprefix + kMaxSeqs + 1);  // [kMaxPairItems]
     int* ubase = reinterpret_cast<int*>(keys + kMaxPairItems);          // [kMaxPairItems]
     int* misc = ubase + kMaxPairItems;                                  // [64]
+    int* pprefix = misc + 64;                                           // [kMaxPairItems + 64]
+    int* order2 = pprefix + kMaxPairItems + 64;                         // [kMaxPairItems]
+    int* cuts = order2 + kMaxPairItems;                                 // [kPlanCutsRoom]
     PlanHeader* hdr = reinterpret_cast<PlanHeader*>(pa.buf);
     const PlanLayout lay = plan_layout(a.num_seqs, pa.n_wg, pa.capacity, pa.waves);
     int* g_prefix = reinterpret_cast<int*>(pa.buf + lay.prefix_off);
@@ -100,7 +112,6 @@ __global__ void __launch_bounds__(512) paged_attn_plan_kernel(const KArgs a, con
     const int n_active = total == 0 ? 0
                          : a.fixed_wg ? a.n_wg
                                       : effective_workgroups(total, n_items, summary.max_tiles, a.n_wg);
-    for (int s = tid; s <= a.num_seqs; s += blockDim.x) g_prefix[s] = prefix[s];
 
     // items before each sequence (row tiles of sequences that have units)
     {
@@ -143,6 +154,7 @@ __global__ void __launch_bounds__(512) paged_attn_plan_kernel(const KArgs a, con
     const int m = n_active;
     bool pairing = pa.allow_pairing && total > 0 && n_items <= m && m <= kMaxPairItems && total >= m;
     bool placed = false;  // cut points placed by cost (mode 2)
+    bool reordered = false;  // the sweep found the second order of the sequences better
     int critical = 0;
     if (pairing) {  // (uniform: every thread takes the same branch)
         int n_sort = 1;
@@ -250,7 +262,17 @@ __global__ void __launch_bounds__(512) paged_attn_plan_kernel(const KArgs a, con
                  n_items <= static_cast<int64_t>(kPlanMaxItemsPerWg) * n_active && total < (1ll << 30);
         // the sweep, where the workgroups divide evenly among the KV heads (whose sequences are the same):
         // 64 capacities, from the mean load (no cuts) upwards in steps of 1 %, one per lane; the smallest
-        // that succeeds is swept once more for its cut points, which every KV head then uses
+        // that succeeds gives the cut points, which every KV head then uses.
+        //
+        // The sweep takes the sequences in the order they have in the unit space, and what it can do
+        // depends on that order: a long sequence must be cut, and what is left of it fills a workgroup
+        // only together with a short neighbour.  So the unit space may list the sequences in another
+        // order than the batch does (the attention kernels never see the difference: their descriptors
+        // name the sequence).  A second order is swept next to the batch's own -- the k-th longest
+        // sequence followed by the k-th shortest, whose units add up to about two workgroups' shares: one
+        // cut per pair at most -- and the order whose smallest capacity is lower is taken (measured at 64
+        // sequences x 4 KV heads of 8-32 tiles on 256 workgroups: 27 cut items per head and the last
+        // workgroup done after 58 us in the batch's order, 16 and 54 in the second).
         bool swept = false;
         const int n_w = a.h_kv > 0 ? n_active / a.h_kv : 0;
         if (placed && blockDim.x == 512 && n_w >= 2 && n_w * a.h_kv == n_active && n_w <= 1023) {  // (uniform)
@@ -263,36 +285,74 @@ __global__ void __launch_bounds__(512) paged_attn_plan_kernel(const KArgs a, con
             nonempty = 0;
             for (int w = 0; w < static_cast<int>(blockDim.x >> 6); ++w) nonempty += misc[40 + w];
             const int base2 = (2 * per_head + kSweepWhole * nonempty + n_w - 1) / n_w;
+            const bool two = !pa.batch_order && a.num_seqs >= 3 && a.num_seqs <= kMaxPairItems && per_head < (1 << 20);
+            if (two) {  // (uniform)
+                int n_sort = 1;
+                while (n_sort < a.num_seqs) n_sort <<= 1;
+                for (int x = tid; x < n_sort; x += blockDim.x)  // (a key of 0 sorts behind every sequence)
+                    keys[x] = x < a.num_seqs ? (static_cast<uint32_t>(prefix[x + 1] - prefix[x]) << 11) | static_cast<uint32_t>(kMaxPairItems - x) : 0u;
+                __syncthreads();
+                bitonic_sort_desc(keys, n_sort);
+                for (int p = tid; p < a.num_seqs; p += blockDim.x) {
+                    const int k = p >> 1;
+                    const int e = (p & 1) ? a.num_seqs - 1 - k : k;  // even positions: the longest ones, odd positions: the shortest
+                    order2[p] = kMaxPairItems - static_cast<int>(keys[e] & 2047u);
+                }
+                __syncthreads();
+                int carry = 0;
+                for (int base = 0; base < a.num_seqs; base += blockDim.x) {
+                    const int p = base + tid;
+                    int u = 0;
+                    if (p < a.num_seqs) u = prefix[order2[p] + 1] - prefix[order2[p]];
+                    int tot;
+                    const int incl = block_inclusive_scan(u, misc, tot);
+                    if (p < a.num_seqs) pprefix[p + 1] = carry + incl;
+                    carry += tot;
+                }
+                if (tid == 0) pprefix[0] = 0;
+                __syncthreads();
+            }
             // every lane keeps the n_w - 1 inner cut points of its capacity (lane-minor, so that the lanes'
-            // stores do not collide) as long as 64 x (n_w - 1) numbers fit; otherwise the best capacity is swept again
-            const bool keep = 64 * (n_w - 1) <= kMaxSeqs + 1;
-            // (8 capacities per wave: lanes of one wave that walk at different speeds wait for each other;
-            // the kernel runs with 8 waves, and every one of the 64 flags is written)
-            int* fits = ubase + 64;  // [64]
+            // stores do not collide) as long as they fit; otherwise the best capacity is swept again
+            const int n_cand = two ? 128 : 64;
+            const bool keep = n_cand * (n_w - 1) <= kPlanCutsRoom;
+            // (8 capacities per wave and order: lanes of one wave that walk at different speeds wait for each
+            // other; the kernel runs with 8 waves, the second order's candidates in waves 4 to 7; every flag
+            // is written)
+            int* fits = ubase + 64;  // [128]
             {
-                const int cand = (tid >> 6) * 8 + (tid & 63);
-                if ((tid & 63) < 8 && cand < 64) {
-                    const bool ok = sweep_head(prefix, a.num_seqs, n_w, base2 + base2 * cand / 100, keep ? iprefix + cand : nullptr, 64);
+                const int per_wave = n_cand / 8;
+                const int cand = (tid >> 6) * per_wave + (tid & 63);
+                if ((tid & 63) < per_wave) {
+                    const int step = cand & 63;
+                    const bool ok = sweep_head((cand >> 6) ? pprefix : prefix, a.num_seqs, n_w, base2 + base2 * step / 100,
+                                               keep ? cuts + cand : nullptr, n_cand);
                     fits[cand] = ok ? 1 : 0;
                 }
             }
             __syncthreads();
             if (tid < 64) {
-                const uint64_t votes = __ballot(fits[tid] != 0);
-                const int best = votes != 0 ? __builtin_ctzll(votes) : 64;
+                const uint64_t votes0 = __ballot(fits[tid] != 0);
+                const uint64_t votes1 = __ballot(two && fits[64 + tid] != 0);
+                const int best0 = votes0 != 0 ? __builtin_ctzll(votes0) : 64;
+                const int best1 = votes1 != 0 ? __builtin_ctzll(votes1) : 64;
                 if (tid == 0) {
                     // (kept in misc: the cut points written below reach into ubase[0] when n_active == 1024)
+                    const bool second = best1 < best0;
+                    const int best = second ? best1 : best0;
                     misc[48] = best;
-                    if (best < 64 && !keep) sweep_head(prefix, a.num_seqs, n_w, base2 + base2 * best / 100, iprefix, 1);
+                    misc[49] = second ? 1 : 0;
+                    if (best < 64 && !keep) sweep_head(second ? pprefix : prefix, a.num_seqs, n_w, base2 + base2 * best / 100, cuts, 1);
                 }
             }
             __syncthreads();
             swept = misc[48] < 64;
+            reordered = swept && misc[49] != 0;
             if (swept) {
-                const int best = misc[48];
+                const int cand = misc[48] + (reordered ? 64 : 0);
                 for (int k = tid; k <= n_active; k += blockDim.x) {
                     const int kvh = k / n_w, w = k - kvh * n_w;  // (k == n_active: the end of the last head)
-                    bounds[k] = kvh * per_head + (w == 0 ? 0 : iprefix[keep ? (w - 1) * 64 + best : w - 1]);
+                    bounds[k] = kvh * per_head + (w == 0 ? 0 : cuts[keep ? (w - 1) * n_cand + cand : w - 1]);
                 }
             }
             __syncthreads();
@@ -343,6 +403,7 @@ __global__ void __launch_bounds__(512) paged_attn_plan_kernel(const KArgs a, con
             __syncthreads();
             placed = misc[32] == 0;
         }
+        reordered = reordered && placed;
         for (int k = tid; k < pa.n_wg; k += blockDim.x) {
             WgWork w;
             w.a0 = w.a1 = w.b0 = w.b1 = 0;
@@ -360,6 +421,12 @@ __global__ void __launch_bounds__(512) paged_attn_plan_kernel(const KArgs a, con
         if (placed)
             for (int k = tid; k <= n_active; k += blockDim.x) g_bounds[k] = bounds[k];
     }
+    // the unit prefix over the positions of the unit space, and who is where
+    {
+        int32_t* g_order = reinterpret_cast<int32_t*>(pa.buf + lay.order_off);
+        for (int s = tid; s <= a.num_seqs; s += blockDim.x) g_prefix[s] = reordered ? pprefix[s] : prefix[s];
+        for (int s = tid; s < a.num_seqs; s += blockDim.x) g_order[s] = reordered ? order2[s] : s;
+    }
     if (tid == 0) {
         PlanHeader h;
         h.magic = total <= pa.capacity ? kPlanMagic : 0u;  // too small a buffer: the kernels plan for themselves
@@ -370,7 +437,8 @@ __global__ void __launch_bounds__(512) paged_attn_plan_kernel(const KArgs a, con
         h.total_units = static_cast<int32_t>(total);
         h.capacity = static_cast<int32_t>(pa.capacity);
         h.critical = critical;
-        for (int i = 0; i < 8; ++i) h.pad[i] = 0;
+        h.reordered = reordered ? 1 : 0;
+        for (int i = 0; i < 7; ++i) h.pad[i] = 0;
         *hdr = h;
     }
 }
@@ -390,6 +458,7 @@ __global__ void __launch_bounds__(64 * NW) paged_attn_plan_fill_kernel(const KAr
     BandDesc* g_bands = reinterpret_cast<BandDesc*>(pa.buf + lay.bands_off);
     for (int s = threadIdx.x; s <= a.num_seqs; s += blockDim.x) at.prefix[s] = g_prefix[s];
     at.per_head = hdr->per_head;
+    if (hdr->reordered) at.order = reinterpret_cast<const int32_t*>(pa.buf + lay.order_off);
     __syncthreads();
     int64_t done = w.ubase;
     at.rel_base = w.a0;

@@ -52,6 +52,8 @@ typedef enum dfx_index_type { DFX_INDEX_I32 = 0, DFX_INDEX_I64 = 1 } dfx_index_t
 #define DFX_ATTN_PAIRING 4      /* dfx_paged_attn_plan: the pairing partition where it applies (see there) */
 #define DFX_ATTN_EQUAL_RANGES 8 /* dfx_paged_attn_plan: equal ranges of the unit space, as a launch without a plan cuts
                                    them (the plan's own cut points are placed by cost; see there) */
+#define DFX_ATTN_BATCH_ORDER 16 /* dfx_paged_attn_plan: keep the sequences in the batch's order when the work is dealt
+                                   to the workgroups (by default the plan may deal them in another order; see there) */
 
 /* ABI version of the loaded library (== DFX_ABI_VERSION it was built with). */
 int dfx_abi_version(void);
@@ -251,7 +253,8 @@ int dfx_paged_attn(const dfx_attn_params* params, dfx_stream_t stream);
  * points between the workgroups' ranges of the unit space by cost rather than by unit count (whole
  * sequences where they fit, no pieces of a few tiles: a sweep with the smallest capacity per
  * workgroup that works, which makes the plan kernel take about 30 us -- a plan is worth building
- * for several launches, not for one);
+ * for several launches, not for one; the sweep runs over the sequences in the batch's order and with
+ * the k-th longest followed by the k-th shortest, and keeps whichever order needs the smaller capacity);
  * DFX_ATTN_EQUAL_RANGES in flags keeps the equal ranges a launch without a plan uses (the results of
  * the two differ in the last bits: other pieces are merged).  DFX_ATTN_PAIRING in flags asks for the pairing partition where there are at most
  * as many (sequence, KV head, row tile) items as workgroups: every item gets a home workgroup and

@@ -72,8 +72,13 @@ struct WgWork {
 };
 static_assert(sizeof(WgWork) == 64, "four 16-byte words");
 
+// Band descriptors of the first kPlanFirst units of every workgroup, a second time and by themselves:
+// a workgroup reads those of its own waves with its plan entry, in one trip to memory, and starts its
+// first tile loads from them while the descriptor tables are still on their way.
+constexpr int kPlanFirst = 4;
+
 struct PlanLayout {
-    int64_t prefix_off, bounds_off, work_off, order_off, units_off, bands_off, bytes;
+    int64_t prefix_off, bounds_off, work_off, order_off, first_off, units_off, bands_off, bytes;
 };
 DFX_HD PlanLayout plan_layout(int num_seqs, int n_wg, int64_t capacity, int waves) {
     PlanLayout l;
@@ -81,7 +86,8 @@ DFX_HD PlanLayout plan_layout(int num_seqs, int n_wg, int64_t capacity, int wave
     l.bounds_off = (l.prefix_off + (static_cast<int64_t>(num_seqs) + 1) * 4 + 63) / 64 * 64;
     l.work_off = (l.bounds_off + (static_cast<int64_t>(n_wg) + 1) * 4 + 63) / 64 * 64;
     l.order_off = (l.work_off + static_cast<int64_t>(n_wg) * sizeof(WgWork) + 63) / 64 * 64;
-    l.units_off = (l.order_off + static_cast<int64_t>(num_seqs) * 4 + 63) / 64 * 64;
+    l.first_off = (l.order_off + static_cast<int64_t>(num_seqs) * 4 + 63) / 64 * 64;
+    l.units_off = l.first_off + static_cast<int64_t>(n_wg) * kPlanFirst * waves * static_cast<int64_t>(sizeof(BandDesc));
     l.bands_off = l.units_off + capacity * static_cast<int64_t>(sizeof(UnitDesc));
     l.bytes = l.bands_off + capacity * waves * static_cast<int64_t>(sizeof(BandDesc));
     return l;
@@ -271,8 +277,9 @@ struct StreamAttn : TileMath<HD, NB, NW, HIDDEN> {
 
     // ---- loads -----------------------------------------------------------------------------
     // Start the loads of planned unit `rel` (this wave's band of K and V rows) into its ring stage.
-    DFX_D void issue_unit(int rel) const {
-        const BandDesc b = bands[rel * NW + wave];
+    DFX_D void issue_unit(int rel) const { issue_unit_desc(bands[rel * NW + wave], rel); }
+    // The same from a band descriptor the caller holds (wave-uniform or not: it is made uniform here).
+    DFX_D void issue_unit_desc(const BandDesc& b, int rel) const {
         const int last = uniform(b.last);
         const int tag = uniform(b.is_ctx);
         const bool is_ctx = tag > 0;
@@ -683,6 +690,134 @@ struct StreamAttn : TileMath<HD, NB, NW, HIDDEN> {
         }
     }
 
+    // Planned start of the pipelined kernel: one trip to memory (scalar loads of the plan's header,
+    // the workgroup's entry and the band descriptors of its waves' first units), after which every
+    // wave requests, in this order, its share of the descriptor tables (straight into LDS, as the
+    // tiles travel), the query rows of the first item and the tiles of the ring fill.  The tables are
+    // then the oldest loads in flight and are waited for alone.  body(n_units, prefilled): prefilled
+    // units have been requested together with the first item's query rows (0: nothing has, the
+    // classic start; later chunks of a long range; launches without a usable plan).
+    static constexpr int kPrefill = 2;  // units requested with the first item's query rows
+    template <typename Body>
+    DFX_D void for_each_chunk_prefetched(Body&& body) {
+        static_assert(HIDDEN && KVB == 2 && C::LOADS_PER_UNIT == 4 && C::kPlanUnits * NW <= 2 * C::THREADS, "table shares and wait counts below");
+        bool planned = false;
+        int64_t n_total = 0, n_first = 0, ubase = 0;
+        int n_active = 0, plan_mode = 0, prefilled = 0;
+        const UnitDesc* g_units = nullptr;
+        const BandDesc* g_bands = nullptr;
+        if (a.plan != nullptr) {
+            // All of it in one trip: five scalar loads issued together.  (The host has told where the
+            // tables start and checked that the buffer holds them: they may be read before the header has
+            // said whether the plan is this launch's.)
+            const PlanLayout lay = plan_layout(a.num_seqs, a.n_wg, a.plan_capacity, NW);
+            const uint8_t* hp = a.plan;
+            const uint8_t* ep = a.plan + lay.work_off + static_cast<int64_t>(blockIdx.x) * sizeof(WgWork);
+            const uint8_t* fp = a.plan + lay.first_off + (static_cast<int64_t>(blockIdx.x) * kPlanFirst * NW + wave_s) * sizeof(BandDesc);
+            typedef uint32_t words8 __attribute__((ext_vector_type(8)));
+            typedef uint32_t words16 __attribute__((ext_vector_type(16)));
+            words8 h;
+            words16 e;
+            u32x4 f[kPrefill];
+            static_assert(NW * sizeof(BandDesc) == 0x80 && sizeof(WgWork) == 64 && kPlanFirst >= kPrefill && kPrefill == 2, "the loads below");
+            asm volatile("s_load_dwordx8 %0, %4, 0x0\n\ts_load_dwordx16 %1, %5, 0x0\n\ts_load_dwordx4 %2, %6, 0x0\n\t"
+                         "s_load_dwordx4 %3, %6, 0x80\n\ts_waitcnt lgkmcnt(0)"
+                         : "=&s"(h), "=&s"(e), "=&s"(f[0]), "=&s"(f[1])
+                         : "s"(hp), "s"(ep), "s"(fp)
+                         : "memory");
+            planned = (h[0] == kPlanMagic) & (h[1] == a.plan_signature) & (static_cast<int32_t>(h[6]) == a.plan_capacity);
+            if (planned) {
+                n_active = static_cast<int>(h[2]);
+                plan_mode = static_cast<int>(h[3]);
+                per_head = static_cast<int>(h[4]);
+                const int64_t total = static_cast<int>(h[5]);
+                if (total == 0) return;
+                auto i64 = [&](int i) { return static_cast<int64_t>((static_cast<uint64_t>(e[i + 1]) << 32) | e[i]); };
+                const int64_t a0 = i64(0);
+                n_first = i64(2) - a0;
+                n_total = n_first + (i64(6) - i64(4));
+                ubase = static_cast<int32_t>(e[9]);
+                if (n_total <= 0) return;
+                split = make_wg_split(total, n_active);
+                if (plan_mode == 2) split.bounds = prefix;
+                rel_base = begin = a0;
+                end = a0 + n_total;
+                g_units = reinterpret_cast<const UnitDesc*>(a.plan + lay.units_off) + ubase;
+                g_bands = reinterpret_cast<const BandDesc*>(a.plan + lay.bands_off) + ubase * NW;
+                const int n_units = static_cast<int>(min(static_cast<int64_t>(C::kPlanUnits), n_total));
+                {
+                    const int t = thread_number_here(wave_s);
+                    const uint32_t share = static_cast<uint32_t>(wave_s) * 1024;
+                    if (t < n_units * 3) async_load16(g_units, t * 16, lds_of(units) + share);
+                    if (t < n_units * NW) async_load16(g_bands, t * 16, lds_of(bands) + share);
+                    if (t + C::THREADS < n_units * NW)
+                        async_load16(reinterpret_cast<const uint8_t*>(g_bands) + C::THREADS * 16, t * 16, lds_of(bands) + C::THREADS * 16 + share);
+                    // the plan's cut points, for the owners of a cut item's pieces (first read when a run ends)
+                    if (plan_mode == 2 && t * 4 <= n_active) async_load16(a.plan + lay.bounds_off, t * 16, lds_of(prefix) + share);
+                }
+                UnitDesc d;
+                d.q0 = static_cast<int32_t>(e[10]);
+                d.q_len = static_cast<int32_t>(e[11]);
+                d.kvh = static_cast<int32_t>(e[12]);
+                d.rt = static_cast<int32_t>(e[13]);
+                request_queries(d);
+                // Two units, not the ring's three: with the third behind them the query rows land later, and
+                // the launch came out no faster than without any of this (paired runs, 64 sequences x 4 KV heads
+                // of 8-32 tiles: one unit -0.2 us, two -0.4, three +0.4 against the copy of the tables through
+                // registers).  (The plan repeats the first units of the workgroup's first range only.)
+                prefilled = static_cast<int>(min(static_cast<int64_t>(min(n_units, kPrefill)), n_first > 0 ? n_first : n_total));
+#pragma unroll
+                for (int u = 0; u < kPrefill; ++u) {
+                    if (u < prefilled) {
+                        BandDesc b;
+                        b.off = static_cast<int64_t>((static_cast<uint64_t>(f[u][1]) << 32) | f[u][0]);
+                        b.last = static_cast<int32_t>(f[u][2]);
+                        b.is_ctx = static_cast<int32_t>(f[u][3]);
+                        issue_unit_desc(b, u);
+                    }
+                }
+                // the tables are this wave's oldest loads: 8 of query rows and 4 per unit are younger
+                static_assert(kPrefill == 2, "wait counts");
+                if (prefilled == 2) wait_async_loads<8 + 8>();
+                else wait_async_loads<8 + 4>();
+            }
+        }
+        if (!planned) {
+            const UnitSummary summary = build_unit_prefix<C::RT>(a, prefix, misc);
+            per_head = summary.per_head;
+            const int64_t total = static_cast<int64_t>(per_head) * a.h_kv;
+            if (total == 0) return;
+            n_active = a.fixed_wg ? a.n_wg
+                                  : effective_workgroups(total, static_cast<int64_t>(summary.items) * a.h_kv, summary.max_tiles, a.n_wg);
+            split = make_wg_split(total, n_active);
+            if (static_cast<int>(blockIdx.x) >= n_active) return;
+            rel_base = begin = split.first(blockIdx.x);
+            end = split.first(blockIdx.x + 1);
+            n_total = end - begin;
+        }
+        for (int64_t done = 0; done < n_total; done += C::kPlanUnits) {
+            const int n_units = static_cast<int>(min(static_cast<int64_t>(C::kPlanUnits), n_total - done));
+            const bool prefetched = planned && done == 0;
+            if (!prefetched) {
+                __syncthreads();  // every wave is done with the previous descriptors and their stages
+                if (planned) {
+                    const int t = thread_number_here(wave_s);
+                    const u32x4* su = reinterpret_cast<const u32x4*>(g_units + done);
+                    u32x4* du = reinterpret_cast<u32x4*>(units);
+                    const u32x4* sb = reinterpret_cast<const u32x4*>(g_bands + done * NW);
+                    u32x4* db = reinterpret_cast<u32x4*>(bands);
+                    for (int i = t; i < n_units * 3; i += C::THREADS) du[i] = su[i];
+                    for (int i = t; i < n_units * NW; i += C::THREADS) db[i] = sb[i];
+                } else {
+                    plan_units(begin + done, n_units);
+                }
+            }
+            __syncthreads();
+            body(n_units, prefetched ? prefilled : 0);
+        }
+    }
+    DFX_D static uint32_t lds_of(const void* p) { return static_cast<uint32_t>(reinterpret_cast<uintptr_t>(p)); }
+
     // Wait until at most `younger` units' loads of this wave are outstanding (younger <= 2).
     DFX_D static void wait_younger(int younger) {
         if (younger >= 2) wait_async_loads<2 * C::LOADS_PER_UNIT>();
@@ -858,25 +993,15 @@ paged_attn_pipe_kernel(const KArgs a) {
     const bool busy = at.wave < a.busy_waves;  // waves whose 32 rows exist in no item of this launch only fetch
     constexpr int kHoleRows = C::ROWS_PER_WAVE;
     static_assert(kHoleRows == 8 || kHoleRows == 16, "mask blocks of attn_pipe_gen.h");
-    // With a plan the query rows of the workgroup's first item are requested as soon as its entry of
-    // the plan has been read, together with the descriptors, instead of a trip to memory later.
-    bool requested_early = false;
-    auto on_work = [&](const WgWork& w) {
-        UnitDesc d;
-        d.q0 = w.q0;
-        d.q_len = w.q_len;
-        d.kvh = w.kvh;
-        d.rt = w.rt;
-        at.request_queries(d);
-        requested_early = true;
-    };
-    at.for_each_chunk([&](int n_units) {
+    // With a plan the query rows of the workgroup's first item and the tiles of the ring fill are
+    // requested as soon as its entry of the plan has been read (for_each_chunk_prefetched: `prefilled`
+    // units are on their way then, behind the query rows).
+    at.for_each_chunk_prefetched([&](int n_units, int prefilled) {
         const WgSplit& split = at.split;
         // An item that opens with this chunk: its query rows first.  Requested behind the ring fill,
         // the wait for them would also wait for every tile of the fill.
         const bool opens = (uniform(at.units[0].flags) & kUnitFirst) != 0;
-        if (opens && !requested_early) at.request_queries(at.units[0]);
-        requested_early = false;
+        if (opens && prefilled == 0) at.request_queries(at.units[0]);
         // While the query rows are on their way: the marks of the plain steps.  They are first read
         // behind the barrier of the first run's first step; they only add bits to the flags that
         // nobody looks at before.  (Not behind the ring fill: a spilled register reloaded here would
@@ -884,10 +1009,13 @@ paged_attn_pipe_kernel(const KArgs a) {
         at.mark_plain_steps(n_units, PREFILL);
         __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the marks are written before this wave reaches that barrier
         if (opens) {
-            wait_async_loads<0>();
+            // the query rows: everything in flight, or everything but the tiles requested behind them
+            if (prefilled == 0) wait_async_loads<0>();
+            else if (prefilled == 1) wait_async_loads<C::LOADS_PER_UNIT>();
+            else wait_async_loads<2 * C::LOADS_PER_UNIT>();
             at.adopt_item(at.units[0]);
         }
-        int issued = 0;  // ring fill: kStages - 1 units in flight
+        int issued = prefilled;  // ring fill: kStages - 1 units in flight
         for (; issued < C::kStages - 1 && issued < n_units; ++issued) at.issue_unit(issued);
 
         auto tile_of = [&](int r) { return smem + C::STAGES_OFF + (static_cast<unsigned>(r) % C::kStages) * C::STAGE_BYTES; };
@@ -1076,7 +1204,7 @@ paged_attn_pipe_kernel(const KArgs a) {
             at.finish_run(rel - 1, split);
             if (next_opens) at.adopt_item(at.units[run_end]);
         }
-    }, on_work);
+    });
 }
 
 // The FP8 kernel with the pipelined tile step: the ring holds the codes as stored (4 stages of

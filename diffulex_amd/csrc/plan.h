@@ -11,6 +11,7 @@
 //                                               item of its first unit
 //   int32 order[num_seqs]                       header.reordered: the sequence at every position of the
 //                                               unit space (prefix[] then runs over positions)
+//   BandDesc first[n_wg][kPlanFirst][NW]        the band descriptors of every workgroup's first units
 //   UnitDesc units[capacity]                    one per unit, in each workgroup's processing order
 //   BandDesc bands[capacity * NW]               one per unit and wave
 // Two kernels fill it: paged_attn_plan_kernel (one workgroup: prefix, partition) and
@@ -470,6 +471,11 @@ __global__ void __launch_bounds__(64 * NW) paged_attn_plan_fill_kernel(const KAr
             const int n = static_cast<int>(min(static_cast<int64_t>(C::kPlanUnits), at.end - chunk));
             at.plan_units(chunk, n, seg == 0 ? w.partner : -1, seg);
             __syncthreads();
+            if (first_chunk && static_cast<int>(threadIdx.x) < min(n, kPlanFirst) * NW) {
+                // the first units' band descriptors once more, where the attention kernel finds them with its entry
+                BandDesc* g_first = reinterpret_cast<BandDesc*>(pa.buf + lay.first_off) + static_cast<int64_t>(blockIdx.x) * kPlanFirst * NW;
+                g_first[threadIdx.x] = at.bands[threadIdx.x];
+            }
             if (first_chunk && threadIdx.x == 0) {
                 // the first unit's item, for the attention kernel to request its query rows early
                 WgWork* mine = reinterpret_cast<WgWork*>(pa.buf + lay.work_off) + blockIdx.x;

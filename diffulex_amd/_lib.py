@@ -53,6 +53,9 @@ class AttnParams(C.Structure):
         ("store_slot_mapping", C.c_void_p), ("store_slot_index_type", C.c_int32),
         ("plan", C.c_void_p), ("plan_bytes", C.c_int64), ("num_new_tokens", C.c_int64),
         ("cache_layout", C.c_int32), ("num_q_tokens", C.c_int32), ("kc_stride", C.c_int64 * 5), ("vc_stride", C.c_int64 * 4),
+        ("rope_cos_sin", C.c_void_p), ("rope_positions", C.c_void_p), ("rope_position_index_type", C.c_int32),
+        ("reserved2", C.c_int32), ("rope_max_position", C.c_int64), ("k_rotated", C.c_void_p),
+        ("kr_stride_token", C.c_int64), ("kr_stride_head", C.c_int64),
     ]
 
 
@@ -82,6 +85,7 @@ class MetadataParams(C.Structure):
         ("cu_seqlens_q", C.c_void_p), ("cu_seqlens_k", C.c_void_p), ("context_lens", C.c_void_p),
         ("seq_lens", C.c_void_p), ("padded_seqs", C.c_int32), ("reserved", C.c_int32),
         ("padded_tokens", C.c_int64), ("summary", C.c_void_p),
+        ("token_ids", C.c_void_p), ("token_ids_stride", C.c_int64), ("input_ids", C.c_void_p),
     ]
 
 

@@ -10,7 +10,7 @@ import torch
 import torch.nn as nn
 
 from . import metadata as _metadata
-from .dllm_flash_attn import dllm_flash_attn_decode, dllm_flash_attn_prefill
+from .dllm_flash_attn import dllm_flash_attn_decode, dllm_flash_attn_prefill, rope_supported
 from .kv_cache_kernels import store_kvcache_distinct_layout, store_kvcache_unified_layout
 
 
@@ -27,7 +27,22 @@ class Attention(nn.Module):
         # looked up at call time so that a later set_fetch_fn_for_attn_metadata() is seen
         self.fetch_attn_metadata = lambda: _metadata.fetch_attn_metadata()
 
-    def forward(self, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask=None) -> torch.Tensor:
+    def forward(self, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask=None, rope=None) -> torch.Tensor:
+        """``rope=(rotary_embedding, positions)`` (extension): q and k are the projections BEFORE the rotary
+        embedding (diffulex/model/dream.py:94-99 applies it right before this call); it is applied inside
+        the attention launch where that launch can (decode, unified layout, ``rope_supported``), by the
+        rotary embedding's own launch otherwise."""
+        if rope is not None:
+            rotary, positions = rope
+            md = self.fetch_attn_metadata()
+            fused = (not md.is_prefill and md.kv_cache_layout == "unified" and self.k_cache.numel() > 0 and
+                     rope_supported(self.num_heads, self.num_kv_heads, self.head_dim, int(md.max_seqlen_q or 0),
+                                    self.k_cache.shape[1], md.cu_seqlens_q.numel() - 1, q.device))
+            if not fused:
+                q, k = rotary(positions, q, k)
+                rope = None
+            else:
+                rope = (rotary.cos_sin_cache, positions)
         q = q.view(q.shape[0], self.num_heads, self.head_dim)
         k = k.view(k.shape[0], self.num_kv_heads, self.head_dim)
         v = v.view(v.shape[0], self.num_kv_heads, self.head_dim)
@@ -46,10 +61,11 @@ class Attention(nn.Module):
                 # launch's worth of time up to about 4 MB of fresh K+V and loses beyond 8 MB, where a
                 # store kernel of its own has far more loads in flight than the attention grid)
                 if (self.fuse_kv_store and is_unified_layout and not attn_metadata.is_prefill
-                        and k.numel() * 4 <= self.fuse_kv_store_max_bytes
+                        and (k.numel() * 4 <= self.fuse_kv_store_max_bytes or rope is not None)
                         and slots.is_contiguous() and slots.dtype in (torch.int32, torch.int64)):
                     fused_slots = slots
                 else:
+                    assert rope is None, "the rotary embedding inside the attention launch stores through that launch"
                     store_kvcache = store_kvcache_unified_layout if is_unified_layout else store_kvcache_distinct_layout
                     store_kvcache(k, v, k_cache, v_cache, slots, attn_metadata)
 
@@ -58,7 +74,7 @@ class Attention(nn.Module):
         else:
             if is_unified_layout:
                 o = dllm_flash_attn_decode(q, k, v, k_cache, v_cache, self.scale, attn_metadata,
-                                           store_slot_mapping=fused_slots)
+                                           store_slot_mapping=fused_slots, rope=rope)
             else:
                 # (the reference raises NotImplementedError here, attn_impl.py:66-69)
                 o = dllm_flash_attn_decode(q, k, v, k_cache, v_cache, self.scale, attn_metadata,

@@ -47,6 +47,16 @@ struct KArgs {
     int store_slots_i64;
     int64_t n_new;            // rows of k_new / v_new (and of the slot mapping)
     int32_t n_q;              // rows of q / out: no row at or beyond it is read or written, whatever the offsets say
+    // Rotary embedding inside the launch (pipelined kernels; null table: off).  q and k_src hold the
+    // projections as they leave the linear layer; the query rows are rotated in the Q operand registers, the
+    // fresh K rows of an item by the workgroup that owns the item's fresh tiles, from k_src into k_new (which
+    // is then an output of the launch that its own tile loads read back), and into the cache with the store.
+    const float* rope_table;  // [rope_max_pos, head_dim] fp32: cosines, then sines
+    const void* rope_pos;     // position of token t: row t of q and row t of k_src / k_new / v_new (the same tokens)
+    int rope_pos_i64;
+    int64_t rope_max_pos;
+    const uint16_t* k_src;
+    int64_t ks_st, ks_sh;
     int64_t v_fresh_delta;    // streaming paths: (token stride of v_new - token stride of k_new) in bytes
     const uint8_t* plan;      // launch plan built by the plan kernels, or null
     uint32_t plan_signature;  // of this launch's configuration: a plan made for another one is ignored
@@ -380,7 +390,11 @@ struct AttnState {
     static constexpr int kDeviceScope = 16;  // cache policy: sc1
 
     DFX_D __amdgpu_buffer_rsrc_t block_resource(int slot, int qb) const {
-        float* bp = slot_ptr(slot) + (wave * NB + qb) * S::BLOCK_FLOATS;
+        // (the wave's number made opaque here: its share of the address, worked out at the kernel's entry,
+        // would wait in scratch until an item is cut, and the reload is a trip to memory)
+        int w = wave;
+        asm volatile("" : "+v"(w));
+        float* bp = slot_ptr(slot) + (w * NB + qb) * S::BLOCK_FLOATS;
         return __builtin_amdgcn_make_buffer_rsrc(bp, 0, S::BLOCK_FLOATS * 4, 0x00020000);
     }
 
@@ -425,8 +439,17 @@ struct AttnState {
         return __builtin_convertvector(__builtin_bit_cast(f16x2, w), f32x2);
     }
 
+    // (the lane's number made opaque where a piece is moved: offsets derived from it at the kernel's entry
+    // would wait in scratch until an item is cut)
+    DFX_D int lane_here() const {
+        int l = lane;
+        asm volatile("" : "+v"(l));
+        return l;
+    }
+
     DFX_D void store_partial(int slot, const float (&l_tot)[NB]) const {
         if (wave >= a.busy_waves) return;  // no rows in any item of the launch: merge_partial skips it too
+        const int lane = lane_here();
 #pragma unroll
         for (int qb = 0; qb < NB; ++qb) {
             const __amdgpu_buffer_rsrc_t rs = block_resource(slot, qb);
@@ -481,6 +504,7 @@ struct AttnState {
         // in this toolchain and fuse like any other.
 #pragma clang fp contract(off)
         if (wave >= a.busy_waves) return;
+        const int lane = lane_here();
 #pragma unroll
         for (int qb = 0; qb < NB; ++qb) {
             const __amdgpu_buffer_rsrc_t rs = block_resource(slot, qb);

@@ -95,7 +95,10 @@ DFX_HD PlanLayout plan_layout(int num_seqs, int n_wg, int64_t capacity, int wave
 
 // UnitDesc::flags: bits 8..15 a bit per band of rows whose page is missing (holes); bits 16..21, set by
 // mark_plain_steps() only, the number of consecutive plain steps that begin with this unit
-enum : int32_t { kUnitCtx = 1, kUnitFirst = 2, kUnitLast = 4, kUnitComplete = 8, kUnitHoleShift = 8, kUnitPlainShift = 16 };
+// kUnitFreshStart: the item's first tile of fresh rows, or the first tile of the workgroup's piece of the item
+// where that is a later one of them (where the fresh rows' rotary embedding is the launch's, the workgroup
+// rotates the item's fresh K rows when it meets this unit)
+enum : int32_t { kUnitCtx = 1, kUnitFirst = 2, kUnitLast = 4, kUnitComplete = 8, kUnitFreshStart = 16, kUnitHoleShift = 8, kUnitPlainShift = 16 };
 DFX_HD uint32_t unit_holes(int flags) { return (static_cast<uint32_t>(flags) >> kUnitHoleShift) & 0xffu; }
 
 // COMPACT: a configuration small enough (2 stages, short plan, at most kCompactMaxSeqs sequences)
@@ -243,7 +246,8 @@ struct StreamAttn : TileMath<HD, NB, NW, HIDDEN> {
                 d.limit = limit;
                 d.flags = (is_ctx ? kUnitCtx : 0) | (tile == tile0 ? kUnitFirst : 0) |
                           (tile == tile1 - 1 ? kUnitLast : 0) |
-                          (tile0 == 0 && tile1 == item_tiles ? kUnitComplete : 0);
+                          (tile0 == 0 && tile1 == item_tiles ? kUnitComplete : 0) |
+                          (!is_ctx && (tile == shp.n_ctx_tiles || tile == tile0) ? kUnitFreshStart : 0);
                 d.partner = partner;
                 d.run = tile1 - tile;
                 d.item_rel = static_cast<int>(pos - tile - rel_base);
@@ -480,6 +484,106 @@ struct StreamAttn : TileMath<HD, NB, NW, HIDDEN> {
         }
         this->reset_accumulators();
     }
+    // ---- rotary embedding inside the launch (KArgs::rope_table) ---------------------------------------
+    DFX_D int64_t rope_position(int64_t token) const {
+        int64_t pos = a.rope_pos_i64 ? static_cast<const int64_t*>(a.rope_pos)[token]
+                                     : static_cast<int64_t>(static_cast<const int32_t*>(a.rope_pos)[token]);
+        // (outside the table: a caller error, clamped as dfx_rope_kv_store clamps it)
+        return pos < 0 ? 0 : (pos >= a.rope_max_pos ? a.rope_max_pos - 1 : pos);
+    }
+    // The query rows of item d are rotated in the Q operand registers once they have landed: the position
+    // of the lane's row first (a load of its own, which the caller lets travel with other work), then the
+    // request for its angles, then pipe_rope_queries().
+    DFX_D int64_t rope_query_position(const UnitDesc& d) const {
+        static_assert(HIDDEN && HD == 128, "pipelined kernels");
+        const int q_len = uniform(d.q_len);
+        const int r = this->row_of(uniform(d.rt), 0);
+        const int i = r < a.group * q_len ? r % q_len : 0;
+        int row = uniform(d.q0) + i;
+        row = row < a.n_q ? row : 0;
+        return rope_position(row);
+    }
+    DFX_D void request_rope_angles(int64_t pos) const {
+        int h = half;  // (opaque: the lane's share of the address is then not worked out at the kernel's entry and kept in scratch)
+        asm volatile("" : "+v"(h));
+        pipe_issue_rope_angles(a.rope_table + pos * HD + h * 8);
+    }
+    DFX_D void rope_queries(const UnitDesc& d) const {
+        request_rope_angles(rope_query_position(d));
+        pipe_rope_queries();
+    }
+    // The fresh K rows of sequence sq, KV head kv_head: rotated from k_src into k_new and, with the fused
+    // store, into their cache slots together with the V rows (what dfx_rope_kv_store does in a launch of its
+    // own, bit for bit).  All threads of the workgroup; a lane takes a pair of 16-byte chunks (c, c + 8) of
+    // a row.  Several workgroups (the row tiles of one sequence and head) may do the same rows: they write
+    // the same bytes.
+    template <bool FP8>
+    DFX_D void rope_fresh_rows(int sq, int kv_head) const {
+        static_assert(HIDDEN && HD == 128, "pipelined kernels");
+        const int64_t n0 = min(static_cast<int64_t>(a.cu_new[sq]), a.n_new), n1 = min(static_cast<int64_t>(a.cu_new[sq + 1]), a.n_new);
+        const int64_t n_slots = a.n_pages * a.page_size;
+        for (int64_t idx = thread_number_here(wave_s); idx < (n1 - n0) * 8; idx += C::THREADS) {
+            const int64_t t = n0 + (idx >> 3);
+            const int c = static_cast<int>(idx & 7);
+            uint32_t lo[4], hi[4];
+            pipe_rope_row(a.k_src + t * a.ks_st + kv_head * a.ks_sh + c * 8, a.rope_table + rope_position(t) * HD + c * 8, lo, hi);
+            const u32x4 o1 = {lo[0], lo[1], lo[2], lo[3]}, o2 = {hi[0], hi[1], hi[2], hi[3]};
+            uint16_t* dst = const_cast<uint16_t*>(a.k_new) + t * a.kn_st + kv_head * a.kn_sh + c * 8;
+            *reinterpret_cast<u32x4*>(dst) = o1;
+            *reinterpret_cast<u32x4*>(dst + HD / 2) = o2;
+            if (a.store_slots == nullptr) continue;
+            int64_t slot = a.store_slots_i64 ? static_cast<const int64_t*>(a.store_slots)[t]
+                                             : static_cast<int64_t>(static_cast<const int32_t*>(a.store_slots)[t]);
+            if (slot < 0 || slot >= n_slots) continue;
+            const int64_t page = a.page_shift >= 0 ? (slot >> a.page_shift) : slot / a.page_size;
+            const int64_t e = page * a.c_sp + (slot - page * a.page_size) * a.c_st + kv_head * a.c_sh + c * 8;  // elements
+            const uint16_t* vp = a.v_new + t * a.vn_st + kv_head * a.vn_sh + c * 8;
+            const u32x4 v1 = *reinterpret_cast<const u32x4*>(vp), v2 = *reinterpret_cast<const u32x4*>(vp + HD / 2);
+            uint8_t* kc = const_cast<uint8_t*>(a.k_cache);
+            uint8_t* vc = const_cast<uint8_t*>(a.v_cache);
+            if constexpr (FP8) {
+                const float ks = a.k_scale[kv_head], vs = a.v_scale[kv_head];
+                *reinterpret_cast<u32x2*>(kc + e) = quantise8(o1, ks);
+                *reinterpret_cast<u32x2*>(kc + e + HD / 2) = quantise8(o2, ks);
+                *reinterpret_cast<u32x2*>(vc + e) = quantise8(v1, vs);
+                *reinterpret_cast<u32x2*>(vc + e + HD / 2) = quantise8(v2, vs);
+            } else {
+                *reinterpret_cast<u32x4*>(kc + e * 2) = o1;
+                *reinterpret_cast<u32x4*>(kc + e * 2 + HD) = o2;
+                *reinterpret_cast<u32x4*>(vc + e * 2) = v1;
+                *reinterpret_cast<u32x4*>(vc + e * 2 + HD) = v2;
+            }
+        }
+    }
+    // The same for every item whose fresh tiles begin among the n_units units in the tables (kUnitFreshStart),
+    // before any of those tiles is requested.  Every thread of the workgroup; the tables are complete.
+    // Returns whether any row was written: the caller then waits for its stores (vmcnt(0)) and lets the
+    // workgroup meet at a barrier before a tile load asks for the rows.
+    template <bool FP8>
+    DFX_D bool rope_fresh_rows_of_chunk(int n_units) const {
+        const int t = thread_number_here(wave_s);
+        const bool starts = t < n_units && (units[t].flags & kUnitFreshStart) != 0;
+        const uint64_t votes = __ballot(starts);
+        if (wave_s < 2 && t == wave_s * 64) {
+            misc[20 + 2 * wave_s] = static_cast<int>(votes);
+            misc[21 + 2 * wave_s] = static_cast<int>(votes >> 32);
+        }
+        __syncthreads();
+        static_assert(C::kPlanUnits <= 128 && NW >= 2, "two waves' ballots cover a table");
+        bool any = false;
+        for (int w = 0; w < 2; ++w) {
+            uint64_t m = (static_cast<uint64_t>(static_cast<uint32_t>(uniform(misc[21 + 2 * w]))) << 32) |
+                         static_cast<uint32_t>(uniform(misc[20 + 2 * w]));
+            while (m != 0) {
+                const int r = w * 64 + __builtin_ctzll(m);
+                m &= m - 1;
+                rope_fresh_rows<FP8>(uniform(units[r].s), uniform(units[r].kvh));
+                any = true;
+            }
+        }
+        return any;
+    }
+
     // First key position the lane's query row does not see under the block-causal mask (fresh tiles
     // only).  Worked out where a tile needs it, once or twice per item, rather than kept per item: a
     // value that lives through the tile loop takes one of the few registers the compiler has there.
@@ -698,6 +802,7 @@ struct StreamAttn : TileMath<HD, NB, NW, HIDDEN> {
     // units have been requested together with the first item's query rows (0: nothing has, the
     // classic start; later chunks of a long range; launches without a usable plan).
     static constexpr int kPrefill = 2;  // units requested with the first item's query rows
+    bool queries_requested = false;     // ... which the planned start has requested (the first chunk's body resets it)
     template <typename Body>
     DFX_D void for_each_chunk_prefetched(Body&& body) {
         static_assert(HIDDEN && KVB == 2 && C::LOADS_PER_UNIT == 4 && C::kPlanUnits * NW <= 2 * C::THREADS, "table shares and wait counts below");
@@ -766,6 +871,9 @@ struct StreamAttn : TileMath<HD, NB, NW, HIDDEN> {
                 // of 8-32 tiles: one unit -0.2 us, two -0.4, three +0.4 against the copy of the tables through
                 // registers).  (The plan repeats the first units of the workgroup's first range only.)
                 prefilled = static_cast<int>(min(static_cast<int64_t>(min(n_units, kPrefill)), n_first > 0 ? n_first : n_total));
+                // (with the rotary embedding inside the launch a tile of fresh rows waits for their rotation)
+                if (a.rope_table != nullptr) prefilled = static_cast<int32_t>(f[0][3]) <= 0 ? 0 : (prefilled == 2 && static_cast<int32_t>(f[1][3]) <= 0 ? 1 : prefilled);
+                queries_requested = true;
 #pragma unroll
                 for (int u = 0; u < kPrefill; ++u) {
                     if (u < prefilled) {
@@ -779,7 +887,8 @@ struct StreamAttn : TileMath<HD, NB, NW, HIDDEN> {
                 // the tables are this wave's oldest loads: 8 of query rows and 4 per unit are younger
                 static_assert(kPrefill == 2, "wait counts");
                 if (prefilled == 2) wait_async_loads<8 + 8>();
-                else wait_async_loads<8 + 4>();
+                else if (prefilled == 1) wait_async_loads<8 + 4>();
+                else wait_async_loads<8>();
             }
         }
         if (!planned) {
@@ -989,7 +1098,8 @@ paged_attn_pipe_kernel(const KArgs a) {
             pipe_set_load_offsets(o[0], o[1]);
         }
     }
-    store_fresh_rows<HD, false, 1>(a);
+    const bool rope = !PREFILL && a.rope_table != nullptr;  // (with it the store travels with the rotation of the fresh K rows)
+    if (!rope) store_fresh_rows<HD, false, 1>(a);
     const bool busy = at.wave < a.busy_waves;  // waves whose 32 rows exist in no item of this launch only fetch
     constexpr int kHoleRows = C::ROWS_PER_WAVE;
     static_assert(kHoleRows == 8 || kHoleRows == 16, "mask blocks of attn_pipe_gen.h");
@@ -1001,7 +1111,25 @@ paged_attn_pipe_kernel(const KArgs a) {
         // An item that opens with this chunk: its query rows first.  Requested behind the ring fill,
         // the wait for them would also wait for every tile of the fill.
         const bool opens = (uniform(at.units[0].flags) & kUnitFirst) != 0;
-        if (opens && prefilled == 0) at.request_queries(at.units[0]);
+        if (opens && !at.queries_requested) at.request_queries(at.units[0]);
+        at.queries_requested = false;
+        // The rotary embedding inside the launch: the fresh K rows of the items that end in this chunk, and the
+        // angles of the first item's query rows, requested behind the stores of those rows so that the two
+        // trips to memory run together.
+        bool rotate_first = false;
+        if constexpr (!PREFILL) {
+            if (rope) {
+                int64_t pos = 0;
+                if (opens) pos = at.rope_query_position(at.units[0]);
+                const bool any = at.template rope_fresh_rows_of_chunk<false>(n_units);
+                if (opens) at.request_rope_angles(pos);
+                rotate_first = opens;
+                if (any) {
+                    wait_async_loads<0>();  // this thread's rows are in memory ...
+                    __syncthreads();        // ... and so are everybody's, before a tile load asks for them
+                }
+            }
+        }
         // While the query rows are on their way: the marks of the plain steps.  They are first read
         // behind the barrier of the first run's first step; they only add bits to the flags that
         // nobody looks at before.  (Not behind the ring fill: a spilled register reloaded here would
@@ -1013,6 +1141,7 @@ paged_attn_pipe_kernel(const KArgs a) {
             if (prefilled == 0) wait_async_loads<0>();
             else if (prefilled == 1) wait_async_loads<C::LOADS_PER_UNIT>();
             else wait_async_loads<2 * C::LOADS_PER_UNIT>();
+            if (rotate_first) pipe_rope_queries();
             at.adopt_item(at.units[0]);
         }
         int issued = prefilled;  // ring fill: kStages - 1 units in flight
@@ -1202,7 +1331,12 @@ paged_attn_pipe_kernel(const KArgs a) {
             }
             if (next_opens) wait_async_loads<0>();  // the next item's query rows (and the tiles requested before them)
             at.finish_run(rel - 1, split);
-            if (next_opens) at.adopt_item(at.units[run_end]);
+            if (next_opens) {
+                if constexpr (!PREFILL) {
+                    if (rope) at.rope_queries(at.units[run_end]);
+                }
+                at.adopt_item(at.units[run_end]);
+            }
         }
     });
 }
@@ -1236,7 +1370,8 @@ paged_attn_pipe_fp8_kernel(const KArgs a) {
                                  wide + SA::L::chunk_offset(row, 2 * cc), wide + SA::L::chunk_offset(row, 2 * cc + 1));
     }
     static_assert(C::IPW == 1, "pipe_widen: one load of codes per wave and matrix");
-    store_fresh_rows<HD, true, 1>(a);
+    const bool rope = a.rope_table != nullptr;  // (with it the store travels with the rotation of the fresh K rows)
+    if (!rope) store_fresh_rows<HD, true, 1>(a);
     const bool busy = at.wave < a.busy_waves;
     constexpr int kHoleRows = C::ROWS_PER_WAVE;
     static_assert(kHoleRows == 8, "mask blocks of attn_pipe_gen.h");
@@ -1266,9 +1401,20 @@ paged_attn_pipe_fp8_kernel(const KArgs a) {
         const bool opens = (uniform(at.units[0].flags) & kUnitFirst) != 0;
         if (opens && !requested_early) at.request_queries(at.units[0]);
         requested_early = false;
+        if (rope) {  // (as in the bf16 kernel)
+            int64_t pos = 0;
+            if (opens) pos = at.rope_query_position(at.units[0]);
+            const bool any = at.template rope_fresh_rows_of_chunk<true>(n_units);
+            if (opens) at.request_rope_angles(pos);
+            if (any) {
+                wait_async_loads<0>();
+                __syncthreads();
+            }
+        }
         at.mark_plain_steps(n_units);  // (while the query rows are on their way; first read behind a barrier)
         if (opens) {
             wait_async_loads<0>();
+            if (rope) pipe_rope_queries();
             adopt(at.units[0]);
         }
         // ring fill, and the tiles the first step reads
@@ -1439,7 +1585,10 @@ paged_attn_pipe_fp8_kernel(const KArgs a) {
             }
             if (next_opens) wait_async_loads<0>();
             at.finish_run(rel - 1, split);
-            if (next_opens) adopt(at.units[run_end]);
+            if (next_opens) {
+                if (rope) at.rope_queries(at.units[run_end]);
+                adopt(at.units[run_end]);
+            }
         }
     }, on_work);
 }

@@ -292,6 +292,77 @@ def mask_block(s, hole_rows):
     return join(ins)
 
 
+def rotate_pairs(ins, x1, x2, cos, sin, y1, y2, t):
+    """Rotates the two bf16 pairs in registers x1 (elements e, e + 1 of the lower half of a head row) and
+    x2 (the same elements of the upper half) by the angles whose cosines / sines are in registers cos,
+    cos + 1 / sin, sin + 1: y1 = x1 * cos - x2 * sin, y2 = x2 * cos + x1 * sin, every product and the sum
+    rounded on their own (the reference evaluates them as separate fp32 tensor operations:
+    diffulex/layer/rotary_embedding.py:13-16), then rounded to nearest even to bf16.  t: 8 scratch registers."""
+    a_lo, a_hi, b_lo, b_hi, p, q, r, u = range(t, t + 8)
+    ins += [f"v_lshlrev_b32 {vr(a_lo)}, 16, {vr(x1)}", f"v_and_b32 {vr(a_hi)}, 0xffff0000, {vr(x1)}",
+            f"v_lshlrev_b32 {vr(b_lo)}, 16, {vr(x2)}", f"v_and_b32 {vr(b_hi)}, 0xffff0000, {vr(x2)}"]
+    for a, b, c, sn, o1, o2 in ((a_lo, b_lo, cos, sin, p, q), (a_hi, b_hi, cos + 1, sin + 1, r, u)):
+        ins += [f"v_mul_f32 {vr(o1)}, {vr(a)}, {vr(c)}", f"v_mul_f32 {vr(o2)}, {vr(b)}, {vr(sn)}",
+                f"v_sub_f32 {vr(o1)}, {vr(o1)}, {vr(o2)}",                    # y1 = x1 c - x2 s
+                f"v_mul_f32 {vr(o2)}, {vr(b)}, {vr(c)}", f"v_mul_f32 {vr(a)}, {vr(a)}, {vr(sn)}",
+                f"v_add_f32 {vr(o2)}, {vr(o2)}, {vr(a)}"]                      # y2 = x2 c + x1 s
+    ins += [f"v_cvt_pk_bf16_f32 {vr(y1)}, {vr(p)}, {vr(r)}", f"v_cvt_pk_bf16_f32 {vr(y2)}, {vr(q)}, {vr(u)}"]
+
+
+def rope_queries_fns():
+    """Rotary embedding of the query rows in the Q operand registers, in two blocks: the request for the
+    cosines / sines of the lane's elements (2 x 32 floats of its position's table row, into the score sets,
+    which are free between two items), and the rotation once they and the query rows have landed.  The lane
+    holds, of its row, elements 16 s + 8 h .. + 7 in slab s (h: the wave's half): slabs s and s + 4 are the
+    two halves a rotation mixes."""
+    loads = []
+    for s in range(NSLAB // 2):
+        for j in range(2):
+            loads.append(f"global_load_dwordx4 {vr(SA + 8 * s + 4 * j, 4)}, %[t], off offset:{(16 * s + 4 * j) * 4}")
+            loads.append(f"global_load_dwordx4 {vr(SB + 8 * s + 4 * j, 4)}, %[t], off offset:{(HD // 2 + 16 * s + 4 * j) * 4}")
+    ins = ["s_waitcnt vmcnt(0)"]
+    x1, x2, t = RING, RING + 1, TMP
+    for s in range(NSLAB // 2):
+        for j in range(4):
+            lo, hi = Q_BASE + 4 * s + j, Q_BASE + 4 * (s + NSLAB // 2) + j
+            ins += [f"v_accvgpr_read_b32 {vr(x1)}, {ar(lo)}", f"v_accvgpr_read_b32 {vr(x2)}, {ar(hi)}"]
+            rotate_pairs(ins, x1, x2, SA + 8 * s + 2 * j, SB + 8 * s + 2 * j, RING + 2, RING + 3, t)
+            ins += [f"v_accvgpr_write_b32 {ar(lo)}, {vr(RING + 2)}", f"v_accvgpr_write_b32 {ar(hi)}, {vr(RING + 3)}"]
+    ins.append("s_nop 1")  # (a matrix instruction may read the operand next)
+    return (asm_fn("pipe_issue_rope_angles", "const void* table_row", join(loads), ins=['[t] "v"(table_row)'], clobbers=["memory"],
+                   comment="Requests the cosines and sines of the lane's query elements: `table_row` is the lane's position's row of\n"
+                           "the angle table plus 8 h floats.  They go to the score sets, which are free between two items.") +
+            asm_fn("pipe_rope_queries", "", join(ins), clobbers=["memory"],
+                   comment="Rotates the query row in the Q operand registers by the angles pipe_issue_rope_angles() has requested:\n"
+                           "the arithmetic of dfx_rope_kv_store, bit for bit.  Waits for every load of the wave in flight (the\n"
+                           "angles, the query rows); the operand ring is free (between two items)."))
+
+
+def rope_row_fn():
+    """Rotary embedding of one pair of 16-byte chunks (c, c + 8) of a fresh K head row, in the blocks' registers:
+    the kernel's per-item rotation of the fresh K rows (the compiler's 32 registers would not hold it)."""
+    ins = [f"global_load_dwordx4 {vr(SA, 4)}, %[k], off", f"global_load_dwordx4 {vr(SA + 4, 4)}, %[k], off offset:{HD}",
+           f"global_load_dwordx4 {vr(SA + 8, 4)}, %[t], off", f"global_load_dwordx4 {vr(SA + 12, 4)}, %[t], off offset:16",
+           f"global_load_dwordx4 {vr(SA + 16, 4)}, %[t], off offset:{HD * 2}",
+           f"global_load_dwordx4 {vr(SA + 20, 4)}, %[t], off offset:{HD * 2 + 16}",
+           "s_waitcnt vmcnt(0)"]
+    for j in range(4):
+        rotate_pairs(ins, SA + j, SA + 4 + j, SA + 8 + 2 * j, SA + 16 + 2 * j, SA + 24 + j, SA + 28 + j, TMP)
+    ins += [f"v_mov_b32 %{j}, {vr(SA + 24 + j)}" for j in range(8)]
+    outs = [f'"=v"(lo[{j}])' for j in range(4)] + [f'"=v"(hi[{j}])' for j in range(4)]
+    return f'''// Rotates chunks c and c + 8 (16 bytes each, HD bytes apart) of the head row at `k_chunk` by the angles of
+// the table row at `table_chunk` (the position's row plus 8 c floats): the arithmetic of dfx_rope_kv_store, bit
+// for bit.  Uses score set A; waits for every load of the wave in flight.
+DFX_D void pipe_rope_row(const void* k_chunk, const void* table_chunk, uint32_t (&lo)[4], uint32_t (&hi)[4]) {{
+    asm volatile("{join(ins)}"
+                 : {", ".join(outs)}
+                 : [k] "v"(k_chunk), [t] "v"(table_chunk)
+                 : "memory");
+}}
+
+'''
+
+
 def asm_fn(name, args, body, outs=(), ins=(), clobbers=(), comment=None):
     head = "".join(f"// {line}\n" for line in (comment or "").split("\n") if line)
     ops = f"\n                 : {', '.join(outs)}\n                 : {', '.join(ins)}"
@@ -414,6 +485,8 @@ namespace dfx {
                                 "stage 0) into the widened tiles at wide_k and wide_v (byte offsets from widened tile 0): both reads first,\n"
                                 "one instruction per pair of codes (exact), in the operand ring's registers, which are free between the\n"
                                 "blocks of two steps.  The writes are waited for by whatever waits for LDS next (lgkmcnt)."))
+    parts.append(rope_queries_fns())
+    parts.append(rope_row_fn())
     for d in range(NDB):
         outs = [f'"=v"(x[{e}])' for e in range(16)]
         body = join(f"v_accvgpr_read_b32 %{e}, {ar(O_BASE + 16 * d + e)}" for e in range(16))

@@ -163,7 +163,10 @@ __global__ void __launch_bounds__(kMetaThreads) build_decode_metadata_kernel(con
         // (block diffusion feeds dbs tokens per sequence; for D2F every fed token has a slot entry)
         const int64_t q0 = p.strategy == DFX_META_D2F ? slot_off[s] : static_cast<int64_t>(s) * dbs;
         for (int i = lane; i < m.seq_len; i += 64) {
-            if (q0 + i < p.token_capacity) p.positions[q0 + i] = m.ctx + i;
+            if (q0 + i < p.token_capacity) {
+                p.positions[q0 + i] = m.ctx + i;
+                if (p.input_ids != nullptr) p.input_ids[q0 + i] = p.token_ids[static_cast<int64_t>(s) * p.token_ids_stride + m.ctx + i];
+            }
         }
         const int32_t* table = p.block_tables + static_cast<int64_t>(s) * p.block_table_stride;
         const int64_t o0 = slot_off[s];
@@ -183,7 +186,10 @@ __global__ void __launch_bounds__(kMetaThreads) build_decode_metadata_kernel(con
     }
 
     // the tail of buffers sized for a larger (captured) batch reads as zeros
-    for (int64_t i = total.q + t; i < p.padded_tokens && i < p.token_capacity; i += kMetaThreads) p.positions[i] = 0;
+    for (int64_t i = total.q + t; i < p.padded_tokens && i < p.token_capacity; i += kMetaThreads) {
+        p.positions[i] = 0;
+        if (p.input_ids != nullptr) p.input_ids[i] = 0;
+    }
     for (int64_t i = total.slots + t; i < p.padded_tokens && i < p.token_capacity; i += kMetaThreads)
         p.slot_mapping[i] = 0;
     for (int s = n + t; s < p.padded_seqs; s += kMetaThreads) {
@@ -222,6 +228,7 @@ extern "C" int dfx_build_decode_metadata(const dfx_metadata_params* p, dfx_strea
         if (p->context_lens == nullptr) return DFX_ERR_INVALID_ARG;
     }
     if (p->token_capacity > 0 && (p->positions == nullptr || p->slot_mapping == nullptr)) return DFX_ERR_INVALID_ARG;
+    if ((p->input_ids != nullptr) != (p->token_ids != nullptr) || p->token_ids_stride < 0) return DFX_ERR_INVALID_ARG;
     if (p->num_seqs > 0) {
         if (p->block_state == nullptr || p->block_tables == nullptr) return DFX_ERR_INVALID_ARG;
         if (p->strategy == DFX_META_BLOCK_DIFFUSION) {

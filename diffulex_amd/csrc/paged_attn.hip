@@ -70,7 +70,7 @@ int make_plan(const dfx_attn_params* p, Plan& plan) {
     if (plan.distinct && plan.fp8) return DFX_ERR_UNSUPPORTED;
     plan.stream = !(p->flags & DFX_ATTN_GENERIC_PATH) && !plan.distinct &&
                   (p->k_cache == nullptr || (p->page_size > 0 && p->page_size % 16 == 0)) &&
-                  p->kn_stride_head == p->vn_stride_head;
+                  (p->rope_cos_sin != nullptr ? p->kr_stride_head : p->kn_stride_head) == p->vn_stride_head;
     // head_dim 128, 65..128 rows: the 8-wave pipelined kernels (their waves without rows only fetch) are
     // faster than 4 waves with a compiler-scheduled step, with or without a second workgroup on the
     // compute unit (C4 -7 %, 112 or 128 rows at the C3 shape -18 %).  Fewer rows: the same (64 or 48 rows
@@ -248,6 +248,13 @@ int check_args(const dfx_attn_params* p, Plan& plan, bool& empty) {
     }
     if (!(p->scale > 0.0f) || p->diffusion_block_size <= 0) return DFX_ERR_INVALID_ARG;
     if (p->mask_mode != DFX_MASK_FULL && p->mask_mode != DFX_MASK_BLOCK_CAUSAL) return DFX_ERR_INVALID_ARG;
+    if (p->rope_cos_sin != nullptr) {
+        if (!plan.pipelined || !has_cache) return DFX_ERR_UNSUPPORTED;
+        if (!p->rope_positions || !p->k_rotated || p->rope_max_position <= 0 || p->k_rotated == p->k_new) return DFX_ERR_INVALID_ARG;
+        if (p->rope_position_index_type != DFX_INDEX_I32 && p->rope_position_index_type != DFX_INDEX_I64) return DFX_ERR_INVALID_ARG;
+        if (p->kr_stride_token < 0 || p->kr_stride_token % 8 || p->kr_stride_head < 0 || p->kr_stride_head % 8) return DFX_ERR_INVALID_ARG;
+        if (!aligned16(p->rope_cos_sin) || !aligned16(p->k_rotated)) return DFX_ERR_INVALID_ARG;
+    }
     const int64_t strides8[] = {p->q_stride_token,  p->q_stride_head,   p->kn_stride_token, p->kn_stride_head,
                                 p->vn_stride_token, p->vn_stride_head};
     for (int64_t v : strides8)
@@ -286,7 +293,9 @@ uint32_t plan_signature(const dfx_attn_params* p, const Plan& plan) {
     mix(plan.hd); mix(plan.nb); mix(plan.n_wg); mix(plan.fp8); mix(plan.stream); mix(plan.compact);
     mix(p->num_seqs); mix(p->num_q_heads); mix(p->num_kv_heads); mix(p->page_size); mix(p->max_pages_per_seq);
     mix(p->max_seqlen_q); mix(p->num_new_tokens); mix(p->diffusion_block_size); mix(p->mask_mode); mix(p->max_workgroups);
-    mix(p->kn_stride_token); mix(p->kn_stride_head); mix(p->vn_stride_token); mix(p->cache_stride_page); mix(p->cache_stride_token);
+    // (the fresh K rows the tiles are made of: with the rotary embedding inside the launch, the rotated copy)
+    const bool rope = p->rope_cos_sin != nullptr;
+    mix(rope ? p->kr_stride_token : p->kn_stride_token); mix(rope ? p->kr_stride_head : p->kn_stride_head); mix(p->vn_stride_token); mix(p->cache_stride_page); mix(p->cache_stride_token);
     mix(p->cache_stride_head); mix(p->block_table_stride); mix(p->n_pages); mix(p->k_cache != nullptr);
     mix(reinterpret_cast<uintptr_t>(p->block_tables)); mix(reinterpret_cast<uintptr_t>(p->context_lens));
     mix(reinterpret_cast<uintptr_t>(p->cu_seqlens_q)); mix(reinterpret_cast<uintptr_t>(p->cu_seqlens_new));
@@ -386,7 +395,22 @@ int run_paged_attn(const dfx_attn_params* p, void* workspace, int64_t workspace_
     ka.c = p->scale * kLog2e;
     ka.n_new = p->num_new_tokens > 0 ? p->num_new_tokens : INT64_MAX;
     ka.n_q = p->num_q_tokens > 0 ? p->num_q_tokens : INT32_MAX;
-    ka.v_fresh_delta = (p->vn_stride_token - p->kn_stride_token) * 2;
+    ka.rope_table = p->rope_cos_sin;
+    ka.rope_pos = p->rope_positions;
+    ka.rope_pos_i64 = p->rope_position_index_type == DFX_INDEX_I64;
+    ka.rope_max_pos = p->rope_max_position;
+    ka.k_src = nullptr;
+    ka.ks_st = ka.ks_sh = 0;
+    if (p->rope_cos_sin != nullptr) {
+        // the tiles of fresh K rows are read from where the launch puts the rotated rows
+        ka.k_src = ka.k_new;
+        ka.ks_st = ka.kn_st;
+        ka.ks_sh = ka.kn_sh;
+        ka.k_new = static_cast<const uint16_t*>(p->k_rotated);
+        ka.kn_st = p->kr_stride_token;
+        ka.kn_sh = p->kr_stride_head;
+    }
+    ka.v_fresh_delta = (p->vn_stride_token - ka.kn_st) * 2;
     ka.plan = nullptr;
     ka.plan_capacity = 0;
     ka.plan_signature = plan_signature(p, plan);

@@ -53,15 +53,17 @@ const float* scale_ptr(const OptTensor& s, int n_heads, const char* name) {
         const OptTensor &out, const OptTensor &block_tables, const OptTensor &context_lens, const Tensor &cu_q,    \
         const Tensor &cu_new, const OptTensor &k_scale, const OptTensor &v_scale, const OptTensor &store_slots,    \
         const OptTensor &plan, double scale, int64_t max_seqlen_q, int64_t mask_mode, int64_t dbs, int64_t max_wg, \
-        int64_t flags, int64_t cache_layout
+        int64_t flags, int64_t cache_layout, const OptTensor &rope_cos_sin, const OptTensor &rope_positions,       \
+        const OptTensor &k_rotated
 #define DFX_ATTN_PASS                                                                                              \
     q, k, v, k_cache, v_cache, out, block_tables, context_lens, cu_q, cu_new, k_scale, v_scale, store_slots, plan, \
-        scale, max_seqlen_q, mask_mode, dbs, max_wg, flags, cache_layout
+        scale, max_seqlen_q, mask_mode, dbs, max_wg, flags, cache_layout, rope_cos_sin, rope_positions, k_rotated
 #define DFX_ATTN_SCHEMA                                                                                            \
     "Tensor q, Tensor k, Tensor v, Tensor(a!)? k_cache, Tensor(b!)? v_cache, Tensor(c!)? out, Tensor? block_tables, "          \
     "Tensor? context_lens, Tensor cu_seqlens_q, Tensor cu_seqlens_new, Tensor? k_scale, Tensor? v_scale, "         \
     "Tensor? store_slot_mapping, Tensor? plan, float scale, int max_seqlen_q, int mask_mode, "                     \
-    "int diffusion_block_size, int max_workgroups, int flags, int cache_layout"
+    "int diffusion_block_size, int max_workgroups, int flags, int cache_layout, Tensor? rope_cos_sin, "            \
+    "Tensor? rope_positions, Tensor(e!)? k_rotated"
 
 dfx_attn_params attn_params(DFX_ATTN_ARGS) {
     TORCH_CHECK(q.is_cuda() && q.scalar_type() == at::kBFloat16 && k.scalar_type() == at::kBFloat16 &&
@@ -150,6 +152,24 @@ dfx_attn_params attn_params(DFX_ATTN_ARGS) {
     p.head_dim = static_cast<int32_t>(hd);
     p.num_new_tokens = k.size(0);
     p.num_q_tokens = static_cast<int32_t>(q.size(0));
+    if (has(rope_cos_sin)) {
+        TORCH_CHECK(rope_cos_sin->is_cuda() && rope_cos_sin->scalar_type() == at::kFloat && rope_cos_sin->is_contiguous() &&
+                        rope_cos_sin->dim() == 2 && rope_cos_sin->size(1) == hd,
+                    "rope_cos_sin: contiguous fp32 [max_position, head_dim]");
+        TORCH_CHECK(has(rope_positions) && rope_positions->is_cuda() && rope_positions->is_contiguous() &&
+                        rope_positions->numel() == q.size(0) && q.size(0) == k.size(0),
+                    "rope_positions: one position per token, the same tokens in q and k");
+        TORCH_CHECK(has(k_rotated) && k_rotated->is_cuda() && k_rotated->scalar_type() == at::kBFloat16 &&
+                        k_rotated->sizes() == k.sizes() && k_rotated->stride(2) == 1,
+                    "k_rotated: a bf16 device tensor shaped like k");
+        p.rope_cos_sin = static_cast<const float*>(rope_cos_sin->data_ptr());
+        p.rope_positions = rope_positions->data_ptr();
+        p.rope_position_index_type = index_type(*rope_positions, "rope_positions");
+        p.rope_max_position = rope_cos_sin->size(0);
+        p.k_rotated = k_rotated->data_ptr();
+        p.kr_stride_token = k_rotated->stride(0);
+        p.kr_stride_head = k_rotated->stride(1);
+    }
     p.max_seqlen_q = static_cast<int32_t>(max_seqlen_q);
     p.diffusion_block_size = static_cast<int32_t>(dbs);
     p.mask_mode = static_cast<int32_t>(mask_mode);
@@ -375,7 +395,8 @@ void build_decode_metadata(int64_t strategy, const Tensor& block_tables, const T
                            int64_t dbs, const OptTensor& num_tokens, const OptTensor& num_pages,
                            const OptTensor& prompt_len, const OptTensor& num_diffusion_blocks, Tensor positions,
                            Tensor slot_mapping, Tensor cu_q, Tensor cu_k, Tensor context_lens, Tensor seq_lens,
-                           Tensor summary, int64_t token_capacity, int64_t padded_seqs, int64_t padded_tokens) {
+                           Tensor summary, int64_t token_capacity, int64_t padded_seqs, int64_t padded_tokens,
+                           const OptTensor& token_ids, const OptTensor& input_ids) {
     const int64_t n = block_tables.size(0);
     const int64_t rows = std::max(n, padded_seqs);
     TORCH_CHECK(block_tables.is_cuda() && block_tables.scalar_type() == at::kInt && block_tables.dim() == 2 &&
@@ -423,6 +444,18 @@ void build_decode_metadata(int64_t strategy, const Tensor& block_tables, const T
     p.padded_seqs = static_cast<int32_t>(padded_seqs);
     p.padded_tokens = padded_tokens;
     p.summary = static_cast<int32_t*>(summary.data_ptr());
+    TORCH_CHECK(has(token_ids) == has(input_ids), "token_ids and input_ids go together");
+    if (has(token_ids)) {
+        TORCH_CHECK(token_ids->is_cuda() && token_ids->scalar_type() == at::kLong && token_ids->dim() == 2 &&
+                        token_ids->size(0) == n && token_ids->stride(1) == 1,
+                    "token_ids: int64 [num_seqs, max_len] with dense rows");
+        TORCH_CHECK(input_ids->is_cuda() && input_ids->scalar_type() == at::kLong && input_ids->is_contiguous() &&
+                        input_ids->numel() >= token_capacity,
+                    "input_ids: int64 [token_capacity]");
+        p.token_ids = static_cast<const int64_t*>(token_ids->data_ptr());
+        p.token_ids_stride = token_ids->stride(0);
+        p.input_ids = static_cast<int64_t*>(input_ids->data_ptr());
+    }
     check(dfx_build_decode_metadata(&p, current_stream()), "dfx_build_decode_metadata");
 }
 
@@ -447,7 +480,7 @@ TORCH_LIBRARY(diffulex_amd, m) {
           "int diffusion_block_size, Tensor? num_tokens, Tensor? num_pages, Tensor? prompt_len, "
           "Tensor? num_diffusion_blocks, Tensor(a!) positions, Tensor(b!) slot_mapping, Tensor(c!) cu_seqlens_q, "
           "Tensor(d!) cu_seqlens_k, Tensor(e!) context_lens, Tensor(f!) seq_lens, Tensor(g!) summary, int token_capacity, int padded_seqs, "
-          "int padded_tokens) -> ()");
+          "int padded_tokens, Tensor? token_ids, Tensor(h!)? input_ids) -> ()");
 }
 
 // The kernels exist for the GPU only: the operators are registered for device tensors and nothing else.

@@ -61,7 +61,7 @@ def paged_attention(q, k, v, k_cache, v_cache, scale, *, block_tables, context_l
                     cu_seqlens_new, max_seqlen_q, mask_mode=_lib.DFX_MASK_FULL, diffusion_block_size=32,
                     k_scale=None, v_scale=None, max_workgroups=0, out=None, flags=0,
                     store_slot_mapping=None, static_scratch=False, plan_cache=None,
-                    cache_layout="unified") -> torch.Tensor:
+                    cache_layout="unified", rope=None, k_rotated=None) -> torch.Tensor:
     """Launch ``dfx_paged_attn`` on the current stream through ``torch.ops.diffulex_amd.paged_attention``
     (which checks the tensors and fills ``dfx_attn_params``).  q: [T, H_q, hd]; k, v: [T_new, H_kv, hd];
     caches [pages, page, H_kv, hd] or None.  ``store_slot_mapping`` ([T_new] int32/int64): the same
@@ -77,7 +77,12 @@ def paged_attention(q, k, v, k_cache, v_cache, scale, *, block_tables, context_l
     change the cache key); a caller that rewrites them behind PyTorch's back, or rewrites tensors made
     under ``torch.inference_mode()`` (which carry no version counter) in place, drops the dict.
     ``cache_layout="distinct"``: k_cache [pages, H_kv, hd / 8, page, 8], v_cache [pages, H_kv, hd,
-    page] (what ``store_kvcache_distinct_layout`` writes); bf16, generic tile path, no fused store."""
+    page] (what ``store_kvcache_distinct_layout`` writes); bf16, generic tile path, no fused store.
+    ``rope=(cos_sin_cache, positions)``: q and k are the projections BEFORE the rotary embedding, which the
+    launch applies itself (``dfx_attn_params.rope_cos_sin``): query rows on their way into the matrix
+    instructions, fresh key rows into ``k_rotated`` (a new [T_new, H_kv, hd] tensor by default) and, with
+    ``store_slot_mapping``, into the cache.  Raises ``DfxError`` (unsupported shape) where the pipelined
+    kernels do not run; ``rope_supported()`` tells beforehand."""
     ops = _lib.ops()
     T, H_q, hd = q.shape
     H_kv = k.shape[1]
@@ -103,6 +108,14 @@ def paged_attention(q, k, v, k_cache, v_cache, scale, *, block_tables, context_l
             int(flags), layout)
     head = (q, k, v, k_cache, v_cache, out, block_tables, context_lens, cu_seqlens_q, cu_seqlens_new, ks, vs,
             store_slot_mapping)
+    if rope is not None:
+        table, positions = rope
+        positions = positions.reshape(-1)
+        if k_rotated is None:
+            k_rotated = torch.empty((k.shape[0], H_kv, hd), dtype=k.dtype, device=k.device)
+        tail = tail + (table, positions if positions.is_contiguous() else positions.contiguous(), k_rotated)
+    else:
+        tail = tail + (None, None, None)
     plan = None
     if plan_cache is not None and has_cache and not distinct:
         # A plan is only as good as the lengths and tables it was made from: see plan_key().
@@ -118,7 +131,8 @@ def paged_attention(q, k, v, k_cache, v_cache, scale, *, block_tables, context_l
             return out
         # (what dfx_paged_attn_workspace_bytes looks at: the shapes, the flags, whether k and v share
         # their head stride -- which decides the tile path -- and the device's compute-unit count)
-        shape_key = (q.device.index, num_seqs, H_q, H_kv, hd, tail[1:], has_cache, fp8, k.stride(1) == v.stride(1),
+        k_eff = k_rotated if rope is not None else k
+        shape_key = (q.device.index, num_seqs, H_q, H_kv, hd, tail[1:7], has_cache, fp8, k_eff.stride(1) == v.stride(1),
                      k_cache.shape[1] if has_cache and not distinct else 0)
         need = _workspace_need.get(shape_key)
         if need is None:
@@ -146,7 +160,8 @@ def plan_key(q, k, k_cache, fp8, tail, meta, capture_id):
     """Cache key of a launch plan: everything ``dfx_paged_attn_plan`` depends on (shapes, strides, the
     metadata tensors and their contents as far as ``_content_token`` sees them) and the graph capture
     the call is recorded into (a plan built outside that capture is not part of its graph)."""
-    return (q.shape[1], k.shape[1], q.shape[2], bool(fp8), tail[1:], k.stride(0), k.stride(1), k_cache.stride()[:3],
+    k_eff = tail[9] if tail[7] is not None else k   # (with the rotary embedding in the launch the tiles come from k_rotated)
+    return (q.shape[1], k.shape[1], q.shape[2], bool(fp8), tail[1:7], k_eff.stride(0), k_eff.stride(1), k_cache.stride()[:3],
             meta[2].numel() - 1, tuple(_content_token(t) for t in meta), int(capture_id))
 
 
@@ -209,11 +224,12 @@ def dllm_flash_attn_decode(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, k_
                            k_scale: Optional[torch.Tensor] = None,
                            v_scale: Optional[torch.Tensor] = None,
                            store_slot_mapping: Optional[torch.Tensor] = None,
-                           kv_cache_layout: str = "unified") -> torch.Tensor:
+                           kv_cache_layout: str = "unified", rope=None) -> torch.Tensor:
     """dllm_flash_attn.py:599-637.  ``store_slot_mapping`` (extension): also store the fresh
     K/V rows into these cache slots in the same launch (see ``paged_attention``).
     ``kv_cache_layout="distinct"`` (extension): the caches are in the layout
-    ``store_kvcache_distinct_layout`` writes.
+    ``store_kvcache_distinct_layout`` writes.  ``rope=(cos_sin_cache, positions)`` (extension): q and k
+    are the projections before the rotary embedding, which the launch applies (see ``paged_attention``).
 
     ``decode_mode == "static"``: ``cu_seqlens_k`` indexes the fresh K/V rows
     (strategy/block_diffusion/engine/model_runner.py:134-139).
@@ -248,4 +264,16 @@ def dllm_flash_attn_decode(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, k_
         cu_seqlens_new=cu_new, max_seqlen_q=_max_seqlen_q(attn_metadata, attn_metadata.cu_seqlens_q),
         mask_mode=mask, diffusion_block_size=attn_metadata.diffusion_block_size,
         k_scale=k_scale, v_scale=v_scale, store_slot_mapping=store_slot_mapping,
-        plan_cache=_plan_cache_of(attn_metadata))
+        plan_cache=_plan_cache_of(attn_metadata), rope=rope)
+
+
+def rope_supported(num_heads: int, num_kv_heads: int, head_dim: int, max_seqlen_q: int, page_size: int, num_seqs: int,
+                   device=None) -> bool:
+    """Whether ``dfx_paged_attn`` can apply the rotary embedding itself for this shape (the
+    software-pipelined kernels: head_dim 128, page size a multiple of 16, more than 64 query rows per KV
+    head and sequence or at most two (sequence, KV head) items per compute unit)."""
+    if head_dim != 128 or page_size % 16 != 0 or num_heads % num_kv_heads != 0:
+        return False
+    rows = num_heads // num_kv_heads * max_seqlen_q
+    cus = torch.cuda.get_device_properties(device if device is not None else torch.cuda.current_device()).multi_processor_count
+    return rows > 64 or num_seqs * num_kv_heads <= 2 * cus

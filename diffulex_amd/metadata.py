@@ -61,7 +61,8 @@ def build_decode_metadata(strategy: str, *, block_tables: torch.Tensor, block_st
                           num_pages: Optional[torch.Tensor] = None, prompt_len: Optional[torch.Tensor] = None,
                           num_diffusion_blocks: Optional[torch.Tensor] = None, token_capacity: int,
                           padded_seqs: int = 0, padded_tokens: int = 0, out: Optional[dict] = None,
-                          kv_cache_layout: str = "unified", sync_summary: bool = False) -> "PagedAttnMetaData":
+                          kv_cache_layout: str = "unified", sync_summary: bool = False,
+                          token_ids: Optional[torch.Tensor] = None) -> "PagedAttnMetaData":
     """The metadata of one decode step from per-sequence state kept on the device
     (``dfx_build_decode_metadata``): what ``prepare_decode`` of the reference's runners computes
     in Python loops and copies over (block_diffusion/engine/model_runner.py:114-173,
@@ -75,6 +76,10 @@ def build_decode_metadata(strategy: str, *, block_tables: torch.Tensor, block_st
     buffers a graph was captured on, padded to ``padded_seqs`` / ``padded_tokens``; by default new
     tensors are made.  Nothing is read back unless ``sync_summary`` is set: ``max_seqlen_q`` is then
     the true maximum, otherwise an upper bound from the shapes (enough for the attention operators).
+    ``token_ids`` (int64 [B, max_len], the sequences' tokens kept on the device): the step's
+    ``input_ids`` -- every fed token's id, the concatenation of ``cur_input_ids`` in the reference's
+    loops -- are gathered in the same launch and attached as ``md.input_ids`` (``out["input_ids"]``
+    if given).
     Returns the metadata object with ``positions`` and ``summary`` attached as attributes."""
     from . import _lib
     from .kv_cache_kernels import _call
@@ -91,10 +96,13 @@ def build_decode_metadata(strategy: str, *, block_tables: torch.Tensor, block_st
     o.setdefault("context_lens", torch.empty(rows, **i32))
     o.setdefault("seq_lens", torch.empty(rows, **i32))
     o.setdefault("summary", torch.empty(8, **i32))
+    if token_ids is not None:
+        o.setdefault("input_ids", torch.empty(cap, dtype=torch.int64, device=dev))
     code = {"block_diffusion": _lib.DFX_META_BLOCK_DIFFUSION, "d2f": _lib.DFX_META_D2F}[strategy]
     _call(_lib.ops().build_decode_metadata, code, block_tables, block_state, int(page_size), int(diffusion_block_size),
           num_tokens, num_pages, prompt_len, num_diffusion_blocks, o["positions"], o["slot_mapping"], o["cu_seqlens_q"],
-          o["cu_seqlens_k"], o["context_lens"], o["seq_lens"], o["summary"], cap, int(padded_seqs), int(padded_tokens))
+          o["cu_seqlens_k"], o["context_lens"], o["seq_lens"], o["summary"], cap, int(padded_seqs), int(padded_tokens),
+          token_ids, o["input_ids"] if token_ids is not None else None)
     d2f = strategy == "d2f"
     n_tokens = cap
     max_q = max_k = 0
@@ -119,6 +127,7 @@ def build_decode_metadata(strategy: str, *, block_tables: torch.Tensor, block_st
         decode_mode="varlen" if d2f else "static", seq_lens_ts=o["seq_lens"][:rows] if d2f else None,
         kv_cache_layout=kv_cache_layout, need_kv_cache_store=need_store)
     md.positions = o["positions"][:n_tokens]
+    md.input_ids = o["input_ids"][:n_tokens] if token_ids is not None else None
     md.summary = o["summary"]
     return md
 

@@ -216,6 +216,27 @@ typedef struct dfx_attn_params {
     int32_t num_q_tokens;
     int64_t kc_stride[5];
     int64_t vc_stride[4];
+    /* Rotary position embedding inside the launch (NULL table: off; q and k_new are then used as they are).
+     * Replaces: RotaryEmbedding.forward on the Q and K projections right before the attention layer
+     *           (diffulex/model/dream.py:94-99, diffulex/layer/rotary_embedding.py:39-66), the launch
+     *           dfx_rope_kv_store otherwise does.
+     * q and k_new hold the projections as they leave the linear layer.  Row t of q and row t of k_new / v_new
+     * are the same token (cu_seqlens_new equals cu_seqlens_q), at position rope_positions[t]; rope_cos_sin is
+     * the table of dfx_rope_kv_store ([rope_max_position, head_dim] fp32: cosines, then sines).  The query rows
+     * are rotated on their way into the matrix instructions and never written; the rotated fresh K rows go to
+     * k_rotated ([T_new, num_kv_heads, head_dim] bf16, its own strides, NOT k_new itself: rows may be rotated
+     * by more than one workgroup), which the launch reads back, and, with store_slot_mapping, into the cache
+     * (FP8 caches: quantised after the rounding to bf16) next to the V rows.  Same bits as dfx_rope_kv_store
+     * followed by this call without rope.  Only where the software-pipelined kernels run (head_dim 128, page
+     * size a multiple of 16, more than 64 query rows per KV head and sequence or few items per compute unit,
+     * a cache present): DFX_ERR_UNSUPPORTED otherwise -- run dfx_rope_kv_store first then. */
+    const float* rope_cos_sin;
+    const void* rope_positions;
+    int32_t rope_position_index_type; /* dfx_index_type */
+    int32_t reserved2;
+    int64_t rope_max_position;
+    void* k_rotated;
+    int64_t kr_stride_token, kr_stride_head;
 } dfx_attn_params;
 
 /* Bytes of scratch dfx_paged_attn needs for these shapes.  It depends on the sizes (num_seqs, heads,
@@ -304,7 +325,8 @@ int dfx_paged_attn_plan(const dfx_attn_params* params, void* plan, int64_t plan_
  *     fed tokens; a token to be cached at position g of the sequence gets slot
  *     block_tables[s][g / page_size] * page_size + g % page_size, every token from the first active
  *     block on gets -1.
- * positions[i] (int64) = position in its sequence of the i-th fed token.
+ * positions[i] (int64) = position in its sequence of the i-th fed token; input_ids[i] (optional) = the
+ * token the sequence holds there.
  *
  * padded_seqs / padded_tokens (0: none): the output arrays are the buffers of a captured graph of
  * that batch size; entries beyond the step's own are set to 0, as the reference's run_model leaves
@@ -348,6 +370,15 @@ typedef struct dfx_metadata_params {
     int32_t reserved;
     int64_t padded_tokens;
     int32_t* summary; /* [8] */
+    /* The step's token ids (both NULL: not wanted).  token_ids: the sequences' tokens as the scheduler
+     * keeps them on the device, int64 [num_seqs, token_ids_stride], row s holding at least
+     * len(sequence s) entries; input_ids [token_capacity] receives, for every fed token, the token at
+     * its position of its sequence (the concatenation of cur_input_ids in the reference's loops:
+     * block_diffusion/engine/model_runner.py:126-130, d2f/engine/model_runner.py:153-158), padded
+     * with zeros up to padded_tokens. */
+    const int64_t* token_ids;
+    int64_t token_ids_stride;
+    int64_t* input_ids;
 } dfx_metadata_params;
 
 int dfx_build_decode_metadata(const dfx_metadata_params* params, dfx_stream_t stream);

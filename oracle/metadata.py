@@ -129,6 +129,23 @@ def d2f_prepare_decode(prompt_len, states, block_tables, page_size, dbs, last_bl
                 max_seqlen_q=max_q, max_seqlen_k=max_k, need_kv_cache_store=need_store)
 
 
+def input_ids_of(meta, token_ids):
+    """The step's ``input_ids``: the reference concatenates every sequence's ``cur_input_ids``
+    (block_diffusion/engine/model_runner.py:126-130 with ``active_block_token_ids``, sequence.py:186-191;
+    d2f/engine/model_runner.py:153-158 with the ``token_ids`` of every block behind the cached ones,
+    sequence.py:369-382), which are the sequence's tokens at the positions the step feeds.
+    ``token_ids[s]``: the token list of sequence s."""
+    out = []
+    pos = meta["positions"].tolist()
+    lens = meta["seq_lens"].tolist()
+    i = 0
+    for s, n in enumerate(lens):
+        for p in pos[i:i + n]:
+            out.append(int(token_ids[s][p]))
+        i += n
+    return np.asarray(out, np.int64)
+
+
 def check_slot_mapping(states, dbs, slot_mapping):
     """The layout ``CHECK_SLOT_MAPPING`` demands of a D2F slot mapping: per sequence, ``dbs``
     real slots for every block to be cached, then -1 from the first active block to the end."""

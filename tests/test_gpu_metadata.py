@@ -50,12 +50,15 @@ def test_block_diffusion_metadata_bits(dev, n_seqs, page, dbs):
     n_tokens, state, tables = _bd_batch(rng, n_seqs, page, dbs)
     want = om.bd_prepare_decode(n_tokens, state, tables, page, dbs)
     width = max(len(t) for t in tables) + 1
+    toks = [rng.integers(0, 150000, n).tolist() for n in n_tokens]
     md = build_decode_metadata(
         "block_diffusion", block_tables=_dev(_padded(tables, width, -1), dev), block_state=_dev(state, dev, torch.uint8),
         page_size=page, diffusion_block_size=dbs, num_tokens=_dev(n_tokens, dev),
-        num_pages=_dev([len(t) for t in tables], dev), token_capacity=n_seqs * dbs)
+        num_pages=_dev([len(t) for t in tables], dev), token_capacity=n_seqs * dbs,
+        token_ids=_dev(_padded(toks, max(n_tokens) + 3, -7, np.int64), dev, torch.int64))
     _check(md, want, n_seqs)
     assert md.decode_mode == "static" and md.max_seqlen_q == dbs
+    assert np.array_equal(md.input_ids.cpu().numpy(), om.input_ids_of(want, toks))
 
 
 @pytest.mark.parametrize("n_seqs,page,dbs,short", [(1, 32, 32, False), (6, 16, 32, True), (64, 32, 32, False),
@@ -67,12 +70,15 @@ def test_d2f_metadata_bits(dev, n_seqs, page, dbs, short):
     if not short:
         assert om.check_slot_mapping(states, dbs, want["slot_mapping"].tolist()) == len(want["slot_mapping"])
     totals = [p + (len(st) - 2) * dbs + l for p, st, l in zip(prompt, states, last)]
+    toks = [rng.integers(0, 150000, n).tolist() for n in totals]
     md = build_decode_metadata(
         "d2f", block_tables=_dev(_padded(tables, max(len(t) for t in tables), -1), dev),
         block_state=_dev(_padded(states, 8, 3, np.uint8), dev, torch.uint8), page_size=page, diffusion_block_size=dbs,
         prompt_len=_dev(prompt, dev), num_diffusion_blocks=_dev([len(s) for s in states], dev),
-        num_tokens=_dev(totals, dev) if short else None, token_capacity=n_seqs * 6 * dbs, sync_summary=True)
+        num_tokens=_dev(totals, dev) if short else None, token_capacity=n_seqs * 6 * dbs, sync_summary=True,
+        token_ids=_dev(_padded(toks, max(totals), -7, np.int64), dev, torch.int64))
     _check(md, want, n_seqs)
+    assert np.array_equal(md.input_ids.cpu().numpy(), om.input_ids_of(want, toks))
     assert np.array_equal(md.seq_lens_ts[:n_seqs].cpu().numpy(), want["seq_lens"])
     assert md.max_seqlen_q == want["max_seqlen_q"] and md.need_kv_cache_store == want["need_kv_cache_store"]
 
@@ -89,14 +95,18 @@ def test_graph_buffers_zero_padded_as_the_reference_leaves_them(dev):
                 slot_mapping=torch.full((padded_seqs * dbs,), 77, **i32),
                 cu_seqlens_q=torch.full((padded_seqs + 1,), 77, **i32), cu_seqlens_k=torch.full((padded_seqs + 1,), 77, **i32),
                 context_lens=torch.full((padded_seqs,), 77, **i32), seq_lens=torch.full((padded_seqs,), 77, **i32),
-                summary=torch.zeros(8, **i32))
+                summary=torch.zeros(8, **i32), input_ids=torch.full((padded_seqs * dbs,), 77, dtype=torch.int64, device=dev))
+    toks = [rng.integers(1, 150000, n).tolist() for n in n_tokens]
     build_decode_metadata(
         "block_diffusion", block_tables=_dev(_padded(tables, 48, 0), dev), block_state=_dev(state, dev, torch.uint8),
         page_size=page, diffusion_block_size=dbs, num_tokens=_dev(n_tokens, dev),
         num_pages=_dev([len(t) for t in tables], dev), token_capacity=padded_seqs * dbs,
-        padded_seqs=padded_seqs, padded_tokens=padded_seqs * dbs, out=bufs)
+        padded_seqs=padded_seqs, padded_tokens=padded_seqs * dbs, out=bufs,
+        token_ids=_dev(_padded(toks, max(n_tokens), 0, np.int64), dev, torch.int64))
     for name in ("positions", "cu_seqlens_q", "cu_seqlens_k", "context_lens"):
         assert np.array_equal(bufs[name].cpu().numpy(), want[name]), name
+    ids = om.input_ids_of(om.bd_prepare_decode(n_tokens, state, tables, page, dbs), toks)
+    assert np.array_equal(bufs["input_ids"].cpu().numpy(), np.concatenate([ids, np.zeros(padded_seqs * dbs - len(ids), np.int64)]))
     # a block that is neither active nor to be cached adds no slot entries: compare what was produced
     n_slot = int(bufs["summary"][1])
     assert np.array_equal(bufs["slot_mapping"].cpu().numpy(), want["slot_mapping"]) and n_slot <= n_seqs * dbs

@@ -144,3 +144,20 @@ def test_graph_buffers_are_zero_filled_behind_the_step():
     g = om.pad_for_graph(m, padded_seqs=4, padded_tokens=128)
     assert g["cu_seqlens_q"].tolist() == [0, 32, 64, 0, 0] and g["context_lens"].tolist() == [32, 64, 0, 0]
     assert g["slot_mapping"][64:].tolist() == [0] * 64 and g["positions"][:64].tolist() == m["positions"].tolist()
+
+
+def test_input_ids_are_the_sequences_tokens_at_the_fed_positions():
+    """Hand-worked: the block-diffusion step feeds the last block of every sequence, the D2F step every
+    block behind the cached ones; their token ids are the sequences' own at those positions."""
+    toks = [list(range(1000, 1096)), list(range(2000, 2064))]
+    m = om.bd_prepare_decode(num_tokens=[96, 64], last_state=[TO, ACT], block_tables=[[5, 2, 9], [3, 8]], page_size=32, dbs=32)
+    assert om.input_ids_of(m, toks).tolist() == list(range(1064, 1096)) + list(range(2032, 2064))
+    d = om.d2f_prepare_decode(prompt_len=[40, 10], states=[[IN, TO, ACT], [IN, ACT, ACT]], block_tables=[[6, 3, 11, 2], [9, 4, 5]],
+                              page_size=32, dbs=32)
+    toks = [list(range(5000, 5104)), list(range(7000, 7074))]
+    assert om.input_ids_of(d, toks).tolist() == list(range(5040, 5104)) + list(range(7010, 7074))
+    # with distinct random ids: position p of sequence s gives exactly token_ids[s][p]
+    rng = np.random.default_rng(3)
+    toks = [rng.integers(0, 50000, 104).tolist(), rng.integers(0, 50000, 74).tolist()]
+    got = om.input_ids_of(d, toks)
+    assert got.tolist() == toks[0][40:104] + toks[1][10:74]

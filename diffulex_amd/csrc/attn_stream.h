@@ -512,15 +512,15 @@ struct StreamAttn : TileMath<HD, NB, NW, HIDDEN> {
         request_rope_angles(rope_query_position(d));
         pipe_rope_queries();
     }
-    // The fresh K rows of sequence sq, KV head kv_head: rotated from k_src into k_new and, with the fused
+    // The fresh K rows of one sequence, KV head kv_head: rotated from k_src into k_new and, with the fused
     // store, into their cache slots together with the V rows (what dfx_rope_kv_store does in a launch of its
     // own, bit for bit).  All threads of the workgroup; a lane takes a pair of 16-byte chunks (c, c + 8) of
     // a row.  Several workgroups (the row tiles of one sequence and head) may do the same rows: they write
     // the same bytes.
+    // The rows are n0 .. n1 - 1 of k_src / k_new / v_new.
     template <bool FP8>
-    DFX_D void rope_fresh_rows(int sq, int kv_head) const {
+    DFX_D void rope_fresh_rows(int64_t n0, int64_t n1, int kv_head) const {
         static_assert(HIDDEN && HD == 128, "pipelined kernels");
-        const int64_t n0 = min(static_cast<int64_t>(a.cu_new[sq]), a.n_new), n1 = min(static_cast<int64_t>(a.cu_new[sq + 1]), a.n_new);
         const int64_t n_slots = a.n_pages * a.page_size;
         for (int64_t idx = thread_number_here(wave_s); idx < (n1 - n0) * 8; idx += C::THREADS) {
             const int64_t t = n0 + (idx >> 3);
@@ -577,7 +577,10 @@ struct StreamAttn : TileMath<HD, NB, NW, HIDDEN> {
             while (m != 0) {
                 const int r = w * 64 + __builtin_ctzll(m);
                 m &= m - 1;
-                rope_fresh_rows<FP8>(uniform(units[r].s), uniform(units[r].kvh));
+                // (the sequence's fresh rows from the descriptors: the first band of a fresh tile names its first row,
+                // the unit the tile's place among the fresh rows and their number -- no trip to the offsets array)
+                const int64_t n0 = -1 - static_cast<int64_t>(uniform(bands[r * NW].is_ctx)) - uniform(units[r].base);
+                rope_fresh_rows<FP8>(n0, n0 + uniform(units[r].limit), uniform(units[r].kvh));
                 any = true;
             }
         }

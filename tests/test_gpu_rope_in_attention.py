@@ -39,6 +39,8 @@ def test_rope_inside_the_launch_gives_the_bits_of_rope_then_attention(dev, name,
     qkv = torch.randn(T, (hq + 2 * hkv) * hd, generator=g).to(torch.bfloat16).to(dev)
     q, k, v = (x.view(T, -1, hd) for x in qkv.split([hq * hd, hkv * hd, hkv * hd], dim=-1))
     pos = torch.randint(0, MAXPOS, (T,), generator=g).to(dev)
+    if max_wg:  # (the cases with a workgroup limit also take the positions as int32)
+        pos = pos.to(torch.int32)
     rope = RotaryEmbedding(hd, hd, MAXPOS, BASE).to(dev)
     kw = dict(block_tables=wl.block_tables, context_lens=wl.context_lens, cu_seqlens_q=wl.cu_seqlens_q,
               cu_seqlens_new=wl.cu_seqlens_q, max_seqlen_q=wl.q_len, mask_mode=wl.mask_mode,
@@ -63,8 +65,8 @@ def test_rope_inside_the_launch_gives_the_bits_of_rope_then_attention(dev, name,
     # and against the oracle: rotary embedding, then fp32 attention
     tab = orot.cos_sin_cache(hd, MAXPOS, BASE)
     c = wl.to("cpu")
-    c.q = orot.apply_rotary(q.reshape(T, -1).cpu(), pos.cpu(), tab, hd).view(T, hq, hd)
-    c.k_new = orot.apply_rotary(k.reshape(T, -1).cpu(), pos.cpu(), tab, hd).view(T, hkv, hd)
+    c.q = orot.apply_rotary(q.reshape(T, -1).cpu(), pos.cpu().long(), tab, hd).view(T, hq, hd)
+    c.k_new = orot.apply_rotary(k.reshape(T, -1).cpu(), pos.cpu().long(), tab, hd).view(T, hkv, hd)
     c.v_new = v.cpu().contiguous()
     assert max_abs_err(got, oracle_fp32(c)) <= (ATOL_FP8 if wl.kv_fp8 else ATOL_BF16)
 

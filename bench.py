@@ -548,6 +548,9 @@ def main():
     ap.add_argument("--page", type=int, default=0,
                     help="tokens per KV-cache page for the attention workloads (default: the workload's 256; the "
                          "reference's default kvcache_block_size is 32, diffulex/config.py:41)")
+    ap.add_argument("--layout", default="unified", choices=["unified", "distinct"],
+                    help="KV-cache layout of the attention workloads (bf16 ones): the reference's kv_cache_layout "
+                         "(diffulex/config.py:43-44); 'distinct' is K [pages, H, hd/8, page, 8], V [pages, H, hd, page]")
     ap.add_argument("--copies", type=int, default=4, help="independent KV-cache copies rotated between steps")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -601,6 +604,13 @@ def main():
     kw = dict(block_tables=wl.block_tables, context_lens=wl.context_lens, cu_seqlens_q=wl.cu_seqlens_q,
               cu_seqlens_new=wl.cu_seqlens_q, max_seqlen_q=wl.q_len, mask_mode=wl.mask_mode,
               diffusion_block_size=wl.diffusion_block_size, k_scale=wl.k_scale, v_scale=wl.v_scale)
+    if args.layout == "distinct":
+        if wl.kv_fp8:
+            sys.exit("the distinct layout holds bf16")
+        pages, page, h, hd = wl.k_cache.shape
+        sets = [(q, kn, vn, out, kc.view(pages, page, h, hd // 8, 8).permute(0, 2, 3, 1, 4).contiguous(),
+                 vc.permute(0, 2, 3, 1).contiguous()) for q, kn, vn, out, kc, vc in sets]
+        kw["cache_layout"] = "distinct"
     plans = {"cache": {}}
 
     def step_reused_plan(i):
@@ -634,9 +644,10 @@ def main():
     nbytes, nflops = algorithmic_bytes(wl), algorithmic_flops(wl)
     gbs = nbytes / (ms * 1e-3) / 1e9
     tflops = nflops / (ms * 1e-3) / 1e12
-    traffic, traffic_source = measured_traffic(args.workload, nbytes) if args.page <= 0 else (None, None)
+    traffic, traffic_source = measured_traffic(args.workload, nbytes) if args.page <= 0 and args.layout == "unified" else (None, None)
     kernel = ("paged_attn_pipe_fp8_kernel<8>" if wl.kv_fp8 else
-              "paged_attn_pipe_kernel<8, false>")
+              "paged_attn_pipe_kernel<8, false>" if args.layout == "unified" else
+              "paged_attn_stream_kernel<128, 1, 8, false, true>")
     result = {
         "metric": "attn query-tokens/sec + achieved HBM GB/s (% of peak), Dream-7B shape, 1 GPU",
         "value": wl.total_q_tokens / (ms * 1e-3), "unit": "query-tokens/s",
@@ -648,7 +659,8 @@ def main():
                         f"H_kv={wl.num_kv_heads}, head_dim={wl.head_dim}, page={wl.page_size}, "
                         f"ctx in [{int(wl.context_lens.min())},{int(wl.context_lens.max())}] "
                         f"(sum {int(wl.context_lens.sum())}), q_len={wl.q_len}, "
-                        f"mask={'block-causal' if wl.mask_mode else 'full'}, kv={'fp8-e4m3' if wl.kv_fp8 else 'bf16'}",
+                        f"mask={'block-causal' if wl.mask_mode else 'full'}, kv={'fp8-e4m3' if wl.kv_fp8 else 'bf16'}"
+                        + (", distinct cache layout" if args.layout == "distinct" else ""),
             "plan": f"built once per {LAYERS_PER_DECODE_STEP} launches inside the timed region (one decoding step's layers)",
             "ms_per_step_plan_per_launch": ms_per_call,
             "ms_per_step_no_plan": ms_no_plan,

@@ -250,7 +250,10 @@ struct AttnState {
     // rescales o when a row maximum grows.  pb[qb][tb][sl] is the B operand of the PV product.
     // before_rescale() runs ahead of any vector-ALU access to o (kernels that issue their matrix
     // instructions behind the compiler's back insert the required wait states there).
-    template <bool SCALE_P, int HOLE_ROWS, typename BeforeRescale>
+    // NATURAL: the key rows went into S^T = K Q^T with quads 1 and 2 of every 16 swapped (scores_chunk_major),
+    // so that a lane's registers hold the scores of tokens 8 * half .. 8 * half + 7 of a 16-token slab, in
+    // order -- the order of a d-major V row; holes then come a tile at a time (any bit set: all of it).
+    template <bool SCALE_P, int HOLE_ROWS, bool NATURAL = false, typename BeforeRescale>
     DFX_D void softmax_tile(f32x16 (&sc)[2][NB], const TileInfo& t, bf16x8 (&pb)[NB][2][2],
                             BeforeRescale&& before_rescale) {
         const bool mask_valid = t.base + S::TN > t.limit;
@@ -267,9 +270,10 @@ struct AttnState {
                 for (int tb = 0; tb < 2; ++tb)
 #pragma unroll
                     for (int e = 0; e < 16; ++e) {
-                        const int in_tile = tb * 32 + (e >> 2) * 8 + (e & 3);
-                        const int tok = t.base + in_tile + half * 4;
-                        if (tok >= lim || ((holes >> (in_tile / HOLE_ROWS)) & 1)) sc[tb][qb][e] = -INFINITY;
+                        const int in_tile = NATURAL ? tb * 32 + (e >> 3) * 16 + ((e >> 2) & 1) * 4 + (e & 3) : tb * 32 + (e >> 2) * 8 + (e & 3);
+                        const int tok = t.base + in_tile + half * (NATURAL ? 8 : 4);
+                        const bool hole = NATURAL ? holes != 0 : ((holes >> (in_tile / HOLE_ROWS)) & 1) != 0;
+                        if (tok >= lim || hole) sc[tb][qb][e] = -INFINITY;
                     }
             }
         }

@@ -147,14 +147,12 @@ struct GenericAttn : TileMath<HD, NB, kWaves> {
         }
     }
 
-    // The V tile stays d-major in LDS, as it is in the distinct layout: row d holds the tile's 64
-    // tokens (128 bytes, eight 16-byte chunks), which is the V^T operand's shape already.  Inside
-    // a 16-token slab the matrix instruction's contraction index runs over tokens 0-3, 8-11 (lower
-    // half of the wave) and 4-7, 12-15 (upper half), as the score registers hold them; the two
-    // chunks of a slab are stored in that order, so that a lane's operand is one 16-byte read:
-    // chunk 2 * slab + h = tokens 4h..4h+3 then 8+4h..8+4h+3 of the slab.  Chunks are swizzled by
-    // (d / 2) % 8: 16 consecutive d of one chunk column then cover all 64 banks once.
-    DFX_HD static int vt_chunk_offset(int d, int chunk) { return d * (C::TN * 2) + ((chunk ^ ((d >> 1) & 7)) * 16); }
+    // The V tile stays d-major in LDS (TileMath::vt_chunk_offset, accumulate_dmajor).  This kernel feeds
+    // the key rows to S^T in their own order, so inside a 16-token slab the matrix instruction's
+    // contraction index runs over tokens 0-3, 8-11 (lower half of the wave) and 4-7, 12-15 (upper half),
+    // as the score registers hold them; the two chunks of a slab are stored in that order, so that a
+    // lane's operand is one 16-byte read: chunk 2 * slab + h = tokens 4h..4h+3 then 8+4h..8+4h+3 of the slab.
+    using Base::vt_chunk_offset;
     // byte offset of token `tok` (0..63) of row d
     DFX_HD static int vt_token_offset(int d, int tok) {
         const int r16 = tok & 15;
@@ -174,34 +172,6 @@ struct GenericAttn : TileMath<HD, NB, kWaves> {
             *reinterpret_cast<u32x2*>(vs + vt_token_offset(d, tg * 8)) = lo;
             *reinterpret_cast<u32x2*>(vs + vt_token_offset(d, tg * 8 + 4)) = hi;
         }
-    }
-
-    // O^T += V^T P^T from a d-major V tile (commit_distinct): the operand of (token slab tb, sl; d
-    // block db) is one 16-byte read per lane, row db * 32 + col, chunk tb * 4 + sl * 2 + half.
-    DFX_D void accumulate_dmajor(const uint8_t* v_tile, const bf16x8 (&pb)[NB][2][2]) {
-        using S = typename Base::S;
-        typedef __attribute__((address_space(3))) bf16x8 lds_bf16x8;
-        constexpr int kSteps = 4 * S::NDB;  // (tb, sl, db)
-        // Row db * 32 + col, chunk (tb * 4 + sl * 2 + half) ^ swizzle: the swizzle depends on col only and
-        // tb * 4 + sl * 2 is even, so the lane's part of the address is one constant, the slab an XOR
-        // on bits 5..6 of the finished address (tiles start at multiples of 256) and the d block an
-        // immediate offset -- four address registers instead of one per operand.
-        const uint32_t v0 = Base::lds_address(v_tile) + static_cast<uint32_t>(vt_chunk_offset(col, half));
-        auto read = [&](int st) {
-            const int tb = st / (2 * S::NDB), sl = (st / S::NDB) & 1, db = st % S::NDB;
-            return *(const lds_bf16x8*)static_cast<uintptr_t>((v0 ^ ((tb * 4 + sl * 2) * 16)) + db * 32 * (C::TN * 2));
-        };
-        bf16x8 va[3];
-        va[0] = read(0);
-        va[1] = read(1);
-#pragma unroll
-        for (int st = 0; st < kSteps; ++st) {
-            const int tb = st / (2 * S::NDB), sl = (st / S::NDB) & 1, db = st % S::NDB;
-            if (st + 2 < kSteps) va[(st + 2) % 3] = read(st + 2);
-#pragma unroll
-            for (int qb = 0; qb < NB; ++qb) mfma_output(o[db][qb], va[st % 3], pb[qb][tb][sl]);
-        }
-        this->outputs_ready();
     }
 
     // global -> registers (rows past the end of the sequence become zeros)
@@ -323,7 +293,7 @@ struct GenericAttn : TileMath<HD, NB, kWaves> {
         this->scores(k_stage(buf), sc);
         bf16x8 pb[NB][2][2];
         this->template softmax_tile<FP8, 1>(sc, t, pb, [&] { this->outputs_ready(); });
-        if constexpr (DISTINCT) accumulate_dmajor(v_stage(buf), pb);  // (one form for every tile: two, chosen at run time, would
+        if constexpr (DISTINCT) this->accumulate_dmajor(v_stage(buf), pb);  // (one form for every tile: two, chosen at run time, would
         else this->accumulate(v_stage(buf), pb);                      //  have the accumulators copied where the paths meet)
     }
 

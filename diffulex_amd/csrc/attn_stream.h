@@ -164,8 +164,17 @@ DFX_D void wait_async_loads() {
     asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
 }
 
-template <int HD, int NB, int NW, bool COMPACT = false, int KVB = 2, bool HIDDEN = false>
+// DISTINCT: the cache is in the distinct layout (K [pages, H, HD / 8, page, 8], V [pages, H, HD, page]; pages of
+// a multiple of 64 tokens, so that a tile lies in one page).  A stage then holds the K tile chunk-major and the
+// V tile d-major (attn_tile.h), both filled by the same direct-to-LDS loads: a wave takes two chunk columns of K
+// (1 KiB contiguous each) and 16 rows of V^T (128 contiguous bytes each).  The descriptors are per tile, the
+// same for every wave: BandDesc::off = page << 20 | first token's place in the page, BandDesc::last = the
+// tile's last valid token.  Fresh rows, row-major in memory: K is gathered into the chunk-major tile by the
+// loads themselves (a lane per token), V lands row-major and is transposed inside LDS before its step
+// (transpose_fresh_v).
+template <int HD, int NB, int NW, bool COMPACT = false, int KVB = 2, bool HIDDEN = false, bool DISTINCT = false>
 struct StreamAttn : TileMath<HD, NB, NW, HIDDEN> {
+    static_assert(!DISTINCT || (KVB == 2 && !HIDDEN && !COMPACT && NW == 8 && HD == 128), "distinct layout: bf16, 8 waves, head_dim 128");
     using Base = TileMath<HD, NB, NW, HIDDEN>;
     using C = StreamCfg<HD, NB, NW, COMPACT, KVB>;
     using L = TileLayout<HD>;
@@ -260,7 +269,20 @@ struct StreamAttn : TileMath<HD, NB, NW, HIDDEN> {
             if (past_end) band = ((limit - 1) / C::ROWS_PER_WAVE) * C::ROWS_PER_WAVE;
             BandDesc b;
             bool hole = false;  // the band's page has no valid block-table entry: its tokens are skipped
-            if (is_ctx) {
+            if constexpr (DISTINCT) {
+                // one descriptor per tile, repeated for every wave
+                if (is_ctx) {
+                    const int p = a.page_shift >= 0 ? (base >> a.page_shift) : (base / a.page_size);
+                    int64_t page = p < a.max_pages ? a.block_tables[static_cast<int64_t>(sq) * a.bt_stride + p] : -1;
+                    hole = page < 0 || page >= a.n_pages;
+                    page = page < 0 ? 0 : (page >= a.n_pages ? a.n_pages - 1 : page);
+                    b.off = (page << 20) | static_cast<int64_t>(base - p * a.page_size);
+                } else {
+                    b.off = ((static_cast<int64_t>(a.cu_new[sq]) + base) * a.kn_st + kv_head * a.kn_sh) * 2;
+                }
+                b.last = limit - 1 - base;
+                b.is_ctx = is_ctx ? 1 : -(1 + a.cu_new[sq] + base);
+            } else if (is_ctx) {
                 const int p = a.page_shift >= 0 ? (band >> a.page_shift) : (band / a.page_size);
                 int64_t page = p < a.max_pages ? a.block_tables[static_cast<int64_t>(sq) * a.bt_stride + p] : -1;
                 hole = !past_end && (page < 0 || page >= a.n_pages);
@@ -269,8 +291,10 @@ struct StreamAttn : TileMath<HD, NB, NW, HIDDEN> {
             } else {
                 b.off = ((static_cast<int64_t>(a.cu_new[sq]) + band) * a.kn_st + kv_head * a.kn_sh) * 2;
             }
-            b.last = limit - 1 - band;
-            b.is_ctx = is_ctx ? 1 : -(1 + a.cu_new[sq] + band);
+            if constexpr (!DISTINCT) {
+                b.last = limit - 1 - band;
+                b.is_ctx = is_ctx ? 1 : -(1 + a.cu_new[sq] + band);
+            }
             bands[slot_in_ring * NW + w] = b;
             // the NW lanes of a unit are neighbours in a wave: its holes as a bit per band
             const uint64_t votes = __ballot(hole);
@@ -289,6 +313,47 @@ struct StreamAttn : TileMath<HD, NB, NW, HIDDEN> {
         const bool is_ctx = tag > 0;
         const int64_t off = (static_cast<int64_t>(uniform(static_cast<int>(b.off >> 32))) << 32) |
                             static_cast<uint32_t>(uniform(static_cast<int>(b.off)));
+        if constexpr (DISTINCT) {
+            const uint32_t dst = stages_lds + (static_cast<unsigned>(rel) % C::kStages) * C::STAGE_BYTES;
+            const int kvh = uniform(units[rel].kvh);
+            const uint32_t tok = static_cast<uint32_t>(min(lane, last));  // tokens past the end re-read the last valid one
+            if (is_ctx) {
+                const int64_t page = off >> 20;
+                const int64_t in_page = off & 0xfffff;
+                const uint8_t* kb = a.k_cache + (page * a.kd_sp + kvh * a.kd_sh + in_page * 8) * 2;
+                const uint8_t* vb = a.v_cache + (page * a.vd_sp + kvh * a.vd_sh + in_page) * 2;
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    const int c = wave_s * 2 + j;  // chunk column: a lane per token
+                    async_load16(kb + static_cast<int64_t>(c) * a.kd_sc * 2, tok * 16, dst + c * Base::CHUNK_COL_BYTES);
+                }
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    // 8 rows of V^T: 8 lanes per row, the chunk at position p of row d holds tokens 8 * (p ^ swizzle(d)) ..;
+                    // chunks past the end re-read the last one with a valid token (clear_v_tail zeroes what is not)
+                    const int d = wave * 16 + j * 8 + (lane >> 3);
+                    const int tc = min((lane & 7) ^ ((d >> 1) & 7), last >> 3);
+                    async_load16(vb, static_cast<uint32_t>(d) * static_cast<uint32_t>(a.vd_sd * 2) + tc * 16,
+                                 dst + C::MAT_BYTES + (wave * 16 + j * 8) * (C::TN * 2));
+                }
+            } else {
+                const uint8_t* kb = reinterpret_cast<const uint8_t*>(a.k_new) + off;
+                const uint8_t* vb = reinterpret_cast<const uint8_t*>(a.v_new) + off + static_cast<int64_t>(-1 - tag) * a.v_fresh_delta;
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    const int c = wave_s * 2 + j;
+                    async_load16(kb + c * 16, tok * static_cast<uint32_t>(a.kn_st * 2), dst + c * Base::CHUNK_COL_BYTES);
+                }
+#pragma unroll
+                for (int j = 0; j < C::IPW; ++j) {  // row-major, as a unified-layout stage holds it
+                    const int r = wave * C::ROWS_PER_WAVE + j * C::RPI + lane / C::CPR;
+                    const int chunk = (lane % C::CPR) ^ C::swizzle(r);
+                    async_load16(vb, static_cast<uint32_t>(min(r, last)) * static_cast<uint32_t>(a.vn_st * 2) + chunk * 16,
+                                 dst + C::MAT_BYTES + wave * (C::IPW * 1024) + j * 1024);
+                }
+            }
+            return;
+        }
         if constexpr (HIDDEN && NW == 8 && KVB == 2) {
             // the common case, a full band of cached rows: offsets precomputed per lane, no vector arithmetic
             if (is_ctx && last >= C::ROWS_PER_WAVE - 1) {
@@ -585,6 +650,60 @@ struct StreamAttn : TileMath<HD, NB, NW, HIDDEN> {
             }
         }
         return any;
+    }
+
+    // ---- distinct layout: what the loads cannot do ---------------------------------------------------
+    // The V half of the stage of a fresh tile holds the rows as they lie in memory (row-major, swizzled as a
+    // unified-layout tile); the step reads d-major.  Transposed in place through registers: every thread
+    // takes two 16-byte chunks (8 values of one token), all read, barrier, all write two bytes at a time.
+    // Every thread of the workgroup; the tile has landed (barrier behind the wait); ends with a barrier.
+    DFX_D void transpose_fresh_v(int rel) const {
+        static_assert(!DISTINCT || C::THREADS * 2 == C::TN * L::CPR, "two chunks per thread");
+        uint8_t* vt = lds + C::STAGES_OFF + (static_cast<unsigned>(rel) % C::kStages) * C::STAGE_BYTES + C::MAT_BYTES;
+        const int t = thread_number_here(wave_s);
+        u32x4 x[2];
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const int idx = t + C::THREADS * i;
+            x[i] = *reinterpret_cast<const u32x4*>(vt + L::chunk_offset(idx / L::CPR, idx % L::CPR));
+        }
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const int idx = t + C::THREADS * i;
+            const int row = idx / L::CPR, cc = idx % L::CPR;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const uint32_t w = x[i][j >> 1];
+                *reinterpret_cast<uint16_t*>(vt + Base::vt_chunk_offset(cc * 8 + j, row >> 3) + (row & 7) * 2) =
+                    static_cast<uint16_t>((j & 1) ? (w >> 16) : w);
+            }
+        }
+        __syncthreads();
+    }
+    // A tile of cached rows that ends before its 64th token: the V^T rows hold whatever the page holds behind
+    // the sequence's end (the chunk with the last valid token) or copies of that chunk (the ones after it), and
+    // a probability of zero does not make a NaN or an infinity harmless.  Zeroes the tokens from n_valid on.
+    // Every thread of the workgroup; the tile has landed; ends with a barrier.
+    DFX_D void clear_v_tail(int rel, int n_valid) const {
+        uint8_t* vt = lds + C::STAGES_OFF + (static_cast<unsigned>(rel) % C::kStages) * C::STAGE_BYTES + C::MAT_BYTES;
+        const int t = thread_number_here(wave_s);
+#pragma unroll
+        for (int i = 0; i < HD * 8 / C::THREADS; ++i) {
+            const int idx = t + C::THREADS * i;
+            const int d = idx >> 3, tc = idx & 7;
+            const int keep = n_valid - tc * 8;  // tokens of this chunk to keep
+            if (keep >= 8) continue;
+            u32x4* p = reinterpret_cast<u32x4*>(vt + Base::vt_chunk_offset(d, tc));
+            u32x4 v = {0, 0, 0, 0};
+            if (keep > 0) {
+                v = *p;
+#pragma unroll
+                for (int k = 0; k < 4; ++k) v[k] &= (2 * k < keep ? 0x0000ffffu : 0u) | (2 * k + 1 < keep ? 0xffff0000u : 0u);
+            }
+            *p = v;
+        }
+        __syncthreads();
     }
 
     // First key position the lane's query row does not see under the block-causal mask (fresh tiles
@@ -938,14 +1057,14 @@ struct StreamAttn : TileMath<HD, NB, NW, HIDDEN> {
     }
 };
 
-template <int HD, int NB, int NW, bool COMPACT>
+template <int HD, int NB, int NW, bool COMPACT, bool DISTINCT = false>
 __global__ void __launch_bounds__(64 * NW, COMPACT ? 2 : 1) paged_attn_stream_kernel(const KArgs a) {
     extern __shared__ __attribute__((aligned(256))) uint8_t smem[];
     using C = StreamCfg<HD, NB, NW, COMPACT>;
-    StreamAttn<HD, NB, NW, COMPACT> at(a, smem);
+    StreamAttn<HD, NB, NW, COMPACT, 2, false, DISTINCT> at(a, smem);
     // The fused cache store comes first, while next to nothing is live in registers: anywhere
     // later its address arithmetic would push values of the tile loop out of their registers.
-    store_fresh_rows<HD, false>(a);
+    if constexpr (!DISTINCT) store_fresh_rows<HD, false>(a);
     at.for_each_chunk([&](int n_units) {
         const WgSplit& split = at.split;
         // An item that opens with this plan: its query rows are requested ahead of the ring fill,
@@ -979,12 +1098,23 @@ __global__ void __launch_bounds__(64 * NW, COMPACT ? 2 : 1) paged_attn_stream_ke
                 t.c_tile = a.c;
                 t.v_mul = 1.0f;
                 const uint8_t* k_tile = smem + C::STAGES_OFF + (static_cast<unsigned>(rel) % C::kStages) * C::STAGE_BYTES;
+                if constexpr (DISTINCT) {  // (once or twice per item)
+                    if (!t.is_ctx) at.transpose_fresh_v(rel);
+                    else if (t.holes != 0) at.clear_v_tail(rel, 0);  // (a page without a table entry: page 0 was read in its place)
+                    else if (t.base + C::TN > t.limit) at.clear_v_tail(rel, t.limit - t.base);
+                }
                 if (at.wave < a.busy_waves) {  // waves whose 32 rows exist in no item of this launch only fetch
                     f32x16 sc[2][NB];
-                    at.scores(k_tile, sc);
                     bf16x8 pb[NB][2][2];
-                    at.template softmax_tile<false, C::ROWS_PER_WAVE>(sc, t, pb, [&] { at.outputs_ready(); });
-                    at.accumulate(k_tile + C::MAT_BYTES, pb);
+                    if constexpr (DISTINCT) {
+                        at.scores_chunk_major(k_tile, sc);
+                        at.template softmax_tile<false, C::ROWS_PER_WAVE, true>(sc, t, pb, [&] { at.outputs_ready(); });
+                        at.accumulate_dmajor(k_tile + C::MAT_BYTES, pb);
+                    } else {
+                        at.scores(k_tile, sc);
+                        at.template softmax_tile<false, C::ROWS_PER_WAVE>(sc, t, pb, [&] { at.outputs_ready(); });
+                        at.accumulate(k_tile + C::MAT_BYTES, pb);
+                    }
                 } else {
                     at.outputs_untouched();
                 }

@@ -230,6 +230,75 @@ struct TileMath : AttnState<HD, NB, NW, HIDDEN> {
         outputs_ready();
     }
 
+    // ---- tiles of a cache in the distinct layout ------------------------------------------------
+    // K [pages, H, HD / 8, page, 8]: 64 consecutive tokens of one chunk column are 1 KiB contiguous, and that
+    // is how the tile lies in LDS: chunk-major, [HD / 8 chunk columns][64 tokens][16 bytes].  The operand of
+    // (token block tb, slab) is chunk column 2 * slab + half, 32 consecutive tokens: 16 lanes read 256
+    // contiguous bytes, no swizzle needed.  The lane that feeds matrix row r reads token swap_quads(r): with
+    // quads 1 and 2 of every 16 rows swapped the score registers of a lane hold 8 consecutive tokens
+    // (softmax_tile<.., NATURAL>), which is the order a d-major V row holds them in.
+    DFX_HD static int swap_quads(int r) { return (r & ~12) | ((r & 4) << 1) | ((r & 8) >> 1); }
+    static constexpr int CHUNK_COL_BYTES = kTileTokens * 16;
+    DFX_D void scores_chunk_major(const uint8_t* k_tile, f32x16 (&sc)[2][NB]) const {
+        typedef __attribute__((address_space(3))) bf16x8 lds_bf16x8;
+        const uint32_t k0 = lds_address(k_tile) + static_cast<uint32_t>(half * CHUNK_COL_BYTES + swap_quads(col) * 16);
+        auto read = [&](int slab, int tb) {
+            return *(const lds_bf16x8*)static_cast<uintptr_t>(k0 + slab * 2 * CHUNK_COL_BYTES + tb * 32 * 16);
+        };
+        bf16x8 ka[2][2];
+#pragma unroll
+        for (int tb = 0; tb < 2; ++tb) ka[0][tb] = read(0, tb);
+#pragma unroll
+        for (int slab = 0; slab < S::NSLAB; ++slab) {
+            if (slab + 1 < S::NSLAB) {
+#pragma unroll
+                for (int tb = 0; tb < 2; ++tb) ka[(slab + 1) & 1][tb] = read(slab + 1, tb);
+            }
+#pragma unroll
+            for (int tb = 0; tb < 2; ++tb)
+#pragma unroll
+                for (int qb = 0; qb < NB; ++qb) {
+                    if (slab == 0) mfma_scores_first(sc[tb][qb], ka[slab & 1][tb], qf[qb][slab]);
+                    else mfma_scores(sc[tb][qb], ka[slab & 1][tb], qf[qb][slab]);
+                }
+        }
+        if constexpr (NB == 2) mfma_results_ready(sc[0][0], sc[0][1], sc[1][0], sc[1][1]);
+        else mfma_results_ready(sc[0][0], sc[1][0]);
+    }
+
+    // V [pages, H, HD, page] is d-major, and so is its tile in LDS: row d holds the tile's 64 tokens (128
+    // bytes, eight 16-byte chunks of 8 tokens), which is the V^T operand's shape already.  Chunks are
+    // swizzled by (d / 2) % 8: 16 consecutive d of one chunk column then cover all 64 banks once.
+    DFX_HD static int vt_chunk_offset(int d, int chunk) { return d * (kTileTokens * 2) + ((chunk ^ ((d >> 1) & 7)) * 16); }
+
+    // O^T += V^T P^T from a d-major V tile: the operand of (token slab tb, sl; d block db) is one 16-byte
+    // read per lane, row db * 32 + col, chunk tb * 4 + sl * 2 + half -- the 8 tokens whose probabilities
+    // the lane's half of the wave holds in pb[.][tb][sl], in the same order (the caller's business: the
+    // chunk holds them as its layout says).
+    DFX_D void accumulate_dmajor(const uint8_t* v_tile, const bf16x8 (&pb)[NB][2][2]) {
+        typedef __attribute__((address_space(3))) bf16x8 lds_bf16x8;
+        constexpr int kSteps = 4 * S::NDB;  // (tb, sl, db)
+        // Row db * 32 + col, chunk (tb * 4 + sl * 2 + half) ^ swizzle: the swizzle depends on col only and
+        // tb * 4 + sl * 2 is even, so the lane's part of the address is one constant, the slab an XOR
+        // on bits 5..6 of the finished address (tiles start at multiples of 256) and the d block an
+        // immediate offset -- four address registers instead of one per operand.
+        const uint32_t v0 = lds_address(v_tile) + static_cast<uint32_t>(vt_chunk_offset(col, half));
+        auto read = [&](int st) {
+            const int tb = st / (2 * S::NDB), sl = (st / S::NDB) & 1, db = st % S::NDB;
+            return *(const lds_bf16x8*)static_cast<uintptr_t>((v0 ^ ((tb * 4 + sl * 2) * 16)) + db * 32 * (kTileTokens * 2));
+        };
+        bf16x8 va[3];
+        va[0] = read(0);
+        va[1] = read(1);
+#pragma unroll
+        for (int st = 0; st < kSteps; ++st) {
+            const int tb = st / (2 * S::NDB), sl = (st / S::NDB) & 1, db = st % S::NDB;
+            if (st + 2 < kSteps) va[(st + 2) % 3] = read(st + 2);
+#pragma unroll
+            for (int qb = 0; qb < NB; ++qb) mfma_output(o[db][qb], va[st % 3], pb[qb][tb][sl]);
+        }
+        outputs_ready();
+    }
 };
 
 }  // namespace dfx

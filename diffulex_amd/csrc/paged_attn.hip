@@ -31,7 +31,7 @@ struct Plan {
     int hd, nb, n_wg;
     bool fp8;
     bool stream;   // streaming tile path (else generic)
-    bool distinct; // the cache is in the "distinct" layout (generic path)
+    bool distinct; // the cache is in the "distinct" layout (streaming path where its kernel serves the shape, else generic)
     bool compact;  // streaming path, two workgroups per compute unit
     bool pipelined;  // streaming path, 8 waves, 4-stage ring: software-pipelined tile step
     int64_t slot_floats;
@@ -71,6 +71,16 @@ int make_plan(const dfx_attn_params* p, Plan& plan) {
     plan.stream = !(p->flags & DFX_ATTN_GENERIC_PATH) && !plan.distinct &&
                   (p->k_cache == nullptr || (p->page_size > 0 && p->page_size % 16 == 0)) &&
                   (p->rope_cos_sin != nullptr ? p->kr_stride_head : p->kn_stride_head) == p->vn_stride_head;
+    // The distinct layout on the streaming path: head_dim 128, a tile inside one page, the 16-byte chunks the
+    // loads move (x == 8, tokens dense in V), offsets inside a (page, head) in 32 bits; one kernel, 8 waves.
+    const bool dstream = plan.distinct && !(p->flags & DFX_ATTN_GENERIC_PATH) && plan.hd == 128 && p->page_size > 0 &&
+                         p->page_size % 64 == 0 && p->page_size < (1 << 20) && p->kn_stride_head == p->vn_stride_head &&
+                         p->kc_stride[4] == 1 && p->kc_stride[3] == 8 && p->vc_stride[3] == 1 &&
+                         p->vc_stride[2] >= 0 && p->vc_stride[2] < (1 << 22) && p->rope_cos_sin == nullptr;
+    if (dstream) {
+        plan.stream = true;
+        plan.nb = 2;
+    }
     // head_dim 128, 65..128 rows: the 8-wave pipelined kernels (their waves without rows only fetch) are
     // faster than 4 waves with a compiler-scheduled step, with or without a second workgroup on the
     // compute unit (C4 -7 %, 112 or 128 rows at the C3 shape -18 %).  Fewer rows: the same (64 or 48 rows
@@ -82,9 +92,10 @@ int make_plan(const dfx_attn_params* p, Plan& plan) {
         if (rows > 64 || items <= 2 * static_cast<int64_t>(device_cu_count())) plan.nb = 2;
     }
     plan.compact = plan.stream && !plan.fp8 && plan.nb == 1 && p->num_seqs <= kCompactMaxSeqs;
+    // (the distinct layout's kernel runs the compiler-scheduled step)
     // (8 waves only: with 4 waves a wave has twice the tile loads to address, and the 32 registers
     // the pipelined kernel leaves the compiler no longer hold that without spilling in the loop)
-    plan.pipelined = plan.stream && !plan.compact && plan.hd == 128 && plan.nb == 2 &&
+    plan.pipelined = plan.stream && !plan.compact && plan.hd == 128 && plan.nb == 2 && !plan.distinct &&
                      !(p->flags & DFX_ATTN_NO_PIPELINE);
     if (p->max_workgroups > 0) {
         plan.n_wg = p->max_workgroups;
@@ -111,17 +122,18 @@ int64_t plan_workspace_bytes(const Plan& plan) {
 
 // Raising a kernel's dynamic LDS limit is idempotent but not free: done once per device and kernel.
 bool ensure_lds_limit(const void* kernel, int slot, int lds) {
-    static std::atomic<uint32_t> configured[64];
+    static std::atomic<uint64_t> configured[64];
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return false;
-    const uint32_t bit = 1u << slot;
+    const uint64_t bit = 1ull << slot;
     if (configured[dev].load(std::memory_order_acquire) & bit) return true;
     if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess) return false;
     configured[dev].fetch_or(bit, std::memory_order_release);
     return true;
 }
 
-// PATH: 0 generic bf16, 1 generic FP8, 2 streaming bf16, 3 streaming FP8, 4 generic bf16 on a distinct-layout cache.
+// PATH: 0 generic bf16, 1 generic FP8, 2 streaming bf16, 3 streaming FP8, 4 generic bf16 on a distinct-layout cache,
+// 5 streaming bf16 on a distinct-layout cache.
 // pa == nullptr: the attention launch.  Otherwise the two plan kernels for that launch (streaming
 // paths only).
 template <int HD, int NB, int PATH>
@@ -184,6 +196,17 @@ int launch(const KArgs& ka, const Plan& plan, hipStream_t st, const PlanArgs* pa
             fill_k = paged_attn_plan_fill_kernel<HD, 1, NW, false, 2>;
             fill_lds = C::STAGES_OFF;
         }
+        threads = 64 * NW;
+    } else if constexpr (PATH == 5) {
+        static_assert(HD == 128 && NB == 2, "the distinct layout's streaming kernel");
+        using C = StreamCfg<HD, 1, NW, false>;
+        main_k = paged_attn_stream_kernel<HD, 1, NW, false, true>;
+        slot = 32;
+        lds = C::LDS_BYTES;
+        plan_k = paged_attn_plan_kernel<C::RT>;
+        plan_slot = C::RT == 256 ? 31 : 30;
+        fill_k = paged_attn_plan_fill_kernel<HD, 1, NW, false, 2, true>;
+        fill_lds = C::STAGES_OFF;
         threads = 64 * NW;
     } else if constexpr (PATH == 4) {
         main_k = paged_attn_generic_kernel<HD, NB, false, true>;
@@ -300,6 +323,10 @@ uint32_t plan_signature(const dfx_attn_params* p, const Plan& plan) {
     mix(reinterpret_cast<uintptr_t>(p->block_tables)); mix(reinterpret_cast<uintptr_t>(p->context_lens));
     mix(reinterpret_cast<uintptr_t>(p->cu_seqlens_q)); mix(reinterpret_cast<uintptr_t>(p->cu_seqlens_new));
     mix(static_cast<uint32_t>(p->flags)); mix(plan.pipelined);
+    if (plan.distinct) {
+        mix(1);
+        for (int i = 0; i < 3; ++i) { mix(p->kc_stride[i]); mix(p->vc_stride[i]); }
+    }
     const uint32_t sig = static_cast<uint32_t>(h ^ (h >> 32));
     return sig == 0 ? 1u : sig;
 }
@@ -428,11 +455,12 @@ int run_paged_attn(const dfx_attn_params* p, void* workspace, int64_t workspace_
 #define DFX_ATTN_CASE(HD_, NB_)                                               \
     if (plan.hd == HD_ && plan.nb == NB_) {                                   \
         if (plan.stream && plan.fp8) return launch<HD_, NB_, 3>(ka, plan, st, pap); \
-        if (plan.stream) return launch<HD_, NB_, 2>(ka, plan, st, pap);       \
+        if (plan.stream && !plan.distinct) return launch<HD_, NB_, 2>(ka, plan, st, pap); \
         if (plan.distinct) return launch<HD_, NB_, 4>(ka, plan, st, pap);     \
         if (plan.fp8) return launch<HD_, NB_, 1>(ka, plan, st, pap);          \
         return launch<HD_, NB_, 0>(ka, plan, st, pap);                        \
     }
+    if (plan.stream && plan.distinct) return launch<128, 2, 5>(ka, plan, st, pap);
     DFX_ATTN_CASE(64, 1)
     DFX_ATTN_CASE(64, 2)
     DFX_ATTN_CASE(128, 1)

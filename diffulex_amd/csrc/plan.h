@@ -445,11 +445,11 @@ __global__ void __launch_bounds__(512) paged_attn_plan_kernel(const KArgs a, con
 }
 
 // Phase two, one workgroup per attention workgroup: the unit and band descriptors of its work.
-template <int HD, int NB, int NW, bool COMPACT, int KVB>
+template <int HD, int NB, int NW, bool COMPACT, int KVB, bool DISTINCT = false>
 __global__ void __launch_bounds__(64 * NW) paged_attn_plan_fill_kernel(const KArgs a, const PlanArgs pa) {
     extern __shared__ __attribute__((aligned(256))) uint8_t smem[];
     using C = StreamCfg<HD, NB, NW, COMPACT, KVB>;
-    StreamAttn<HD, NB, NW, COMPACT, KVB> at(a, smem);
+    StreamAttn<HD, NB, NW, COMPACT, KVB, false, DISTINCT> at(a, smem);
     const PlanHeader* hdr = reinterpret_cast<const PlanHeader*>(pa.buf);
     if (hdr->magic != kPlanMagic) return;
     const PlanLayout lay = plan_layout(a.num_seqs, pa.n_wg, pa.capacity, NW);

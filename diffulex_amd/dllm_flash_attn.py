@@ -77,7 +77,8 @@ def paged_attention(q, k, v, k_cache, v_cache, scale, *, block_tables, context_l
     change the cache key); a caller that rewrites them behind PyTorch's back, or rewrites tensors made
     under ``torch.inference_mode()`` (which carry no version counter) in place, drops the dict.
     ``cache_layout="distinct"``: k_cache [pages, H_kv, hd / 8, page, 8], v_cache [pages, H_kv, hd,
-    page] (what ``store_kvcache_distinct_layout`` writes); bf16, generic tile path, no fused store.
+    page] (what ``store_kvcache_distinct_layout`` writes); bf16, no fused store; head_dim 128 with pages of
+    a multiple of 64 tokens streams (and takes a plan), other shapes take the generic tile path.
     ``rope=(cos_sin_cache, positions)``: q and k are the projections BEFORE the rotary embedding, which the
     launch applies itself (``dfx_attn_params.rope_cos_sin``): query rows on their way into the matrix
     instructions, fresh key rows into ``k_rotated`` (a new [T_new, H_kv, hd] tensor by default) and, with
@@ -117,14 +118,15 @@ def paged_attention(q, k, v, k_cache, v_cache, scale, *, block_tables, context_l
     else:
         tail = tail + (None, None, None)
     plan = None
-    if plan_cache is not None and has_cache and not distinct:
+    page_size = (k_cache.shape[3] if distinct else k_cache.shape[1]) if has_cache else 0
+    if plan_cache is not None and has_cache:
         # A plan is only as good as the lengths and tables it was made from: see plan_key().
         key = plan_key(q, k, k_cache, fp8, tail, (block_tables, context_lens, cu_seqlens_q, cu_seqlens_new),
-                       int(ops.stream_capture_id()))
+                       int(ops.stream_capture_id()), v_cache if distinct else None)
         plan = plan_cache.get(key, False)
         if plan is False:
             plan = plan_cache[key] = _build_plan(ops, head, tail, H_q // H_kv, int(max_seqlen_q), num_seqs,
-                                                 block_tables.shape[1], k_cache.shape[1], k.shape[0])
+                                                 block_tables.shape[1], page_size, k.shape[0])
     try:
         if static_scratch:
             ops.paged_attention(*head, plan, *tail, None, True)
@@ -133,7 +135,7 @@ def paged_attention(q, k, v, k_cache, v_cache, scale, *, block_tables, context_l
         # their head stride -- which decides the tile path -- and the device's compute-unit count)
         k_eff = k_rotated if rope is not None else k
         shape_key = (q.device.index, num_seqs, H_q, H_kv, hd, tail[1:7], has_cache, fp8, k_eff.stride(1) == v.stride(1),
-                     k_cache.shape[1] if has_cache and not distinct else 0)
+                     page_size, distinct and (k_cache.stride()[2:], v_cache.stride()[2:]))
         need = _workspace_need.get(shape_key)
         if need is None:
             need = _workspace_need[shape_key] = int(ops.paged_attention_workspace_bytes(*head, None, *tail))
@@ -156,12 +158,14 @@ def _content_token(t: torch.Tensor):
     return (t.data_ptr(), -1 if t.is_inference() else t._version)
 
 
-def plan_key(q, k, k_cache, fp8, tail, meta, capture_id):
+def plan_key(q, k, k_cache, fp8, tail, meta, capture_id, v_cache=None):
     """Cache key of a launch plan: everything ``dfx_paged_attn_plan`` depends on (shapes, strides, the
     metadata tensors and their contents as far as ``_content_token`` sees them) and the graph capture
     the call is recorded into (a plan built outside that capture is not part of its graph)."""
     k_eff = tail[9] if tail[7] is not None else k   # (with the rotary embedding in the launch the tiles come from k_rotated)
-    return (q.shape[1], k.shape[1], q.shape[2], bool(fp8), tail[1:7], k_eff.stride(0), k_eff.stride(1), k_cache.stride()[:3],
+    # (v_cache: the distinct layout, whose two caches have strides of their own; its page size is a dimension)
+    cache = k_cache.stride()[:3] if v_cache is None else (k_cache.stride(), v_cache.stride(), k_cache.shape[3])
+    return (q.shape[1], k.shape[1], q.shape[2], bool(fp8), tail[1:7], k_eff.stride(0), k_eff.stride(1), cache,
             meta[2].numel() - 1, tuple(_content_token(t) for t in meta), int(capture_id))
 
 
@@ -254,7 +258,8 @@ def dllm_flash_attn_decode(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, k_
             q, k, v, k_cache, v_cache, scale, block_tables=attn_metadata.block_tables,
             context_lens=attn_metadata.context_lens, cu_seqlens_q=attn_metadata.cu_seqlens_q,
             cu_seqlens_new=cu_new, max_seqlen_q=_max_seqlen_q(attn_metadata, attn_metadata.cu_seqlens_q),
-            mask_mode=mask, diffusion_block_size=attn_metadata.diffusion_block_size, cache_layout="distinct")
+            mask_mode=mask, diffusion_block_size=attn_metadata.diffusion_block_size, cache_layout="distinct",
+            plan_cache=_plan_cache_of(attn_metadata))
     if k_cache.dtype in _FP8_DTYPES:
         k_scale = k_scale if k_scale is not None else getattr(attn_metadata, "k_scale", None)
         v_scale = v_scale if v_scale is not None else getattr(attn_metadata, "v_scale", None)

@@ -208,8 +208,12 @@ typedef struct dfx_attn_params {
      * strides below (kc_stride[3] == 8, kc_stride[4] == 1, vc_stride[3] == 1, the others multiples of
      * 8; page_size a multiple of 8).  The reference stores into this layout
      * (diffulex_kernel/python/kv_cache_kernels.py:35-83) but its decode refuses it
-     * (diffulex/attention/attn_impl.py:66-69); here it runs on the generic tile path.  No fused store,
-     * no FP8, no plan with it. */
+     * (diffulex/attention/attn_impl.py:66-69); here it is decoded.  head_dim 128 with pages of a multiple
+     * of 64 tokens (fresh K and V with one head stride, vc_stride[2] below 2^22) streams -- the K tile
+     * chunk-major and the V tile d-major in LDS, as the layout has them -- and takes a plan; other shapes,
+     * and DFX_ATTN_GENERIC_PATH, run the generic tile path, which takes none.  No fused store, no FP8, no
+     * rotary embedding inside the launch with it.  What a page holds behind a sequence's end is never
+     * used, whatever it is. */
     int32_t cache_layout;
     /* Rows of q and out.  No row at or beyond it is read or written, whatever cu_seqlens_q (or a plan
      * built from an earlier state of it) says.  0: unknown, the offsets are trusted. */

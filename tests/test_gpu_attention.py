@@ -295,11 +295,80 @@ def test_decode_on_the_distinct_cache_layout(dev, name, over, max_wg):
     args = dict(block_tables=g.block_tables, context_lens=g.context_lens, cu_seqlens_q=g.cu_seqlens_q,
                 cu_seqlens_new=g.cu_seqlens_q, max_seqlen_q=g.q_len, mask_mode=g.mask_mode,
                 diffusion_block_size=g.diffusion_block_size, max_workgroups=max_wg)
-    got = dfx.paged_attention(g.q, g.k_new, g.v_new, kd, vd, g.scale, cache_layout="distinct", **args)
+    got = dfx.paged_attention(g.q, g.k_new, g.v_new, kd, vd, g.scale, cache_layout="distinct", flags=GENERIC, **args)
     same = dfx.paged_attention(g.q, g.k_new, g.v_new, g.k_cache, g.v_cache, g.scale, flags=GENERIC, **args)
+    # (without the flag: head_dim 128 with pages of a multiple of 64 tokens streams, other shapes run the same kernel)
+    dflt = dfx.paged_attention(g.q, g.k_new, g.v_new, kd, vd, g.scale, cache_layout="distinct", **args)
     torch.cuda.synchronize()
     assert max_abs_err(got, want) <= ATOL_BF16
     assert torch.equal(got, same)
+    assert max_abs_err(dflt, want) <= ATOL_BF16
+
+
+STREAMED_DISTINCT = [
+    ("c3", dict(num_seqs=6, ctx=(300, 1500)), 0),                                  # Dream heads, 256-token pages, cut items
+    ("c3", dict(num_seqs=5, ctx=[0, 1, 7, 64, 129], page=64), 0),                  # no context, a context inside one chunk of 8 tokens
+    ("c3", dict(num_seqs=4, ctx=[63, 65, 200, 511], page=128), 5),                 # tile and page ends, five workgroups
+    ("c3", dict(num_seqs=3, ctx=[700, 513, 1000]), 3),
+    ("c4", dict(num_seqs=3, ctx=(100, 700)), 0),                                   # 96 fresh rows: two fresh tiles, block-causal
+    ("c4", dict(num_seqs=2, ctx=(100, 300), h_q=8, h_kv=2, q_len=128, dbs=32), 7), # several row tiles per sequence and head
+    ("c3", dict(num_seqs=9, ctx=(30, 400), h_q=8, h_kv=8, q_len=32, page=64), 0),  # 32 rows per item: most waves only fetch
+]
+
+
+@pytest.mark.parametrize("name,over,max_wg", STREAMED_DISTINCT)
+@pytest.mark.parametrize("planned", [False, True])
+def test_distinct_layout_on_the_streaming_path(dev, name, over, max_wg, planned):
+    """head_dim 128 and pages of a multiple of 64 tokens: the distinct layout streams (K tile chunk-major, V tile
+    d-major, the layout's own shapes).  Against the oracle, and against the generic kernel on the same cache; what
+    lies in a page behind a sequence's end (NaN here, in K and in V) must not reach the result, nor must a page
+    without a table entry."""
+    wl = make_workload(name, seed=97, **over)
+    bt = wl.block_tables.clone()
+    if wl.num_seqs > 2 and int(wl.context_lens[2]) > wl.page_size:
+        bt[2, 1] = -1
+        wl.block_tables = bt
+    want = oracle_fp32(wl)
+    g = wl.to(dev)
+    kc, vc = g.k_cache.clone(), g.v_cache.clone()
+    for s in range(g.num_seqs):   # poison the rest of the page that holds the sequence's end
+        ctx = int(g.context_lens[s])
+        p, used = divmod(ctx, g.page_size)
+        if used and int(g.block_tables[s, p]) >= 0:
+            kc[int(g.block_tables[s, p]), used:] = float("nan")
+            vc[int(g.block_tables[s, p]), used:] = float("nan")
+    kd, vd = _to_distinct(kc)[0], _to_distinct(vc)[1]
+    args = dict(block_tables=g.block_tables, context_lens=g.context_lens, cu_seqlens_q=g.cu_seqlens_q,
+                cu_seqlens_new=g.cu_seqlens_q, max_seqlen_q=g.q_len, mask_mode=g.mask_mode,
+                diffusion_block_size=g.diffusion_block_size, max_workgroups=max_wg)
+    cache = {} if planned else None
+    got = dfx.paged_attention(g.q, g.k_new, g.v_new, kd, vd, g.scale, cache_layout="distinct", plan_cache=cache, **args)
+    again = dfx.paged_attention(g.q, g.k_new, g.v_new, kd, vd, g.scale, cache_layout="distinct", plan_cache=cache, **args)
+    gen = dfx.paged_attention(g.q, g.k_new, g.v_new, kd, vd, g.scale, cache_layout="distinct", flags=GENERIC, **args)
+    torch.cuda.synchronize()
+    if planned:
+        assert len(cache) == 1 and next(iter(cache.values())) is not None, "the streaming path takes a plan"
+    assert torch.isfinite(got.float()).all()
+    assert max_abs_err(got, want) <= ATOL_BF16
+    assert max_abs_err(got, gen) <= 1e-2
+    assert torch.equal(got, again)
+
+
+def test_distinct_layout_streams_with_v_sliced_out_of_the_projection(dev):
+    """Fresh V as a column slice of the QKV projection (another token stride than K's) on the distinct layout's
+    streaming path: the fresh tile's V rows land row-major and are transposed inside LDS."""
+    wl = make_workload("c3", seed=99, num_seqs=4, ctx=(200, 900)).to(dev)
+    want = oracle_fp32(wl)
+    T, hq, hkv, hd = wl.q.shape[0], wl.num_q_heads, wl.num_kv_heads, wl.head_dim
+    qkv = torch.empty(T, (hq + 2 * hkv) * hd, dtype=torch.bfloat16, device=dev)
+    q, k, v = (x.view(T, -1, hd) for x in qkv.split([hq * hd, hkv * hd, hkv * hd], dim=-1))
+    q.copy_(wl.q), k.copy_(wl.k_new), v.copy_(wl.v_new)
+    kd, vd = _to_distinct(wl.k_cache)[0], _to_distinct(wl.v_cache)[1]
+    got = dfx.paged_attention(q, k.contiguous(), v, kd, vd, wl.scale, cache_layout="distinct", block_tables=wl.block_tables,
+                              context_lens=wl.context_lens, cu_seqlens_q=wl.cu_seqlens_q, cu_seqlens_new=wl.cu_seqlens_q,
+                              max_seqlen_q=wl.q_len, mask_mode=wl.mask_mode, diffusion_block_size=wl.diffusion_block_size)
+    torch.cuda.synchronize()
+    assert max_abs_err(got, want) <= ATOL_BF16
 
 
 def test_attention_module_on_the_distinct_layout(dev):

@@ -477,7 +477,7 @@ def test_plan_cache_key_works_on_inference_tensors_and_sees_in_place_updates():
     q = torch.zeros(64, 28, 128, dtype=torch.bfloat16)
     k = torch.zeros(64, 4, 128, dtype=torch.bfloat16)
     kc = torch.zeros(4, 256, 4, 128, dtype=torch.bfloat16)
-    tail = (0.1, 32, 0, 32, 0, 0, 0)
+    tail = (0.1, 32, 0, 32, 0, 0, 0, None, None, None)   # (no rotary embedding inside the launch)
 
     def meta():
         return (torch.zeros(2, 8, dtype=torch.int32), torch.zeros(2, dtype=torch.int32),

@@ -645,7 +645,8 @@ def main():
     gbs = nbytes / (ms * 1e-3) / 1e9
     tflops = nflops / (ms * 1e-3) / 1e12
     traffic, traffic_source = measured_traffic(args.workload, nbytes) if args.page <= 0 and args.layout == "unified" else (None, None)
-    kernel = ("paged_attn_pipe_fp8_kernel<8>" if wl.kv_fp8 else
+    kernel = ("paged_attn_stream_kernel (head_dim 64: the compiler-scheduled step)" if wl.head_dim != 128 else
+              "paged_attn_pipe_fp8_kernel<8>" if wl.kv_fp8 else
               "paged_attn_pipe_kernel<8, false>" if args.layout == "unified" else
               "paged_attn_stream_kernel<128, 1, 8, false, true>")
     result = {

@@ -551,6 +551,9 @@ def main():
     ap.add_argument("--layout", default="unified", choices=["unified", "distinct"],
                     help="KV-cache layout of the attention workloads (bf16 ones): the reference's kv_cache_layout "
                          "(diffulex/config.py:43-44); 'distinct' is K [pages, H, hd/8, page, 8], V [pages, H, hd, page]")
+    ap.add_argument("--head-dim", type=int, default=0, choices=[0, 64, 128],
+                    help="head_dim of the attention workloads (default: the workload's own); 64 is what the reference's "
+                         "kernel tests use (tests/python/kernel/test_dllm_flash_attn_decode_kernel.py:223-391)")
     ap.add_argument("--copies", type=int, default=4, help="independent KV-cache copies rotated between steps")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -595,7 +598,8 @@ def main():
     if args.workload == "d2f-small":
         bench_d2f_small(args, dev)
         return
-    wl = make_workload(args.workload, device=dev, **({"page": args.page} if args.page > 0 else {}))
+    over = {**({"page": args.page} if args.page > 0 else {}), **({"hd": args.head_dim} if args.head_dim > 0 else {})}
+    wl = make_workload(args.workload, device=dev, **over)
     # every tensor a launch touches exists `copies` times; step i uses set i % copies
     sets = [(wl.q, wl.k_new, wl.v_new, torch.empty_like(wl.q), wl.k_cache, wl.v_cache)]
     for _ in range(args.copies - 1):
@@ -644,7 +648,7 @@ def main():
     nbytes, nflops = algorithmic_bytes(wl), algorithmic_flops(wl)
     gbs = nbytes / (ms * 1e-3) / 1e9
     tflops = nflops / (ms * 1e-3) / 1e12
-    traffic, traffic_source = measured_traffic(args.workload, nbytes) if args.page <= 0 and args.layout == "unified" else (None, None)
+    traffic, traffic_source = measured_traffic(args.workload, nbytes) if not over and args.layout == "unified" else (None, None)
     kernel = ("paged_attn_stream_kernel (head_dim 64: the compiler-scheduled step)" if wl.head_dim != 128 else
               "paged_attn_pipe_fp8_kernel<8>" if wl.kv_fp8 else
               "paged_attn_pipe_kernel<8, false>" if args.layout == "unified" else
@@ -680,7 +684,7 @@ def main():
         },
     }
     if not args.no_cpu:
-        result["cpu_baseline"] = cpu_baseline(args.workload, **({"page": args.page} if args.page > 0 else {}))
+        result["cpu_baseline"] = cpu_baseline(args.workload, **over)
     print(json.dumps(result))
 
 

@@ -201,6 +201,12 @@ struct StreamAttn : TileMath<HD, NB, NW, HIDDEN> {
     // null where the sequences follow each other in their own order
     const int32_t* order = nullptr;
     float k_mul, v_inv;  // FP8: the current item's K scale and the reciprocal of its V scale
+    // Units described at a time.  The 8-wave kernel on a cache of codes raises it where a plan has done the
+    // planning: the unit prefix over the sequences, a tenth of the LDS, is then not needed, and the tables
+    // take its place -- at its benchmark shape a workgroup's 170 units then fit one table instead of two,
+    // and every table's end costs it a drained pipeline and a prologue of three widened matrices.
+    static constexpr bool kGrowTables = KVB == 1 && NW == 8 && !COMPACT;
+    int chunk_cap = C::kPlanUnits;
 
     DFX_D StreamAttn(const KArgs& args, uint8_t* smem)
         : Base(args), lds(smem), prefix(reinterpret_cast<int*>(smem)),
@@ -629,14 +635,15 @@ struct StreamAttn : TileMath<HD, NB, NW, HIDDEN> {
         const int t = thread_number_here(wave_s);
         const bool starts = t < n_units && (units[t].flags & kUnitFreshStart) != 0;
         const uint64_t votes = __ballot(starts);
-        if (wave_s < 2 && t == wave_s * 64) {
+        constexpr int kBallots = kGrowTables ? 4 : 2;  // waves whose ballots cover a table
+        if (wave_s < kBallots && t == wave_s * 64) {
             misc[20 + 2 * wave_s] = static_cast<int>(votes);
             misc[21 + 2 * wave_s] = static_cast<int>(votes >> 32);
         }
         __syncthreads();
-        static_assert(C::kPlanUnits <= 128 && NW >= 2, "two waves' ballots cover a table");
+        static_assert(C::kPlanUnits <= 128 && NW >= kBallots, "the ballots cover a table");
         bool any = false;
-        for (int w = 0; w < 2; ++w) {
+        for (int w = 0; w < kBallots; ++w) {
             uint64_t m = (static_cast<uint64_t>(static_cast<uint32_t>(uniform(misc[21 + 2 * w]))) << 32) |
                          static_cast<uint32_t>(uniform(misc[20 + 2 * w]));
             while (m != 0) {
@@ -884,6 +891,20 @@ struct StreamAttn : TileMath<HD, NB, NW, HIDDEN> {
             for (int i = thread_number_here(wave_s); i <= n_active; i += C::THREADS) prefix[i] = g_bounds[i];
             split.bounds = prefix;
         }
+        if constexpr (kGrowTables) {
+            if (planned) {
+                // [cut points][scratch][unit table][band table] up to where the stages begin
+                const int bounds_bytes = plan_mode == 2 ? ((n_active + 1) * 4 + 255) & ~255 : 0;
+                const int per_unit = static_cast<int>(sizeof(UnitDesc)) + NW * static_cast<int>(sizeof(BandDesc));
+                const int cap = (C::STAGES_OFF - bounds_bytes - C::S::MISC_BYTES) / per_unit;
+                if (cap > C::kPlanUnits) {
+                    chunk_cap = min(cap, 256);  // (a thread per unit where the fresh rows' beginnings are looked for)
+                    misc = reinterpret_cast<int*>(lds + bounds_bytes);
+                    units = reinterpret_cast<UnitDesc*>(lds + bounds_bytes + C::S::MISC_BYTES);
+                    bands = reinterpret_cast<BandDesc*>(reinterpret_cast<uint8_t*>(units) + chunk_cap * static_cast<int>(sizeof(UnitDesc)));
+                }
+            }
+        }
         if (!planned && static_cast<int>(blockIdx.x) < n_active) {
             w.a0 = split.first(blockIdx.x);
             w.a1 = split.first(blockIdx.x + 1);
@@ -894,8 +915,8 @@ struct StreamAttn : TileMath<HD, NB, NW, HIDDEN> {
         const int64_t n_total = (w.a1 - w.a0) + (planned ? w.b1 - w.b0 : 0);
         begin = w.a0;
         end = planned ? w.a0 + n_total : w.a1;  // (with a plan only the length matters from here on)
-        for (int64_t done = 0; done < n_total; done += C::kPlanUnits) {
-            const int n_units = static_cast<int>(min(static_cast<int64_t>(C::kPlanUnits), n_total - done));
+        for (int64_t done = 0; done < n_total; done += chunk_cap) {
+            const int n_units = static_cast<int>(min(static_cast<int64_t>(chunk_cap), n_total - done));
             __syncthreads();  // every wave is done with the previous descriptors and their stages
             if (planned) {
                 // descriptors are multiples of 16 bytes: copied as such.  The lane's addresses are worked

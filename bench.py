@@ -652,7 +652,7 @@ def main():
     kernel = ("paged_attn_stream_kernel (head_dim 64: the compiler-scheduled step)" if wl.head_dim != 128 else
               "paged_attn_pipe_fp8_kernel<8>" if wl.kv_fp8 else
               "paged_attn_pipe_kernel<8, false>" if args.layout == "unified" else
-              "paged_attn_stream_kernel<128, 1, 8, false, true>")
+              "paged_attn_pipe_kernel<8, false, true>")
     result = {
         "metric": "attn query-tokens/sec + achieved HBM GB/s (% of peak), Dream-7B shape, 1 GPU",
         "value": wl.total_q_tokens / (ms * 1e-3), "unit": "query-tokens/s",

@@ -168,13 +168,13 @@ DFX_D void wait_async_loads() {
 // a multiple of 64 tokens, so that a tile lies in one page).  A stage then holds the K tile chunk-major and the
 // V tile d-major (attn_tile.h), both filled by the same direct-to-LDS loads: a wave takes two chunk columns of K
 // (1 KiB contiguous each) and 16 rows of V^T (128 contiguous bytes each).  The descriptors are per tile, the
-// same for every wave: BandDesc::off = page << 20 | first token's place in the page, BandDesc::last = the
-// tile's last valid token.  Fresh rows, row-major in memory: K is gathered into the chunk-major tile by the
+// same for every wave: BandDesc::off = KV head << 52 | page << 20 | first token's place in the page,
+// BandDesc::last = the tile's last valid token.  Fresh rows, row-major in memory: K is gathered into the chunk-major tile by the
 // loads themselves (a lane per token), V lands row-major and is transposed inside LDS before its step
 // (transpose_fresh_v).
 template <int HD, int NB, int NW, bool COMPACT = false, int KVB = 2, bool HIDDEN = false, bool DISTINCT = false>
 struct StreamAttn : TileMath<HD, NB, NW, HIDDEN> {
-    static_assert(!DISTINCT || (KVB == 2 && !HIDDEN && !COMPACT && NW == 8 && HD == 128), "distinct layout: bf16, 8 waves, head_dim 128");
+    static_assert(!DISTINCT || (KVB == 2 && !COMPACT && NW == 8 && HD == 128), "distinct layout: bf16, 8 waves, head_dim 128");
     using Base = TileMath<HD, NB, NW, HIDDEN>;
     using C = StreamCfg<HD, NB, NW, COMPACT, KVB>;
     using L = TileLayout<HD>;
@@ -214,7 +214,12 @@ struct StreamAttn : TileMath<HD, NB, NW, HIDDEN> {
           units(reinterpret_cast<UnitDesc*>(smem + C::UNIT_TABLE_OFF)),
           bands(reinterpret_cast<BandDesc*>(smem + C::BAND_TABLE_OFF)),
           stages_lds(static_cast<uint32_t>(reinterpret_cast<uintptr_t>(smem)) + C::STAGES_OFF),
-          wave_s(uniform(static_cast<int>(threadIdx.x >> 6))) {}
+          wave_s(uniform(static_cast<int>(threadIdx.x >> 6))) {
+        if constexpr (DISTINCT) {  // the lane's operand offsets in a chunk-major K tile and a d-major V tile (attn_tile.h)
+            this->k_lane = static_cast<uint32_t>(half * Base::CHUNK_COL_BYTES + Base::swap_quads(col) * 16);
+            this->v_lane = static_cast<uint32_t>(Base::vt_chunk_offset(col, half));
+        }
+    }
 
     // ---- planning --------------------------------------------------------------------------
     // Describe units [first, first + count) in the plan table (entry i is unit first + i); one
@@ -282,7 +287,7 @@ struct StreamAttn : TileMath<HD, NB, NW, HIDDEN> {
                     int64_t page = p < a.max_pages ? a.block_tables[static_cast<int64_t>(sq) * a.bt_stride + p] : -1;
                     hole = page < 0 || page >= a.n_pages;
                     page = page < 0 ? 0 : (page >= a.n_pages ? a.n_pages - 1 : page);
-                    b.off = (page << 20) | static_cast<int64_t>(base - p * a.page_size);
+                    b.off = (static_cast<int64_t>(kv_head) << 52) | (page << 20) | static_cast<int64_t>(base - p * a.page_size);
                 } else {
                     b.off = ((static_cast<int64_t>(a.cu_new[sq]) + base) * a.kn_st + kv_head * a.kn_sh) * 2;
                 }
@@ -321,10 +326,10 @@ struct StreamAttn : TileMath<HD, NB, NW, HIDDEN> {
                             static_cast<uint32_t>(uniform(static_cast<int>(b.off)));
         if constexpr (DISTINCT) {
             const uint32_t dst = stages_lds + (static_cast<unsigned>(rel) % C::kStages) * C::STAGE_BYTES;
-            const int kvh = uniform(units[rel].kvh);
             const uint32_t tok = static_cast<uint32_t>(min(lane, last));  // tokens past the end re-read the last valid one
             if (is_ctx) {
-                const int64_t page = off >> 20;
+                const int64_t kvh = static_cast<int64_t>(static_cast<uint64_t>(off) >> 52);
+                const int64_t page = (off >> 20) & 0xffffffffll;
                 const int64_t in_page = off & 0xfffff;
                 const uint8_t* kb = a.k_cache + (page * a.kd_sp + kvh * a.kd_sh + in_page * 8) * 2;
                 const uint8_t* vb = a.v_cache + (page * a.vd_sp + kvh * a.vd_sh + in_page) * 2;
@@ -797,7 +802,7 @@ struct StreamAttn : TileMath<HD, NB, NW, HIDDEN> {
 #pragma unroll
                 for (int w = 0; w < NW; ++w) {
                     const BandDesc& b = bands[(r + kPlainAhead) * NW + w];
-                    full = full && (b.is_ctx > 0) != fresh_bands && b.last >= C::ROWS_PER_WAVE - 1;
+                    full = full && (b.is_ctx > 0) != fresh_bands && b.last >= (DISTINCT ? C::TN : C::ROWS_PER_WAVE) - 1;
                 }
                 flags = units[r].flags;
                 const UnitDesc& nxt = units[r + 1];
@@ -805,6 +810,9 @@ struct StreamAttn : TileMath<HD, NB, NW, HIDDEN> {
                 if (!(nxt.flags & kUnitCtx) && a.mask_mode == DFX_MASK_BLOCK_CAUSAL)
                     masked = masked || nxt.base + C::TN > clear_limit(nxt.rt, nxt.q_len);
                 plain = full && !(flags & kUnitLast) && !masked;
+                // distinct layout: the step's own tile must need nothing done to its V^T rows first (a fresh tile is
+                // transposed, one that ends early or lies on a missing page is cleared: the general step does that)
+                if (DISTINCT) plain = plain && (flags & kUnitCtx) != 0 && units[r].base + C::TN <= units[r].limit && unit_holes(flags) == 0;
                 // codes: the step also widens K of unit r + 2 and V of unit r + 1, and a plain one only knows cached rows
                 if (KVB == 1) plain = plain && (flags & nxt.flags & units[r + 2].flags & kUnitCtx) != 0;
             }
@@ -1216,16 +1224,54 @@ __global__ void __launch_bounds__(64 * NW, 1) paged_attn_stream_fp8_kernel(const
 // PREFILL: the variant for launches without a cache.  Every tile
 // is one of fresh rows there, and its plain steps fetch full bands of those the way the other variant's
 // fetch bands of cached rows (which keeps its fresh tiles, one or two per item, on the general step).
-template <int NW, bool PREFILL = false>
+// The blocks of attn_pipe_gen.h for the tile layout of the kernel's cache.
+template <bool DISTINCT>
+struct PipeBlocks {
+#define DFX_PIPE_BLOCK(name, params, args)                     \
+    DFX_D static void name params {                            \
+        if constexpr (DISTINCT) pipe_d_##name args;            \
+        else pipe_##name args;                                 \
+    }
+    DFX_PIPE_BLOCK(first_scores, (uint32_t k, float& mx), (k, mx))
+    DFX_PIPE_BLOCK(mask_a_8, (int thr, uint32_t holes, float& mx), (thr, holes, mx))
+    DFX_PIPE_BLOCK(mask_a_16, (int thr, uint32_t holes, float& mx), (thr, holes, mx))
+    DFX_PIPE_BLOCK(mask_b_8, (int thr, uint32_t holes, float& mx), (thr, holes, mx))
+    DFX_PIPE_BLOCK(mask_b_16, (int thr, uint32_t holes, float& mx), (thr, holes, mx))
+    DFX_PIPE_BLOCK(step_ab_x, (uint32_t k, uint32_t v, float c, float nm, float& l), (k, v, c, nm, l))
+    DFX_PIPE_BLOCK(step_ab_y, (float c, float nm, float& l, float& mx), (c, nm, l, mx))
+    DFX_PIPE_BLOCK(step_ba_x, (uint32_t k, uint32_t v, float c, float nm, float& l), (k, v, c, nm, l))
+    DFX_PIPE_BLOCK(step_ba_y, (float c, float nm, float& l, float& mx), (c, nm, l, mx))
+    DFX_PIPE_BLOCK(last_a_x, (uint32_t v, float c, float nm, float& l), (v, c, nm, l))
+    DFX_PIPE_BLOCK(last_a_y, (float c, float nm, float& l), (c, nm, l))
+    DFX_PIPE_BLOCK(last_b_x, (uint32_t v, float c, float nm, float& l), (v, c, nm, l))
+    DFX_PIPE_BLOCK(last_b_y, (float c, float nm, float& l), (c, nm, l))
+#undef DFX_PIPE_BLOCK
+};
+
+// DISTINCT: the cache is in the distinct layout (StreamAttn): the blocks read a chunk-major K tile and a d-major V
+// tile, a full tile of cached rows is fetched by pipe_d_issue_band, and the general step first does to its own
+// tile's V^T rows what the loads could not (transpose_fresh_v, clear_v_tail); no store, no rotary embedding.
+template <int NW, bool PREFILL = false, bool DISTINCT = false>
 __global__ void __launch_bounds__(64 * NW, 1) __attribute__((amdgpu_num_vgpr(32)))
 paged_attn_pipe_kernel(const KArgs a) {
+    static_assert(!(PREFILL && DISTINCT), "a launch without a cache has no cache layout");
     extern __shared__ __attribute__((aligned(256))) uint8_t smem[];
     constexpr int HD = 128;
     using C = StreamCfg<HD, 1, NW, false>;
-    using SA = StreamAttn<HD, 1, NW, false, 2, true>;
+    using SA = StreamAttn<HD, 1, NW, false, 2, true, DISTINCT>;
+    using PB = PipeBlocks<DISTINCT>;
     SA at(a, smem);
     pipe_reserve();
-    {
+    if constexpr (DISTINCT) {
+        // a lane per token of a chunk column of K; 8 lanes per row of V^T, the wave's rows 16 w + lane / 8 and 8 further
+        uint32_t v[2];
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int d = at.wave * 16 + j * 8 + (at.lane >> 3);
+            v[j] = static_cast<uint32_t>(d) * static_cast<uint32_t>(a.vd_sd * 2) + ((at.lane & 7) ^ ((d >> 1) & 7)) * 16;
+        }
+        pipe_d_set_load_offsets(at.lane * 16, v[0], v[1]);
+    } else {
         uint32_t o[2];
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
@@ -1252,8 +1298,10 @@ paged_attn_pipe_kernel(const KArgs a) {
             pipe_set_load_offsets(o[0], o[1]);
         }
     }
-    const bool rope = !PREFILL && a.rope_table != nullptr;  // (with it the store travels with the rotation of the fresh K rows)
-    if (!rope) store_fresh_rows<HD, false, 1>(a);
+    const bool rope = !PREFILL && !DISTINCT && a.rope_table != nullptr;  // (with it the store travels with the rotation of the fresh K rows)
+    if constexpr (!DISTINCT) {
+        if (!rope) store_fresh_rows<HD, false, 1>(a);
+    }
     const bool busy = at.wave < a.busy_waves;  // waves whose 32 rows exist in no item of this launch only fetch
     constexpr int kHoleRows = C::ROWS_PER_WAVE;
     static_assert(kHoleRows == 8 || kHoleRows == 16, "mask blocks of attn_pipe_gen.h");
@@ -1271,7 +1319,7 @@ paged_attn_pipe_kernel(const KArgs a) {
         // angles of the first item's query rows, requested behind the stores of those rows so that the two
         // trips to memory run together.
         bool rotate_first = false;
-        if constexpr (!PREFILL) {
+        if constexpr (!PREFILL && !DISTINCT) {
             if (rope) {
                 int64_t pos = 0;
                 if (opens) pos = at.rope_query_position(at.units[0]);
@@ -1328,14 +1376,14 @@ paged_attn_pipe_kernel(const KArgs a) {
             if (!(t.base + C::TN > t.limit || t.holes != 0 || bc)) return;
             int lim = t.limit;
             if (bc) lim = min(lim, at.visible_limit(at.units[r]));
-            const int thr = lim - t.base - 4 * at.half;
+            const int thr = lim - t.base - (DISTINCT ? 8 : 4) * at.half;
             const uint32_t holes = static_cast<uint32_t>(t.holes);
             if (set_a) {
-                if constexpr (kHoleRows == 8) pipe_mask_a_8(thr, holes, mx_lane);
-                else pipe_mask_a_16(thr, holes, mx_lane);
+                if constexpr (kHoleRows == 8) PB::mask_a_8(thr, holes, mx_lane);
+                else PB::mask_a_16(thr, holes, mx_lane);
             } else {
-                if constexpr (kHoleRows == 8) pipe_mask_b_8(thr, holes, mx_lane);
-                else pipe_mask_b_16(thr, holes, mx_lane);
+                if constexpr (kHoleRows == 8) PB::mask_b_8(thr, holes, mx_lane);
+                else PB::mask_b_16(thr, holes, mx_lane);
             }
         };
 
@@ -1380,7 +1428,7 @@ paged_attn_pipe_kernel(const KArgs a) {
                 neg_m = (m_run == -INFINITY) ? 0.0f : -m_run;
             };
             if (busy) {
-                pipe_first_scores(at.lds_address(tile_of(rel)) + at.k_lane, mx_lane);
+                PB::first_scores(at.lds_address(tile_of(rel)) + at.k_lane, mx_lane);
                 mask(rel, true, mx_lane);
                 if (compute_first) prepare();
             }
@@ -1390,6 +1438,12 @@ paged_attn_pipe_kernel(const KArgs a) {
             // youngest tile load in flight was issued, instead of in front of an idle matrix unit.
             const bool next_opens = run_end < n_units;
             auto step = [&](int r, bool cur_is_a) {
+                if constexpr (DISTINCT) {  // (unit r landed before the step that read its K tile; every wave comes here)
+                    const TileInfo tr = at.tile_info_of(r);
+                    if (!tr.is_ctx) at.transpose_fresh_v(r);
+                    else if (tr.holes != 0) at.clear_v_tail(r, 0);  // (a page without a table entry: page 0 was read in its place)
+                    else if (tr.base + C::TN > tr.limit) at.clear_v_tail(r, tr.limit - tr.base);
+                }
                 const bool has_next = r + 1 < run_end;
                 const bool fetch = has_next && admit(r + 1, r);
                 if (!has_next && next_opens) at.request_queries(at.units[run_end]);
@@ -1402,20 +1456,20 @@ paged_attn_pipe_kernel(const KArgs a) {
                     if (has_next) {
                         const uint32_t k_next = at.lds_address(tile_of(r + 1)) + at.k_lane;
                         if (cur_is_a) {
-                            pipe_step_ab_x(k_next, v_cur, a.c, neg_m, at.l_run[0]);
-                            pipe_step_ab_y(a.c, neg_m, at.l_run[0], mx_lane);
+                            PB::step_ab_x(k_next, v_cur, a.c, neg_m, at.l_run[0]);
+                            PB::step_ab_y(a.c, neg_m, at.l_run[0], mx_lane);
                         } else {
-                            pipe_step_ba_x(k_next, v_cur, a.c, neg_m, at.l_run[0]);
-                            pipe_step_ba_y(a.c, neg_m, at.l_run[0], mx_lane);
+                            PB::step_ba_x(k_next, v_cur, a.c, neg_m, at.l_run[0]);
+                            PB::step_ba_y(a.c, neg_m, at.l_run[0], mx_lane);
                         }
                         mask(r + 1, !cur_is_a, mx_lane);
                     } else {
                         if (cur_is_a) {
-                            pipe_last_a_x(v_cur, a.c, neg_m, at.l_run[0]);
-                            pipe_last_a_y(a.c, neg_m, at.l_run[0]);
+                            PB::last_a_x(v_cur, a.c, neg_m, at.l_run[0]);
+                            PB::last_a_y(a.c, neg_m, at.l_run[0]);
                         } else {
-                            pipe_last_b_x(v_cur, a.c, neg_m, at.l_run[0]);
-                            pipe_last_b_y(a.c, neg_m, at.l_run[0]);
+                            PB::last_b_x(v_cur, a.c, neg_m, at.l_run[0]);
+                            PB::last_b_y(a.c, neg_m, at.l_run[0]);
                         }
                     }
                     if (compute_first) {
@@ -1429,9 +1483,17 @@ paged_attn_pipe_kernel(const KArgs a) {
             // the offset of this wave's band of the unit to fetch.
             auto plain_step = [&](int r, bool cur_is_a, int64_t off, int row) {
                 auto issue_band = [&](int dst) {
-                    if constexpr (PREFILL) pipe_issue_band_fresh(reinterpret_cast<const uint8_t*>(a.k_new) + off,
-                                                                 reinterpret_cast<const uint8_t*>(a.v_new) + off + static_cast<int64_t>(row) * a.v_fresh_delta, dst);
-                    else pipe_issue_band(a.k_cache + off, a.v_cache + off, dst);
+                    if constexpr (PREFILL) {
+                        pipe_issue_band_fresh(reinterpret_cast<const uint8_t*>(a.k_new) + off,
+                                              reinterpret_cast<const uint8_t*>(a.v_new) + off + static_cast<int64_t>(row) * a.v_fresh_delta, dst);
+                    } else if constexpr (DISTINCT) {
+                        const int64_t kvh = static_cast<int64_t>(static_cast<uint64_t>(off) >> 52);
+                        const int64_t page = (off >> 20) & 0xffffffffll, in_page = off & 0xfffff;
+                        const uint8_t* kb = a.k_cache + (page * a.kd_sp + kvh * a.kd_sh + in_page * 8 + at.wave_s * 2 * a.kd_sc) * 2;
+                        pipe_d_issue_band(kb, kb + a.kd_sc * 2, a.v_cache + (page * a.vd_sp + kvh * a.vd_sh + in_page) * 2, dst);
+                    } else {
+                        pipe_issue_band(a.k_cache + off, a.v_cache + off, dst);
+                    }
                 };
                 wait_async_loads<C::LOADS_PER_UNIT>();  // unit r + 1 has landed; unit r + 2 may be on its way
                 __builtin_amdgcn_s_barrier();
@@ -1445,11 +1507,11 @@ paged_attn_pipe_kernel(const KArgs a) {
                     const uint32_t v_cur = at.lds_address(tile_of(r) + C::MAT_BYTES) + at.v_lane;
                     const uint32_t k_next = at.lds_address(tile_of(r + 1)) + at.k_lane;
                     if (cur_is_a) {
-                        pipe_step_ab_x(k_next, v_cur, a.c, neg_m, at.l_run[0]);
-                        pipe_step_ab_y(a.c, neg_m, at.l_run[0], mx_lane);
+                        PB::step_ab_x(k_next, v_cur, a.c, neg_m, at.l_run[0]);
+                        PB::step_ab_y(a.c, neg_m, at.l_run[0], mx_lane);
                     } else {
-                        pipe_step_ba_x(k_next, v_cur, a.c, neg_m, at.l_run[0]);
-                        pipe_step_ba_y(a.c, neg_m, at.l_run[0], mx_lane);
+                        PB::step_ba_x(k_next, v_cur, a.c, neg_m, at.l_run[0]);
+                        PB::step_ba_y(a.c, neg_m, at.l_run[0], mx_lane);
                     }
                     if (compute_first) {
                         issue_band(dst);

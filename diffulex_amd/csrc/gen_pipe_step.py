@@ -63,6 +63,12 @@ LOAD_OFF = 43               # two registers: byte offsets of the lane's chunk in
 WIDEN_ADDR = 45             # three registers: LDS addresses for pipe_widen (cache of one-byte codes)
 FRESH_OFF = 45              # two registers: LOAD_OFF for a band of fresh rows (two-byte cache elements: no pipe_widen there)
 MAT_BYTES = 64 * ROWB       # K tile; the V tile of a ring stage follows it
+# Tile layout the blocks being generated read: 'u' (cache in the unified layout: both tiles row-major, 16-byte chunks
+# swizzled by the row) or 'd' (distinct layout: K tile chunk-major [HD / 8][64 tokens][16 bytes], V tile d-major
+# [HD][64 tokens] with chunks swizzled by (d / 2) % 8; the key rows feed S^T with quads 1 and 2 of every 16 swapped, so
+# that a lane's 8 scores of a 16-token slab are 8 consecutive tokens, as a chunk of a V^T row holds them).
+LAYOUT = "u"
+CHUNK_COL_BYTES = 64 * 16
 NEG_INF = "0xff800000"
 MFMA_TO_VALU = ["s_nop 15", "s_nop 1"]  # 18 wait states: the longest the ISA asks for
 
@@ -145,6 +151,11 @@ def pair_instrs(cur, pr):
 def vaddr_instrs():
     """V^T operand addresses vx[z] = %[v0] ^ const_z."""
     out = []
+    if LAYOUT == "d":  # one per 16-token slab z = 2 tb + sl: chunk 2 z + half; the d block is an immediate offset
+        for z in range(4):
+            out.append((f"v_mov_b32 {vr(T_VADDR)}, %[v0]", {T_VADDR}) if z == 0 else
+                       (f"v_xor_b32 {vr(T_VADDR + z)}, {z * 32:#x}, %[v0]", {T_VADDR + z}))
+        return out
     for z in range(2 * NDB):
         const = (((z >> 1) * 4) ^ swizzle((z & 1) * 8)) * 16
         if z == 0:
@@ -184,6 +195,9 @@ def phase_x(b, nxt, stream, quotas):
 
     def read(i):
         slab, tb = i >> 1, i & 1
+        if LAYOUT == "d":  # chunk column 2 slab + half, tokens 32 tb ..: every offset an immediate
+            b.lds_read(f"ds_read_b128 {vr(RING + 4 * (i % 4), 4)}, %[k0] offset:{slab * 2 * CHUNK_COL_BYTES + tb * 32 * 16}", ("k", i))
+            return
         if tb == 0 and slab > 0:
             b.valu(f"v_xor_b32 {vr(T_ADDR)}, {slab * 32:#x}, %[k0]", {T_ADDR})
         addr = "%[k0]" if slab == 0 else vr(T_ADDR)
@@ -208,6 +222,9 @@ def phase_y(b, cur, stream, quotas):
 
     def read(j):
         tb, sl, db = j // (2 * NDB), (j // NDB) & 1, j % NDB
+        if LAYOUT == "d":  # row 32 db + lane % 32 of V^T, the 8 tokens of the lane's half of the slab: one read
+            b.lds_read(f"ds_read_b128 {vr(RING + 4 * (j % 4), 4)}, {vr(T_VADDR + 2 * tb + sl)} offset:{db * 32 * 128}", ("v", j, 1))
+            return
         for ii in range(2):
             off = (tb * 32 + sl * 16 + ii * 8) * ROWB
             b.lds_read(f"ds_read_b64_tr_b16 {vr(RING + 4 * (j % 4) + 2 * ii, 2)}, {vr(T_VADDR + 2 * db + ii)} offset:{off}",
@@ -286,7 +303,9 @@ def mask_block(s, hole_rows):
                 f"v_cndmask_b32 {vr(t)}, %[thr], -1, vcc"]
         for j in range(4):
             reg = s + 16 * tb + 4 * q + j
-            ins += [f"v_cmp_lt_i32 vcc, {g * 8 + j}, {vr(t)}",
+            # token of the element (the wave's upper half sits 4 higher, 8 with the swapped quads: in %[thr])
+            token = g * 8 + j if LAYOUT == "u" else tb * 32 + (q >> 1) * 16 + (q & 1) * 4 + j
+            ins += [f"v_cmp_lt_i32 vcc, {token}, {vr(t)}",
                     f"v_cndmask_b32 {vr(reg)}, {vr(ninf)}, {vr(reg)}, vcc"]
     ins += [text for text, _ in max_instrs(s)]
     return join(ins)
@@ -532,22 +551,39 @@ DFX_D void pipe_set_output(int db, const f32x16& v) {
 DFX_D void pipe_outputs_ready() { asm volatile("s_nop 15\\n\\ts_nop 1" ::: "memory"); }
 
 ''')
-    parts.append(asm_fn("pipe_first_scores", "uint32_t k_next, float& mx", first_scores_block(SA),
-                        ['[mx] "=&v"(mx)'], ['[k0] "v"(k_next)'], ["memory"],
-                        "S^T of a run's first tile (LDS address k_next: tile + the lane's K operand offset) into score\nset A, and the lane's maximum."))
-    for hole_rows in (8, 16):
-        for nm, s in (("a", SA), ("b", SB)):
-            parts.append(asm_fn(f"pipe_mask_{nm}_{hole_rows}", "int thr, uint32_t holes, float& mx", mask_block(s, hole_rows),
-                                ['[mx] "=&v"(mx)'], ['[thr] "v"(thr)', '[holes] "s"(holes)'], ["vcc", "scc"],
-                                f"Mask of score set {nm.upper()} (tokens >= thr of the tile, and the {hole_rows}-token bands whose bit in `holes` is set,\n"
-                                "become -inf) and the lane's maximum of the masked set."))
-    parts.append(step_fns("pipe_step_ab", SA, SB, True,
-                          "One step, in two halves (_x then _y): softmax and O^T += V^T P^T of the current score set (A; v_cur:\n"
-                          "LDS address of the V tile + the lane's V^T operand offset), S^T of the next tile into the other set\n"
-                          "and its lane maximum."))
-    parts.append(step_fns("pipe_step_ba", SB, SA, True))
-    parts.append(step_fns("pipe_last_a", SA, SB, False, "Last step of a run: no next tile."))
-    parts.append(step_fns("pipe_last_b", SB, SA, False))
+    global LAYOUT
+    for LAYOUT, pre, what in (("u", "pipe_", ""), ("d", "pipe_d_", "  Tiles of a cache in the distinct layout.")):
+        parts.append(asm_fn(pre + "first_scores", "uint32_t k_next, float& mx", first_scores_block(SA),
+                            ['[mx] "=&v"(mx)'], ['[k0] "v"(k_next)'], ["memory"],
+                            "S^T of a run's first tile (LDS address k_next: tile + the lane's K operand offset) into score\nset A, and the lane's maximum." + what))
+        for hole_rows in (8, 16):
+            for nm, s in (("a", SA), ("b", SB)):
+                parts.append(asm_fn(f"{pre}mask_{nm}_{hole_rows}", "int thr, uint32_t holes, float& mx", mask_block(s, hole_rows),
+                                    ['[mx] "=&v"(mx)'], ['[thr] "v"(thr)', '[holes] "s"(holes)'], ["vcc", "scc"],
+                                    f"Mask of score set {nm.upper()} (tokens >= thr of the tile, and the {hole_rows}-token bands whose bit in `holes` is set,\n"
+                                    "become -inf) and the lane's maximum of the masked set." + what))
+        parts.append(step_fns(pre + "step_ab", SA, SB, True,
+                              "One step, in two halves (_x then _y): softmax and O^T += V^T P^T of the current score set (A; v_cur:\n"
+                              "LDS address of the V tile + the lane's V^T operand offset), S^T of the next tile into the other set\n"
+                              "and its lane maximum." + what))
+        parts.append(step_fns(pre + "step_ba", SB, SA, True))
+        parts.append(step_fns(pre + "last_a", SA, SB, False, "Last step of a run: no next tile." + what))
+        parts.append(step_fns(pre + "last_b", SB, SA, False))
+    LAYOUT = "u"
+    parts.append(asm_fn("pipe_d_set_load_offsets", "uint32_t k, uint32_t v0, uint32_t v1",
+                        join(f"v_mov_b32 {vr(LOAD_OFF + j)}, %{j}" for j in range(3)), ins=['"v"(k)', '"v"(v0)', '"v"(v1)'],
+                        comment="Once per kernel (distinct layout): the lane's byte offsets for the wave's loads of a full tile of cached\n"
+                                "rows: inside a chunk column of K (its token), and inside the (page, head) of V for the two rows of V^T it\n"
+                                "fetches a chunk of (row * row stride + the chunk its place in the row holds)."))
+    issue_d = [f"s_add_u32 m0, %[d], 0", f"global_load_lds_dwordx4 {vr(LOAD_OFF)}, %[k0] nt",
+               f"s_add_u32 m0, %[d], 1024", f"global_load_lds_dwordx4 {vr(LOAD_OFF)}, %[k1] nt",
+               f"s_add_u32 m0, %[d], {MAT_BYTES}", f"global_load_lds_dwordx4 {vr(LOAD_OFF + 1)}, %[vb] nt",
+               f"s_add_u32 m0, %[d], {MAT_BYTES + 1024}", f"global_load_lds_dwordx4 {vr(LOAD_OFF + 2)}, %[vb] nt"]
+    parts.append(asm_fn("pipe_d_issue_band", "const void* k_col0, const void* k_col1, const void* v_rows, uint32_t lds_dst", join(issue_d),
+                        ins=['[k0] "s"(k_col0)', '[k1] "s"(k_col1)', '[vb] "s"(v_rows)', '[d] "s"(lds_dst)'], clobbers=["memory", "m0", "scc"],
+                        comment="The wave's four direct-to-LDS loads of a full tile of cached rows in the distinct layout: its two chunk\n"
+                                "columns of K (64 tokens of each at k_col0 / k_col1) and its 16 rows of V^T (v_rows: the tile's first token\n"
+                                "in row 0 of the (page, head)); lds_dst: the wave's place in the K tile of the ring stage."))
     parts.append("}  // namespace dfx\n")
     return "".join(parts)
 

@@ -92,10 +92,10 @@ int make_plan(const dfx_attn_params* p, Plan& plan) {
         if (rows > 64 || items <= 2 * static_cast<int64_t>(device_cu_count())) plan.nb = 2;
     }
     plan.compact = plan.stream && !plan.fp8 && plan.nb == 1 && p->num_seqs <= kCompactMaxSeqs;
-    // (the distinct layout's kernel runs the compiler-scheduled step)
+
     // (8 waves only: with 4 waves a wave has twice the tile loads to address, and the 32 registers
     // the pipelined kernel leaves the compiler no longer hold that without spilling in the loop)
-    plan.pipelined = plan.stream && !plan.compact && plan.hd == 128 && plan.nb == 2 && !plan.distinct &&
+    plan.pipelined = plan.stream && !plan.compact && plan.hd == 128 && plan.nb == 2 &&
                      !(p->flags & DFX_ATTN_NO_PIPELINE);
     if (p->max_workgroups > 0) {
         plan.n_wg = p->max_workgroups;
@@ -202,6 +202,10 @@ int launch(const KArgs& ka, const Plan& plan, hipStream_t st, const PlanArgs* pa
         using C = StreamCfg<HD, 1, NW, false>;
         main_k = paged_attn_stream_kernel<HD, 1, NW, false, true>;
         slot = 32;
+        if (plan.pipelined) {
+            main_k = paged_attn_pipe_kernel<NW, false, true>;
+            slot = 33;
+        }
         lds = C::LDS_BYTES;
         plan_k = paged_attn_plan_kernel<C::RT>;
         plan_slot = C::RT == 256 ? 31 : 30;
@@ -272,7 +276,7 @@ int check_args(const dfx_attn_params* p, Plan& plan, bool& empty) {
     if (!(p->scale > 0.0f) || p->diffusion_block_size <= 0) return DFX_ERR_INVALID_ARG;
     if (p->mask_mode != DFX_MASK_FULL && p->mask_mode != DFX_MASK_BLOCK_CAUSAL) return DFX_ERR_INVALID_ARG;
     if (p->rope_cos_sin != nullptr) {
-        if (!plan.pipelined || !has_cache) return DFX_ERR_UNSUPPORTED;
+        if (!plan.pipelined || !has_cache || plan.distinct) return DFX_ERR_UNSUPPORTED;
         if (!p->rope_positions || !p->k_rotated || p->rope_max_position <= 0 || p->k_rotated == p->k_new) return DFX_ERR_INVALID_ARG;
         if (p->rope_position_index_type != DFX_INDEX_I32 && p->rope_position_index_type != DFX_INDEX_I64) return DFX_ERR_INVALID_ARG;
         if (p->kr_stride_token < 0 || p->kr_stride_token % 8 || p->kr_stride_head < 0 || p->kr_stride_head % 8) return DFX_ERR_INVALID_ARG;

@@ -210,7 +210,8 @@ typedef struct dfx_attn_params {
      * (diffulex_kernel/python/kv_cache_kernels.py:35-83) but its decode refuses it
      * (diffulex/attention/attn_impl.py:66-69); here it is decoded.  head_dim 128 with pages of a multiple
      * of 64 tokens (fresh K and V with one head stride, vc_stride[2] below 2^22) streams -- the K tile
-     * chunk-major and the V tile d-major in LDS, as the layout has them -- and takes a plan; other shapes,
+     * chunk-major and the V tile d-major in LDS, as the layout has them, through the same pipelined step as
+     * the unified layout -- and takes a plan; other shapes,
      * and DFX_ATTN_GENERIC_PATH, run the generic tile path, which takes none.  No fused store, no FP8, no
      * rotary embedding inside the launch with it.  What a page holds behind a sequence's end is never
      * used, whatever it is. */

@@ -345,12 +345,17 @@ def test_distinct_layout_on_the_streaming_path(dev, name, over, max_wg, planned)
     got = dfx.paged_attention(g.q, g.k_new, g.v_new, kd, vd, g.scale, cache_layout="distinct", plan_cache=cache, **args)
     again = dfx.paged_attention(g.q, g.k_new, g.v_new, kd, vd, g.scale, cache_layout="distinct", plan_cache=cache, **args)
     gen = dfx.paged_attention(g.q, g.k_new, g.v_new, kd, vd, g.scale, cache_layout="distinct", flags=GENERIC, **args)
+    # the compiler-scheduled step on the same tiles (the default is the generated one)
+    cs = dfx.paged_attention(g.q, g.k_new, g.v_new, kd, vd, g.scale, cache_layout="distinct", flags=_lib.DFX_ATTN_NO_PIPELINE,
+                             plan_cache={} if planned else None, **args)
     torch.cuda.synchronize()
     if planned:
         assert len(cache) == 1 and next(iter(cache.values())) is not None, "the streaming path takes a plan"
-    assert torch.isfinite(got.float()).all()
-    assert max_abs_err(got, want) <= ATOL_BF16
-    assert max_abs_err(got, gen) <= 1e-2
+    for out in (got, cs):
+        assert torch.isfinite(out.float()).all()
+        assert max_abs_err(out, want) <= ATOL_BF16
+        assert max_abs_err(out, gen) <= 1e-2
+    assert max_abs_err(got, cs) <= 1e-2
     assert torch.equal(got, again)
 
 

@@ -55,11 +55,12 @@ def _tile_loop(isa_text, mangled_prefix):
 # kernel, hand-placed vmcnt waits in its loop (three alternatives of wait_younger; the FP8 kernel
 # also waits inside the branch that copies fresh bf16 rows, once per load round of a wave)
 KERNELS = [
-    ("_ZN3dfx24paged_attn_stream_kernelILi128ELi1ELi8ELb0E", 3),
-    ("_ZN3dfx24paged_attn_stream_kernelILi128ELi1ELi4ELb1E", 3),
-    ("_ZN3dfx24paged_attn_stream_kernelILi128ELi1ELi4ELb0E", 3),
-    ("_ZN3dfx24paged_attn_stream_kernelILi64ELi1ELi8ELb0E", 3),
-    ("_ZN3dfx24paged_attn_stream_kernelILi64ELi1ELi4ELb1E", 3),
+    ("_ZN3dfx24paged_attn_stream_kernelILi128ELi1ELi8ELb0ELb0E", 3),
+    ("_ZN3dfx24paged_attn_stream_kernelILi128ELi1ELi4ELb1ELb0E", 3),
+    ("_ZN3dfx24paged_attn_stream_kernelILi128ELi1ELi4ELb0ELb0E", 3),
+    ("_ZN3dfx24paged_attn_stream_kernelILi64ELi1ELi8ELb0ELb0E", 3),
+    ("_ZN3dfx24paged_attn_stream_kernelILi64ELi1ELi4ELb1ELb0E", 3),
+    ("_ZN3dfx24paged_attn_stream_kernelILi128ELi1ELi8ELb0ELb1E", 3),   # the distinct cache layout
     ("_ZN3dfx28paged_attn_stream_fp8_kernelILi128ELi1ELi8E", 3 + 2),
     ("_ZN3dfx28paged_attn_stream_fp8_kernelILi128ELi1ELi4E", 3 + 3),
 ]
@@ -80,7 +81,8 @@ def test_tile_loop_has_no_spills_and_no_compiler_waits(isa, kernel, max_waits):
     assert ops["global_load_lds_dwordx4"] in (2, 4, 8)   # a wave's share of the 64 * head_dim * elt * 2 bytes of a tile
 
 
-PIPE_KERNELS = ["_ZN3dfx22paged_attn_pipe_kernelILi8ELb0E", "_ZN3dfx22paged_attn_pipe_kernelILi8ELb1E",
+PIPE_KERNELS = ["_ZN3dfx22paged_attn_pipe_kernelILi8ELb0ELb0E", "_ZN3dfx22paged_attn_pipe_kernelILi8ELb1ELb0E",
+                "_ZN3dfx22paged_attn_pipe_kernelILi8ELb0ELb1E",   # the distinct cache layout
                 "_ZN3dfx26paged_attn_pipe_fp8_kernelILi8E"]
 
 

@@ -1437,6 +1437,10 @@ paged_attn_pipe_kernel(const KArgs a) {
             // step of this run and waited for behind that step's matrix work, one step later than the
             // youngest tile load in flight was issued, instead of in front of an idle matrix unit.
             const bool next_opens = run_end < n_units;
+            // (requested behind the S^T of the run's last tile, the last matrix work that reads the query rows
+            // in place -- a step and a half before they are waited for; in the last step where there was no
+            // such step, or a plain one)
+            bool queries_asked = false;
             auto step = [&](int r, bool cur_is_a) {
                 if constexpr (DISTINCT) {  // (unit r landed before the step that read its K tile; every wave comes here)
                     const TileInfo tr = at.tile_info_of(r);
@@ -1446,20 +1450,25 @@ paged_attn_pipe_kernel(const KArgs a) {
                 }
                 const bool has_next = r + 1 < run_end;
                 const bool fetch = has_next && admit(r + 1, r);
-                if (!has_next && next_opens) at.request_queries(at.units[run_end]);
+                if (!has_next && next_opens && !queries_asked) at.request_queries(at.units[run_end]);
+                const bool ask_queries = next_opens && r + 2 == run_end;
+                queries_asked = queries_asked || ask_queries;
                 if (!compute_first || !busy) {
                     if (fetch) at.issue_unit(issued);
                     if (busy) prepare();
                 }
+                if (!busy && ask_queries) at.request_queries(at.units[run_end]);
                 if (busy) {
                     const uint32_t v_cur = at.lds_address(tile_of(r) + C::MAT_BYTES) + at.v_lane;
                     if (has_next) {
                         const uint32_t k_next = at.lds_address(tile_of(r + 1)) + at.k_lane;
                         if (cur_is_a) {
                             PB::step_ab_x(k_next, v_cur, a.c, neg_m, at.l_run[0]);
+                            if (ask_queries) at.request_queries(at.units[run_end]);
                             PB::step_ab_y(a.c, neg_m, at.l_run[0], mx_lane);
                         } else {
                             PB::step_ba_x(k_next, v_cur, a.c, neg_m, at.l_run[0]);
+                            if (ask_queries) at.request_queries(at.units[run_end]);
                             PB::step_ba_y(a.c, neg_m, at.l_run[0], mx_lane);
                         }
                         mask(r + 1, !cur_is_a, mx_lane);

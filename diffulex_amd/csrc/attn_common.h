@@ -500,8 +500,25 @@ struct AttnState {
         }
     }
 
-    // Merge one stored piece into the running state (l_run holds whole-row sums here).
-    DFX_D void merge_partial(int slot) {
+    // HIDDEN kernels: the wave's block of the stored piece `slot` on its way into the registers of the score
+    // sets (free between two runs), all nine loads at once -- through the compiler's few registers they would go
+    // three at a time, a trip to memory each.  Asked for before this workgroup rounds its own piece, which takes
+    // as long as the trip.
+    DFX_D void request_partial(int slot) const {
+        static_assert(HIDDEN && NB == 1, "registers of attn_pipe_gen.h");
+        if (wave >= a.busy_waves) return;
+        int w = wave;
+        asm volatile("" : "+v"(w));
+        const uint8_t* p = reinterpret_cast<const uint8_t*>(slot_ptr(slot) + w * S::BLOCK_FLOATS) + lane_here() * 16;
+        pipe_request_partial(p, p + 3 * 1024, p + 6 * 1024);
+    }
+
+    // Merge one stored piece into the running state (l_run holds whole-row sums here): the piece in `slot`, or
+    // (REQUESTED) the one request_partial() has asked for.
+    DFX_D void merge_partial(int slot) { merge_partial_from<false>(slot); }
+    DFX_D void merge_requested_partial() { merge_partial_from<true>(0); }
+    template <bool REQUESTED>
+    DFX_D void merge_partial_from(int slot) {
         // No fused multiply-add in here: a * wa + b * wb must round both products, or merging a
         // into b and b into a differ in the last bit (an fma keeps one product exact, and which
         // one depends on who merges).  __fmul_rn / __fadd_rn would not do: they are plain operators
@@ -509,11 +526,17 @@ struct AttnState {
 #pragma clang fp contract(off)
         if (wave >= a.busy_waves) return;
         const int lane = lane_here();
+        if constexpr (REQUESTED) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 #pragma unroll
         for (int qb = 0; qb < NB; ++qb) {
-            const __amdgpu_buffer_rsrc_t rs = block_resource(slot, qb);
-            const f32x4 st = __builtin_bit_cast(
-                f32x4, __builtin_amdgcn_raw_buffer_load_b128(rs, kStatsOff + lane * 16, 0, kDeviceScope));
+            __amdgpu_buffer_rsrc_t rs;
+            if constexpr (!REQUESTED) rs = block_resource(slot, qb);
+            // piece c of the block: chunks 0 .. kChunks - 1, then the statistics
+            auto piece = [&](int c) {
+                if constexpr (REQUESTED) return __builtin_bit_cast(u32x4v, pipe_partial_chunk(c));
+                else return __builtin_amdgcn_raw_buffer_load_b128(rs, (c * 64 + lane) * 16, 0, kDeviceScope);
+            };
+            const f32x4 st = __builtin_bit_cast(f32x4, piece(kChunks));
             const float mp = st[0], lp = st[1], up = st[2];
             const float mn = fmaxf(m_run[qb], mp);
             const float wa = (m_run[qb] == -INFINITY) ? 0.0f : fast_exp2(m_run[qb] - mn);
@@ -529,7 +552,7 @@ struct AttnState {
 #pragma unroll
                 for (int hc = 0; hc < 2; ++hc) {
                     const int c = db * 2 + hc, e0 = hc * 8;
-                    const u32x4v w = __builtin_amdgcn_raw_buffer_load_b128(rs, (c * 64 + lane) * 16, 0, kDeviceScope);
+                    const u32x4v w = piece(c);
                     const uint32_t ws[4] = {w.x, w.y, w.z, w.w};
 #pragma unroll
                     for (int j = 0; j < 4; ++j) {
@@ -624,8 +647,15 @@ DFX_D bool finish_cut_item(AttnState<HD, NB, NW, HIDDEN>& at, int rt, int64_t it
             __syncthreads();
             if (!sibling_there) return false;  // the sibling's carrier will find this state
         }
-        at.round_to_stored_form();
-        at.merge_partial(slot_of_piece(later_half ? second - half : second));
+        const int other = slot_of_piece(later_half ? second - half : second);
+        if constexpr (HIDDEN) {
+            at.request_partial(other);
+            at.round_to_stored_form();
+            at.merge_requested_partial();
+        } else {
+            at.round_to_stored_form();
+            at.merge_partial(other);
+        }
         if (threadIdx.x == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         j &= ~(2 * half - 1);
     }

@@ -504,6 +504,36 @@ namespace dfx {
                                 "stage 0) into the widened tiles at wide_k and wide_v (byte offsets from widened tile 0): both reads first,\n"
                                 "one instruction per pair of codes (exact), in the operand ring's registers, which are free between the\n"
                                 "blocks of two steps.  The writes are waited for by whatever waits for LDS next (lgkmcnt)."))
+    # a stored piece of a cut item (a block of 8 chunks and the statistics, 1 KiB apart, 16 bytes per lane) into
+    # score set A and the first registers of set B, all nine loads in flight at once
+    req = []
+    for c in range(9):
+        req.append(f"global_load_dwordx4 {vr(SA + 4 * c, 4)}, %[p{c // 3}], off offset:{(c % 3) * 1024} sc1")
+    parts.append(asm_fn("pipe_request_partial", "const void* p0, const void* p1, const void* p2", join(req),
+                        ins=['[p0] "v"(p0)', '[p1] "v"(p1)', '[p2] "v"(p2)'], clobbers=["memory"],
+                        comment="Requests the lane's nine 16-byte pieces of a stored block (p0: the lane's address in the block's first\n"
+                                "chunk; p1, p2: 3 and 6 KiB further) with device scope into the score sets, which are free between two\n"
+                                "runs.  The caller waits for the loads (vmcnt) before pipe_partial_chunk()."))
+    for c in range(9):
+        outs = [f'"=v"(x[{e}])' for e in range(4)]
+        body = join(f"v_mov_b32 %{e}, {vr(SA + 4 * c + e)}" for e in range(4))
+        parts.append(f'''DFX_D u32x4 pipe_partial_chunk_{c}() {{
+    uint32_t x[4];
+    asm volatile("{body}"
+                 : {", ".join(outs)});
+    return u32x4{{x[0], x[1], x[2], x[3]}};
+}}
+
+''')
+    parts.append('''// Piece c (0..7: chunks, 8: the statistics; a compile-time constant after unrolling) of what
+// pipe_request_partial() has loaded.
+DFX_D u32x4 pipe_partial_chunk(int c) {
+    switch (c) {
+''' + "".join(f"        case {c}: return pipe_partial_chunk_{c}();\n" for c in range(8)) + '''        default: return pipe_partial_chunk_8();
+    }
+}
+
+''')
     parts.append(rope_queries_fns())
     parts.append(rope_row_fn())
     for d in range(NDB):

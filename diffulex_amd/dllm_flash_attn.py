@@ -169,12 +169,29 @@ def plan_key(q, k, k_cache, fp8, tail, meta, capture_id, v_cache=None):
             meta[2].numel() - 1, tuple(_content_token(t) for t in meta), int(capture_id))
 
 
+# Launches whose units (an upper bound from the shapes) number fewer than this per workgroup are not planned.
+PLAN_MIN_UNITS_PER_WORKGROUP = 2
+_cu_count = {}
+
+
+def _compute_units(device) -> int:
+    n = _cu_count.get(device.index)
+    if n is None:
+        n = _cu_count[device.index] = torch.cuda.get_device_properties(device).multi_processor_count
+    return n
+
+
 def _build_plan(ops, head, tail, group, max_seqlen_q, num_seqs, max_pages, page_size, t_new):
     """Launch ``dfx_paged_attn_plan`` for this configuration; None where no plan applies (generic
     tile path).  The unit capacity is an upper bound from the shapes alone: no device data is read."""
     row_tiles = -(-group * max_seqlen_q // 128)
     tiles = num_seqs * (-(-max_pages * page_size // 64) + 1) + t_new // 64
     h_kv = head[1].shape[1]
+    # (a launch of at most a tile or two per compute unit has nothing to plan: the plan kernels would cost
+    # it more than they save -- 2 sequences x 2 KV heads of 3 tiles: 15.2 us with a plan, 12.4 without)
+    n_wg = tail[4] if tail[4] > 0 else _compute_units(head[0].device)   # (max_workgroups, or a workgroup per compute unit)
+    if h_kv * row_tiles * tiles < PLAN_MIN_UNITS_PER_WORKGROUP * n_wg:
+        return None
     nbytes = int(ops.paged_attention_plan_bytes(*head, None, *tail, h_kv * row_tiles * tiles))
     if nbytes < 0:
         return None

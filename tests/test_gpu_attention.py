@@ -9,6 +9,7 @@ import torch
 
 import diffulex_amd as dfx
 from diffulex_amd import _lib
+from diffulex_amd import dllm_flash_attn as dfa
 from diffulex_amd.workloads import make_workload, MASK_FULL, MASK_BLOCK_CAUSAL
 from util import ATOL_BF16, ATOL_FP8, metadata_for, oracle_fp32, max_abs_err
 
@@ -318,11 +319,12 @@ STREAMED_DISTINCT = [
 
 @pytest.mark.parametrize("name,over,max_wg", STREAMED_DISTINCT)
 @pytest.mark.parametrize("planned", [False, True])
-def test_distinct_layout_on_the_streaming_path(dev, name, over, max_wg, planned):
+def test_distinct_layout_on_the_streaming_path(dev, name, over, max_wg, planned, monkeypatch):
     """head_dim 128 and pages of a multiple of 64 tokens: the distinct layout streams (K tile chunk-major, V tile
     d-major, the layout's own shapes).  Against the oracle, and against the generic kernel on the same cache; what
     lies in a page behind a sequence's end (NaN here, in K and in V) must not reach the result, nor must a page
     without a table entry."""
+    monkeypatch.setattr(dfa, "PLAN_MIN_UNITS_PER_WORKGROUP", 0)   # (plan the tiny cases too)
     wl = make_workload(name, seed=97, **over)
     bt = wl.block_tables.clone()
     if wl.num_seqs > 2 and int(wl.context_lens[2]) > wl.page_size:
@@ -1005,9 +1007,10 @@ def _read_plan(plan, num_seqs, n_wg):
 
 @pytest.mark.parametrize("name,over", PLAN_CASES)
 @pytest.mark.parametrize("max_wg", [0, 7])
-def test_planned_launch_with_equal_ranges_gives_the_same_bits(dev, name, over, max_wg):
+def test_planned_launch_with_equal_ranges_gives_the_same_bits(dev, name, over, max_wg, monkeypatch):
     """With equal ranges the plan describes the partition the kernels work out for themselves:
     reading it must not change a bit."""
+    monkeypatch.setattr(dfa, "PLAN_MIN_UNITS_PER_WORKGROUP", 0)   # (plan the tiny cases too)
     wl = make_workload(name, device=dev, **over)
     want = _run(wl, max_wg)
     cache = {}
@@ -1020,10 +1023,11 @@ def test_planned_launch_with_equal_ranges_gives_the_same_bits(dev, name, over, m
 @pytest.mark.parametrize("name,over", PLAN_CASES + [("c3", dict(num_seqs=40, ctx=(64, 1500))),
                                                     ("c3", dict(num_seqs=24, ctx=[70] * 12 + [2900] * 12))])
 @pytest.mark.parametrize("max_wg", [0, 7, 40])
-def test_planned_launch_with_cut_points_placed_by_cost(dev, name, over, max_wg):
+def test_planned_launch_with_cut_points_placed_by_cost(dev, name, over, max_wg, monkeypatch):
     """The default plan: ranges of equal cost, cut points moved onto a sequence's first unit where one is
     near.  Other pieces are merged than without a plan, so the rows differ in the last bits only;
     every launch with the plan gives the same bits; the ranges tile the unit space."""
+    monkeypatch.setattr(dfa, "PLAN_MIN_UNITS_PER_WORKGROUP", 0)   # (plan the tiny cases too)
     wl = make_workload(name, device=dev, **over)
     cache = {}
     got = _run(wl, max_wg, plan_cache=cache)
@@ -1158,3 +1162,14 @@ def test_plan_made_for_another_configuration_is_ignored(dev):
     got2 = _run(wl, plan_cache=p_cache)
     assert max_abs_err(got2, want) <= 1e-2 and torch.equal(got2, want)
     assert max_abs_err(out, want) <= 1e-2
+
+
+def test_a_launch_of_a_few_tiles_is_not_planned(dev):
+    """The operators skip the plan where a launch has at most a tile or two per workgroup (the plan kernels
+    would take longer than they save); the launch plans for itself then, as without a plan cache."""
+    wl = make_workload("c1", device=dev)
+    cache = {}
+    got = _run(wl, plan_cache=cache)
+    assert list(cache.values()) == [None]
+    assert torch.equal(got, _run(wl))
+    assert max_abs_err(got, oracle_fp32(wl)) <= ATOL_BF16

@@ -76,7 +76,8 @@ int make_plan(const dfx_attn_params* p, Plan& plan) {
     const bool dstream = plan.distinct && !(p->flags & DFX_ATTN_GENERIC_PATH) && plan.hd == 128 && p->page_size > 0 &&
                          p->page_size % 64 == 0 && p->page_size < (1 << 20) && p->kn_stride_head == p->vn_stride_head &&
                          p->kc_stride[4] == 1 && p->kc_stride[3] == 8 && p->vc_stride[3] == 1 &&
-                         p->vc_stride[2] >= 0 && p->vc_stride[2] < (1 << 22) && p->rope_cos_sin == nullptr;
+                         p->vc_stride[2] >= 0 && p->vc_stride[2] < (1 << 22) && p->rope_cos_sin == nullptr &&
+                         p->num_kv_heads < (1 << 12) && p->n_pages < (1ll << 32);  // (what a tile's descriptor packs)
     if (dstream) {
         plan.stream = true;
         plan.nb = 2;

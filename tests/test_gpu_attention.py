@@ -1173,3 +1173,57 @@ def test_a_launch_of_a_few_tiles_is_not_planned(dev):
     assert list(cache.values()) == [None]
     assert torch.equal(got, _run(wl))
     assert max_abs_err(got, oracle_fp32(wl)) <= ATOL_BF16
+
+
+def test_distinct_layout_in_a_captured_graph_and_through_the_static_entry(dev):
+    """The distinct layout's streaming kernel the ways a serving loop reaches it: Attention.forward captured in a
+    graph and replayed (the plan built inside the capture, eager launches between the replays), and the entry point
+    that allocates nothing."""
+    wl = make_workload("c3", num_seqs=6, ctx=(300, 1200), seed=45).to(dev)
+    want = oracle_fp32(wl)
+    att = dfx.Attention(wl.num_q_heads, wl.head_dim, wl.scale, wl.num_kv_heads)
+    att.k_cache, att.v_cache = _to_distinct(wl.k_cache)[0], _to_distinct(wl.v_cache)[1]
+    md = metadata_for(wl, "static")
+    md.kv_cache_layout = "distinct"
+    dfx.set_fetch_fn_for_attn_metadata(lambda: md)
+    t = wl.q.shape[0]
+    q, k, v = (x.reshape(t, -1).clone() for x in (wl.q, wl.k_new, wl.v_new))
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        eager = att(q, k, v)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    assert max_abs_err(eager.view(t, wl.num_q_heads, wl.head_dim), want) <= ATOL_BF16
+    kc0, vc0 = att.k_cache.clone(), att.v_cache.clone()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        o_static = att(q, k, v)
+    for _ in range(3):
+        graph.replay()
+        att(q, k, v)               # eager work between the replays
+        torch.cuda.synchronize()
+        assert torch.equal(o_static, eager)
+    assert torch.equal(att.k_cache, kc0) and torch.equal(att.v_cache, vc0)   # (the same block stored again)
+    out = torch.empty_like(wl.q)
+    got = dfx.paged_attention(wl.q, wl.k_new, wl.v_new, att.k_cache, att.v_cache, wl.scale, out=out, static_scratch=True,
+                              cache_layout="distinct", block_tables=wl.block_tables, context_lens=wl.context_lens,
+                              cu_seqlens_q=wl.cu_seqlens_q, cu_seqlens_new=wl.cu_seqlens_q, max_seqlen_q=wl.q_len,
+                              mask_mode=wl.mask_mode, diffusion_block_size=wl.diffusion_block_size)
+    torch.cuda.synchronize()
+    assert max_abs_err(got, want) <= ATOL_BF16
+
+
+@pytest.mark.parametrize("ctx", [[0, 0, 700, 0, 64], [900, 5, 5, 5, 900, 5], [64, 64]])
+def test_reordered_plan_with_sequences_of_no_or_few_tiles(dev, ctx):
+    """The plan's second order of the sequences (k-th longest, k-th shortest) on batches whose short sequences have
+    no context at all, or are all alike, or are too few for a second order: the same rows as the batch's order up to
+    the rounding of other merges, and as the oracle."""
+    wl = make_workload("c3", num_seqs=len(ctx), ctx=ctx, seed=47).to(dev)
+    want = oracle_fp32(wl)
+    for max_wg in (0, 6):
+        got = _run(wl, max_wg, plan_cache={})
+        kept = _run(wl, max_wg, plan_cache={}, flags=_lib.DFX_ATTN_BATCH_ORDER)
+        torch.cuda.synchronize()
+        assert max_abs_err(got, want) <= ATOL_BF16
+        assert max_abs_err(got, kept) <= 1e-2

@@ -116,3 +116,37 @@ def test_shapes_without_a_pipelined_kernel_refuse_the_rope_and_the_module_falls_
     att2 = dfx.Attention(hq, hd, wl.scale, hkv)
     att2.k_cache, att2.v_cache = wl.k_cache.clone(), wl.v_cache.clone()
     assert torch.equal(_bits(out), _bits(att2(rq, rk, wl.v_new.reshape(T, -1))))
+
+
+def test_rope_inside_the_launch_in_a_captured_graph(dev):
+    """The one-launch layer step captured and replayed, with new projections in the same tensors between the
+    replays: every replay equals the eager two-launch result on the same inputs."""
+    wl = make_workload("c3", num_seqs=6, ctx=(300, 900), seed=7).to(dev)
+    T, hq, hkv, hd = wl.q.shape[0], wl.num_q_heads, wl.num_kv_heads, wl.head_dim
+    rope = RotaryEmbedding(hd, hd, MAXPOS, BASE).to(dev)
+    att = dfx.Attention(hq, hd, wl.scale, hkv)
+    att.k_cache, att.v_cache = wl.k_cache.clone(), wl.v_cache.clone()
+    md = metadata_for(wl, "static")
+    dfx.set_fetch_fn_for_attn_metadata(lambda: md)
+    g = torch.Generator("cpu").manual_seed(9)
+    qkv = torch.randn(T, (hq + 2 * hkv) * hd, generator=g).to(torch.bfloat16).to(dev)
+    pos = torch.randint(0, MAXPOS, (T,), generator=g).to(dev)
+    q, k, v = qkv.split([hq * hd, hkv * hd, hkv * hd], dim=-1)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        att(q, k, v, rope=(rope, pos))       # warm-up on the capture stream
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        o_static = att(q, k, v, rope=(rope, pos))
+    for i in range(3):
+        qkv.copy_(torch.randn(qkv.shape, generator=g).to(torch.bfloat16))
+        graph.replay()
+        torch.cuda.synchronize()
+        cache_after = att.k_cache.clone()
+        rq, rk = rope(pos, q, k)             # the two launches, eagerly, on the same inputs
+        want = att(rq, rk, v)
+        torch.cuda.synchronize()
+        assert torch.equal(_bits(o_static), _bits(want)), i
+        assert torch.equal(_bits(att.k_cache), _bits(cache_after)), i

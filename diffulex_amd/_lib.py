@@ -10,7 +10,7 @@ from pathlib import Path
 
 LIB_PATH = Path(__file__).resolve().parent / "libdiffulex_amd.so"
 
-DFX_ABI_VERSION = 7
+DFX_ABI_VERSION = 8
 DFX_OK = 0
 DFX_KV_BF16, DFX_KV_FP8_E4M3 = 0, 1
 DFX_MASK_FULL, DFX_MASK_BLOCK_CAUSAL = 0, 1
@@ -71,6 +71,7 @@ class RopeParams(C.Structure):
         ("k_cache", C.c_void_p), ("v_cache", C.c_void_p),
         ("slot_mapping", C.c_void_p), ("slot_index_type", C.c_int32), ("n_slots", C.c_int64),
         ("k_scale", C.c_void_p), ("v_scale", C.c_void_p),
+        ("cache_layout", C.c_int32), ("page_size", C.c_int32), ("kc_stride", C.c_int64 * 3), ("vc_stride", C.c_int64 * 3),
     ]
 
 

@@ -31,18 +31,25 @@ class Attention(nn.Module):
         """``rope=(rotary_embedding, positions)`` (extension): q and k are the projections BEFORE the rotary
         embedding (diffulex/model/dream.py:94-99 applies it right before this call); it is applied inside
         the attention launch where that launch can (decode, unified layout, ``rope_supported``), by the
-        rotary embedding's own launch otherwise."""
+        rotary embedding's own launch otherwise -- which then also stores the block, in either cache layout,
+        where a store is due."""
+        stored = False
         if rope is not None:
             rotary, positions = rope
             md = self.fetch_attn_metadata()
             fused = (not md.is_prefill and md.kv_cache_layout == "unified" and self.k_cache.numel() > 0 and
                      rope_supported(self.num_heads, self.num_kv_heads, self.head_dim, int(md.max_seqlen_q or 0),
                                     self.k_cache.shape[1], md.cu_seqlens_q.numel() - 1, q.device))
-            if not fused:
-                q, k = rotary(positions, q, k)
-                rope = None
-            else:
+            if fused:
                 rope = (rotary.cos_sin_cache, positions)
+            else:
+                rope = None
+                if (self.k_cache.numel() and self.v_cache.numel() and md.need_kv_cache_store
+                        and self.k_cache.dtype == torch.bfloat16 and md.slot_mapping.numel() == k.shape[0]):
+                    q, k = rotary.forward_and_store(positions, q, k, v, self.k_cache, self.v_cache, md.slot_mapping, md)
+                    stored = True
+                else:
+                    q, k = rotary(positions, q, k)
         q = q.view(q.shape[0], self.num_heads, self.head_dim)
         k = k.view(k.shape[0], self.num_kv_heads, self.head_dim)
         v = v.view(v.shape[0], self.num_kv_heads, self.head_dim)
@@ -55,7 +62,7 @@ class Attention(nn.Module):
         # stored follows the attended context, so the two never touch the same slots).
         fused_slots = None
         if k_cache.numel() and v_cache.numel():
-            if attn_metadata.need_kv_cache_store:
+            if attn_metadata.need_kv_cache_store and not stored:
                 slots = attn_metadata.slot_mapping
                 # (worth it while the block is small: measured on an MI355X the fused form saves a
                 # launch's worth of time up to about 4 MB of fresh K+V and loses beyond 8 MB, where a

@@ -6,6 +6,7 @@
 // registers between the load and the (half-width) store.
 #include "dfx_common.h"
 #include "fp8_e4m3.h"
+#include "distinct_tile.h"
 
 namespace dfx {
 namespace {
@@ -100,7 +101,7 @@ kv_store_distinct_kernel(const uint16_t* __restrict__ key, const uint16_t* __res
 // column of consecutive tokens (their 16-byte pieces are adjacent in the cache when their slots
 // are), and V leaves transposed, eight consecutive tokens of one d per store where those eight
 // have consecutive slots starting at a multiple of 8 in one page (two bytes at a time otherwise).
-constexpr int kDistinctTokens = 16;
+constexpr int kDistinctTokens = DistinctTile<128>::kTokens;
 
 template <typename SlotT, int HD>
 __global__ void __launch_bounds__(kThreads)
@@ -108,10 +109,9 @@ kv_store_distinct_tiled(const uint16_t* __restrict__ key, const uint16_t* __rest
                         int64_t value_stride, uint16_t* __restrict__ k_cache, uint16_t* __restrict__ v_cache,
                         DistinctStrides st, const SlotT* __restrict__ slots, int64_t n_tokens, int64_t n_pages,
                         int page_size) {
-    constexpr int CPR = HD / 8;             // 16-byte chunks per row
-    constexpr int VPITCH = HD * 2 + 4;      // V rows padded by one word: column reads then spread over the banks
-    __shared__ __attribute__((aligned(16))) uint8_t k_tile[kDistinctTokens * HD * 2];
-    __shared__ __attribute__((aligned(16))) uint8_t v_tile[kDistinctTokens * VPITCH];
+    using Tile = DistinctTile<HD>;
+    __shared__ __attribute__((aligned(16))) uint8_t k_tile[Tile::K_BYTES];
+    __shared__ __attribute__((aligned(16))) uint8_t v_tile[Tile::V_BYTES];
     __shared__ int64_t slot_of[kDistinctTokens];
     const int64_t t0 = static_cast<int64_t>(blockIdx.x) * kDistinctTokens;
     const int h = blockIdx.y;
@@ -122,57 +122,19 @@ kv_store_distinct_tiled(const uint16_t* __restrict__ key, const uint16_t* __rest
         if (slot >= 0 && slot / page_size >= n_pages) slot = -1;
         slot_of[tid] = slot;
     }
-    for (int c = tid; c < kDistinctTokens * CPR; c += kThreads) {
-        const int r = c / CPR, cc = c % CPR;
+    for (int c = tid; c < kDistinctTokens * Tile::CPR; c += kThreads) {
+        const int r = c / Tile::CPR, cc = c % Tile::CPR;
         const int64_t t = t0 + r;
         u32x4 kk = {0, 0, 0, 0}, vv = {0, 0, 0, 0};
         if (t < n_tokens) {
             kk = *reinterpret_cast<const u32x4*>(key + t * key_stride + h * HD + cc * 8);
             vv = *reinterpret_cast<const u32x4*>(value + t * value_stride + h * HD + cc * 8);
         }
-        *reinterpret_cast<u32x4*>(k_tile + r * (HD * 2) + ((cc ^ (r % CPR)) * 16)) = kk;
-        uint32_t* vrow = reinterpret_cast<uint32_t*>(v_tile + r * VPITCH + cc * 16);
-        vrow[0] = vv.x; vrow[1] = vv.y; vrow[2] = vv.z; vrow[3] = vv.w;
+        *reinterpret_cast<u32x4*>(k_tile + Tile::k_offset(r, cc)) = kk;
+        Tile::put_v(v_tile, r, cc, vv);
     }
     __syncthreads();
-    // K: consecutive lanes take consecutive tokens of one chunk column
-    for (int c = tid; c < kDistinctTokens * CPR; c += kThreads) {
-        const int r = c % kDistinctTokens, cc = c / kDistinctTokens;
-        const int64_t slot = slot_of[r];
-        if (slot < 0) continue;
-        const int64_t blk = slot / page_size, off = slot - blk * page_size;
-        const u32x4 kk = *reinterpret_cast<const u32x4*>(k_tile + r * (HD * 2) + ((cc ^ (r % CPR)) * 16));
-        *reinterpret_cast<u32x4*>(k_cache + blk * st.k[0] + h * st.k[1] + cc * st.k[2] + off * 8) = kk;
-    }
-    // V: eight consecutive lanes take the eight 8-token groups of one d
-    for (int c = tid; c < (kDistinctTokens / 8) * HD; c += kThreads) {
-        const int tg = c % (kDistinctTokens / 8), d = c / (kDistinctTokens / 8);
-        const int r0 = tg * 8;
-        uint16_t e[8];
-#pragma unroll
-        for (int j = 0; j < 8; ++j) e[j] = *reinterpret_cast<const uint16_t*>(v_tile + (r0 + j) * VPITCH + d * 2);
-        const int64_t s0 = slot_of[r0];
-        bool run = s0 >= 0 && (s0 % 8) == 0 && (s0 % page_size) + 8 <= page_size;
-#pragma unroll
-        for (int j = 1; j < 8; ++j) run = run && slot_of[r0 + j] == s0 + j;
-        if (run) {
-            const int64_t blk = s0 / page_size, off = s0 - blk * page_size;
-            u32x4 w;
-            w.x = e[0] | (static_cast<uint32_t>(e[1]) << 16);
-            w.y = e[2] | (static_cast<uint32_t>(e[3]) << 16);
-            w.z = e[4] | (static_cast<uint32_t>(e[5]) << 16);
-            w.w = e[6] | (static_cast<uint32_t>(e[7]) << 16);
-            *reinterpret_cast<u32x4*>(v_cache + blk * st.v[0] + h * st.v[1] + d * st.v[2] + off) = w;
-        } else {
-#pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                const int64_t slot = slot_of[r0 + j];
-                if (slot < 0) continue;
-                const int64_t blk = slot / page_size, off = slot - blk * page_size;
-                v_cache[blk * st.v[0] + h * st.v[1] + d * st.v[2] + off] = e[j];
-            }
-        }
-    }
+    Tile::store(k_tile, v_tile, slot_of, k_cache, v_cache, st.k, st.v, h, page_size, tid, kThreads);
 }
 
 // ---------------------------------------------------------------- load (gather)

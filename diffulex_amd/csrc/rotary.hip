@@ -6,9 +6,11 @@
 // its positions' angle table row, rotates in fp32 exactly as the reference does (two rounded
 // products, one rounded sum, then round-to-nearest-even to bf16), writes both chunks back and,
 // for K, also into the row's cache slot; V lanes only copy into the cache.  Consecutive lanes
-// cover consecutive chunks, so a wavefront moves whole runs of a token row.
+// cover consecutive chunks, so a wavefront moves whole runs of a token row.  (A cache in the distinct layout is
+// written by workgroups of their own, 16 tokens of a KV head each, through LDS: rope_store_distinct_kernel.)
 #include "dfx_common.h"
 #include "fp8_e4m3.h"
+#include "distinct_tile.h"
 
 namespace dfx {
 namespace {
@@ -32,6 +34,9 @@ struct RopeArgs {
     int64_t n_slots;
     const float* k_scale;
     const float* v_scale;
+    // distinct layout (bf16): K [pages, h_kv, hd / 8, page, 8], V [pages, h_kv, hd, page], strides in elements
+    int distinct, page_size;
+    int64_t kd[3], vd[3];
 };
 
 DFX_D u32x4 pack8(const float (&y)[8]) {
@@ -66,12 +71,35 @@ DFX_D void rotate8(const float (&x1)[8], const float (&x2)[8], const float (&c)[
     }
 }
 
+// The chunk pair (lo, hi = lo + hd / 2) of the head row at `src` rotated by the angles of position `pos`.
+template <typename PosT>
+DFX_D void rotate_pair(const RopeArgs& a, const uint16_t* src, const PosT* __restrict__ positions, int64_t t, int lo, int hi,
+                       u32x4& o1, u32x4& o2) {
+    const u32x4 w1 = *reinterpret_cast<const u32x4*>(src + lo);
+    const u32x4 w2 = *reinterpret_cast<const u32x4*>(src + hi);
+    // a position outside the table is a caller error (the reference's gather would fail); it is
+    // clamped here so that no lane reads outside the table
+    int64_t pos = static_cast<int64_t>(positions[t]);
+    pos = pos < 0 ? 0 : (pos >= a.max_position ? a.max_position - 1 : pos);
+    const float* row = a.table + pos * a.hd;
+    float cs[8], sn[8];
+    *reinterpret_cast<f32x4*>(cs) = *reinterpret_cast<const f32x4*>(row + lo);
+    *reinterpret_cast<f32x4*>(cs + 4) = *reinterpret_cast<const f32x4*>(row + lo + 4);
+    *reinterpret_cast<f32x4*>(sn) = *reinterpret_cast<const f32x4*>(row + hi);
+    *reinterpret_cast<f32x4*>(sn + 4) = *reinterpret_cast<const f32x4*>(row + hi + 4);
+    float x1[8], x2[8], y1[8], y2[8];
+    unpack8(w1, x1);
+    unpack8(w2, x2);
+    rotate8(x1, x2, cs, sn, y1, y2);
+    o1 = pack8(y1);
+    o2 = pack8(y2);
+}
+
+// One thread's work of the flat launch: work item idx of n_tokens * (h_q + h_kv + v_heads) * hd / 16.
 template <bool FP8, typename PosT, typename SlotT>
-__global__ void __launch_bounds__(kThreads)
-rope_kv_store_kernel(const RopeArgs a, const PosT* __restrict__ positions, const SlotT* __restrict__ slots) {
+DFX_D void rope_work_item(const RopeArgs& a, const PosT* __restrict__ positions, const SlotT* __restrict__ slots, int64_t idx) {
     const int cph = a.hd >> 4;  // chunk pairs per head row
     const int slots_per_token = (a.h_q + a.h_kv + a.v_heads) * cph;
-    const int64_t idx = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
     if (idx >= a.n_tokens * slots_per_token) return;
     const int64_t t = idx / slots_per_token;
     const int r = static_cast<int>(idx - t * slots_per_token);
@@ -109,23 +137,8 @@ rope_kv_store_kernel(const RopeArgs a, const PosT* __restrict__ positions, const
     const int h = is_k ? head - a.h_q : head;
     const uint16_t* src = is_k ? a.k + t * a.k_st + h * a.hd : a.q + t * a.q_st + h * a.hd;
     uint16_t* dst = is_k ? a.k_out + t * a.ko_st + h * a.hd : a.q_out + t * a.qo_st + h * a.hd;
-    const u32x4 w1 = *reinterpret_cast<const u32x4*>(src + lo);
-    const u32x4 w2 = *reinterpret_cast<const u32x4*>(src + hi);
-    // a position outside the table is a caller error (the reference's gather would fail); it is
-    // clamped here so that no lane reads outside the table
-    int64_t pos = static_cast<int64_t>(positions[t]);
-    pos = pos < 0 ? 0 : (pos >= a.max_position ? a.max_position - 1 : pos);
-    const float* row = a.table + pos * a.hd;
-    float cs[8], sn[8];
-    *reinterpret_cast<f32x4*>(cs) = *reinterpret_cast<const f32x4*>(row + lo);
-    *reinterpret_cast<f32x4*>(cs + 4) = *reinterpret_cast<const f32x4*>(row + lo + 4);
-    *reinterpret_cast<f32x4*>(sn) = *reinterpret_cast<const f32x4*>(row + hi);
-    *reinterpret_cast<f32x4*>(sn + 4) = *reinterpret_cast<const f32x4*>(row + hi + 4);
-    float x1[8], x2[8], y1[8], y2[8];
-    unpack8(w1, x1);
-    unpack8(w2, x2);
-    rotate8(x1, x2, cs, sn, y1, y2);
-    const u32x4 o1 = pack8(y1), o2 = pack8(y2);
+    u32x4 o1, o2;
+    rotate_pair(a, src, positions, t, lo, hi, o1, o2);
     *reinterpret_cast<u32x4*>(dst + lo) = o1;
     *reinterpret_cast<u32x4*>(dst + hi) = o2;
     if (is_k && slot >= 0) {
@@ -140,6 +153,88 @@ rope_kv_store_kernel(const RopeArgs a, const PosT* __restrict__ positions, const
             *reinterpret_cast<u32x4*>(kc + hi) = o2;
         }
     }
+}
+
+template <bool FP8, typename PosT, typename SlotT>
+__global__ void __launch_bounds__(kThreads)
+rope_kv_store_kernel(const RopeArgs a, const PosT* __restrict__ positions, const SlotT* __restrict__ slots) {
+    rope_work_item<FP8>(a, positions, slots, static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x);
+}
+
+// The same with the store going into a cache in the distinct layout (bf16).  The first q_blocks workgroups rotate
+// the Q rows as above; each of the others takes 16 tokens of one KV head: rotates their K rows (k_out receives
+// them as well), stages them and the V rows in LDS and writes both the way dfx_kv_store_distinct does
+// (distinct_tile.h) -- one chunk at a time from the rotating threads, the V rows would leave two bytes at a time.
+template <typename PosT, typename SlotT, int HD>
+__global__ void __launch_bounds__(kThreads)
+rope_store_distinct_kernel(const RopeArgs a, const PosT* __restrict__ positions, const SlotT* __restrict__ slots, int q_blocks) {
+    using Tile = DistinctTile<HD>;
+    __shared__ __attribute__((aligned(16))) uint8_t k_tile[Tile::K_BYTES];
+    __shared__ __attribute__((aligned(16))) uint8_t v_tile[Tile::V_BYTES];
+    __shared__ int64_t slot_of[Tile::kTokens];
+    const int tid = threadIdx.x;
+    if (static_cast<int>(blockIdx.x) < q_blocks) {
+        RopeArgs q_only = a;
+        q_only.h_kv = q_only.v_heads = 0;
+        rope_work_item<false>(q_only, positions, static_cast<const SlotT*>(nullptr), static_cast<int64_t>(blockIdx.x) * kThreads + tid);
+        return;
+    }
+    const int tile = static_cast<int>(blockIdx.x) - q_blocks;
+    const int h = tile % a.h_kv;
+    const int64_t t0 = static_cast<int64_t>(tile / a.h_kv) * Tile::kTokens;
+    if (tid < Tile::kTokens) {
+        const int64_t t = t0 + tid;
+        int64_t slot = t < a.n_tokens ? static_cast<int64_t>(slots[t]) : -1;
+        if (slot >= a.n_slots) slot = -1;
+        slot_of[tid] = slot;
+    }
+    constexpr int cph = HD / 16;
+    for (int w = tid; w < Tile::kTokens * cph; w += kThreads) {
+        const int r = w / cph, c = w % cph;
+        const int64_t t = t0 + r;
+        u32x4 o1 = {0, 0, 0, 0}, o2 = {0, 0, 0, 0};
+        if (t < a.n_tokens) {
+            const int lo = c * 8, hi = lo + HD / 2;
+            rotate_pair(a, a.k + t * a.k_st + h * HD, positions, t, lo, hi, o1, o2);
+            uint16_t* dst = a.k_out + t * a.ko_st + h * HD;
+            *reinterpret_cast<u32x4*>(dst + lo) = o1;
+            *reinterpret_cast<u32x4*>(dst + hi) = o2;
+        }
+        *reinterpret_cast<u32x4*>(k_tile + Tile::k_offset(r, c)) = o1;
+        *reinterpret_cast<u32x4*>(k_tile + Tile::k_offset(r, c + cph)) = o2;
+    }
+    for (int c = tid; c < Tile::kTokens * Tile::CPR; c += kThreads) {
+        const int r = c / Tile::CPR, cc = c % Tile::CPR;
+        const int64_t t = t0 + r;
+        u32x4 vv = {0, 0, 0, 0};
+        if (t < a.n_tokens) vv = *reinterpret_cast<const u32x4*>(a.v + t * a.v_st + h * HD + cc * 8);
+        Tile::put_v(v_tile, r, cc, vv);
+    }
+    __syncthreads();
+    Tile::store(k_tile, v_tile, slot_of, static_cast<uint16_t*>(a.k_cache), static_cast<uint16_t*>(a.v_cache), a.kd, a.vd, h,
+                a.page_size, tid, kThreads);
+}
+
+template <typename PosT>
+int launch_rope_distinct(const RopeArgs& a, const void* positions, const void* slots, int slot_type, hipStream_t st) {
+    const int64_t q_work = a.n_tokens * a.h_q * (a.hd >> 4);
+    const int64_t q_blocks = (q_work + kThreads - 1) / kThreads;
+    const int64_t tiles = (a.n_tokens + DistinctTile<128>::kTokens - 1) / DistinctTile<128>::kTokens * a.h_kv;
+    if (q_blocks + tiles > INT32_MAX) return DFX_ERR_UNSUPPORTED;
+    const dim3 grid(static_cast<unsigned>(q_blocks + tiles)), block(kThreads);
+    const PosT* pos = static_cast<const PosT*>(positions);
+#define DFX_ROPE_DISTINCT(SLOT_T, HD_)                                                                                   \
+    hipLaunchKernelGGL((rope_store_distinct_kernel<PosT, SLOT_T, HD_>), grid, block, 0, st, a, pos,                      \
+                       static_cast<const SLOT_T*>(slots), static_cast<int>(q_blocks))
+    if (a.hd == 128) {
+        if (slot_type == DFX_INDEX_I64) DFX_ROPE_DISTINCT(int64_t, 128);
+        else DFX_ROPE_DISTINCT(int32_t, 128);
+    } else {
+        if (slot_type == DFX_INDEX_I64) DFX_ROPE_DISTINCT(int64_t, 64);
+        else DFX_ROPE_DISTINCT(int32_t, 64);
+    }
+#undef DFX_ROPE_DISTINCT
+    return launch_status();
 }
 
 template <bool FP8, typename PosT>
@@ -207,6 +302,18 @@ extern "C" int dfx_rope_kv_store(const dfx_rope_params* p, dfx_stream_t stream) 
         if (!aligned16(p->k_cache) || !aligned16(p->v_cache)) return DFX_ERR_INVALID_ARG;
         if (p->slot_index_type != DFX_INDEX_I32 && p->slot_index_type != DFX_INDEX_I64) return DFX_ERR_INVALID_ARG;
         if (fp8 != (p->k_scale != nullptr) || fp8 != (p->v_scale != nullptr)) return DFX_ERR_INVALID_ARG;
+        if (p->cache_layout != DFX_CACHE_UNIFIED && p->cache_layout != DFX_CACHE_DISTINCT) return DFX_ERR_INVALID_ARG;
+        if (p->cache_layout == DFX_CACHE_DISTINCT) {
+            if (fp8 || (p->head_dim != 64 && p->head_dim != 128)) return DFX_ERR_UNSUPPORTED;
+            if (p->page_size <= 0 || p->n_slots % p->page_size != 0) return DFX_ERR_INVALID_ARG;
+            for (int i = 0; i < 3; ++i) {
+                if (p->kc_stride[i] < 0 || p->kc_stride[i] % 8 || p->vc_stride[i] < 0) return DFX_ERR_INVALID_ARG;
+                a.kd[i] = p->kc_stride[i];
+                a.vd[i] = p->vc_stride[i];
+            }
+            a.distinct = 1;
+            a.page_size = p->page_size;
+        }
         a.v_heads = a.h_kv;
         a.k_cache = p->k_cache;
         a.v_cache = p->v_cache;
@@ -217,6 +324,10 @@ extern "C" int dfx_rope_kv_store(const dfx_rope_params* p, dfx_stream_t stream) 
         return DFX_ERR_INVALID_ARG;
     }
     hipStream_t st = static_cast<hipStream_t>(stream);
+    if (a.distinct)
+        return p->position_index_type == DFX_INDEX_I64
+                   ? launch_rope_distinct<int64_t>(a, p->positions, p->slot_mapping, p->slot_index_type, st)
+                   : launch_rope_distinct<int32_t>(a, p->positions, p->slot_mapping, p->slot_index_type, st);
     const bool q8 = store && fp8;
     if (p->position_index_type == DFX_INDEX_I64)
         return q8 ? launch_rope<true, int64_t>(a, p->positions, p->slot_mapping, p->slot_index_type, st)

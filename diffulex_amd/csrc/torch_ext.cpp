@@ -369,9 +369,25 @@ void rope_kv_store(const Tensor& positions, const Tensor& query, const Tensor& k
         const int64_t tv = rows_of(*value, head_size, hv, "value");
         const int64_t row = hk * head_size;
         TORCH_CHECK(tv == tk && hv == hk, "value does not fit key");
-        TORCH_CHECK(k_cache->is_contiguous() && v_cache->is_contiguous() && k_cache->dim() == 4 &&
-                        k_cache->stride(1) == row && v_cache->stride(1) == row,
-                    "caches: contiguous [pages, page, H_kv, hd]");
+        const bool distinct = k_cache->dim() == 5;   // K [pages, H_kv, hd / 8, page, 8], V [pages, H_kv, hd, page]
+        if (distinct) {
+            TORCH_CHECK(v_cache->dim() == 4 && k_cache->size(1) == hk && v_cache->size(1) == hk && k_cache->size(4) == 8 &&
+                            k_cache->size(2) * 8 == head_size && v_cache->size(2) == head_size &&
+                            k_cache->size(3) == v_cache->size(3) && k_cache->size(0) == v_cache->size(0) &&
+                            k_cache->stride(4) == 1 && k_cache->stride(3) == 8 && v_cache->stride(3) == 1 &&
+                            k_cache->scalar_type() == at::kBFloat16 && v_cache->scalar_type() == at::kBFloat16,
+                        "distinct layout: bf16 K [pages, H_kv, hd / 8, page, 8] and V [pages, H_kv, hd, page], tokens dense");
+            p.cache_layout = DFX_CACHE_DISTINCT;
+            p.page_size = static_cast<int32_t>(k_cache->size(3));
+            for (int i = 0; i < 3; ++i) {
+                p.kc_stride[i] = k_cache->stride(i);
+                p.vc_stride[i] = v_cache->stride(i);
+            }
+        } else {
+            TORCH_CHECK(k_cache->is_contiguous() && v_cache->is_contiguous() && k_cache->dim() == 4 &&
+                            k_cache->stride(1) == row && v_cache->stride(1) == row,
+                        "caches: contiguous [pages, page, H_kv, hd]");
+        }
         TORCH_CHECK(slot_mapping->is_contiguous() && slot_mapping->numel() == tk, "`N`: ", tk,
                     ", `slot_mapping.numel()`: ", slot_mapping->numel());
         p.v = value->data_ptr();
@@ -380,8 +396,8 @@ void rope_kv_store(const Tensor& positions, const Tensor& query, const Tensor& k
         p.v_cache = v_cache->data_ptr();
         p.slot_mapping = slot_mapping->data_ptr();
         p.slot_index_type = index_type(*slot_mapping, "slot_mapping");
-        p.n_slots = k_cache->size(0) * k_cache->size(1);
-        if (is_fp8_cache(*k_cache)) {
+        p.n_slots = distinct ? k_cache->size(0) * k_cache->size(3) : k_cache->size(0) * k_cache->size(1);
+        if (!distinct && is_fp8_cache(*k_cache)) {
             p.kv_dtype = DFX_KV_FP8_E4M3;
             p.k_scale = scale_ptr(k_scale, static_cast<int>(hk), "k_scale");
             p.v_scale = scale_ptr(v_scale, static_cast<int>(hk), "v_scale");

@@ -72,7 +72,9 @@ class RotaryEmbedding(nn.Module):
                           slot_mapping: torch.Tensor, attn_metadata=None,
                           k_scale: Optional[torch.Tensor] = None, v_scale: Optional[torch.Tensor] = None
                           ) -> Tuple[torch.Tensor, torch.Tensor]:
-        """forward() and store_kvcache_unified_layout(rotated key, value, ...) in one launch."""
+        """forward() and store_kvcache_unified_layout(rotated key, value, ...) in one launch -- or
+        store_kvcache_distinct_layout(...) where the caches are in that layout (k_cache [pages, H_kv, hd / 8,
+        page, 8], v_cache [pages, H_kv, hd, page], bf16)."""
         q_out = torch.empty(query.shape, dtype=query.dtype, device=query.device)
         k_out = torch.empty(key.shape, dtype=key.dtype, device=key.device)
         self._launch(positions, query, key, q_out, k_out, value, k_cache, v_cache, slot_mapping,

@@ -19,7 +19,7 @@
 extern "C" {
 #endif
 
-#define DFX_ABI_VERSION 7
+#define DFX_ABI_VERSION 8
 
 typedef void* dfx_stream_t; /* a hipStream_t; NULL is the default stream */
 
@@ -454,6 +454,15 @@ typedef struct dfx_rope_params {
     int64_t n_slots;
     const float* k_scale;        /* fp32[num_kv_heads], FP8 caches only */
     const float* v_scale;
+    /* Layout of the caches the store writes.  DFX_CACHE_UNIFIED (0): as above.  DFX_CACHE_DISTINCT: what
+     * dfx_kv_store_distinct writes with x == 8 -- K [pages, num_kv_heads, head_dim / 8, page_size, 8] and
+     * V [pages, num_kv_heads, head_dim, page_size], bf16 -- through the element strides of their first three
+     * dimensions (multiples of 8; tokens of a page 8 elements apart in K, dense in V); slot s is token
+     * s % page_size of page s / page_size, n_slots = pages * page_size. */
+    int32_t cache_layout;
+    int32_t page_size;
+    int64_t kc_stride[3];
+    int64_t vc_stride[3];
 } dfx_rope_params;
 
 int dfx_rope_kv_store(const dfx_rope_params* params, dfx_stream_t stream);

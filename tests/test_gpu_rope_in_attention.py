@@ -116,6 +116,48 @@ def test_shapes_without_a_pipelined_kernel_refuse_the_rope_and_the_module_falls_
     att2 = dfx.Attention(hq, hd, wl.scale, hkv)
     att2.k_cache, att2.v_cache = wl.k_cache.clone(), wl.v_cache.clone()
     assert torch.equal(_bits(out), _bits(att2(rq, rk, wl.v_new.reshape(T, -1))))
+    # (the fallback rotates and stores in one launch: the same cache as the store of the rotated rows)
+    assert torch.equal(_bits(att.k_cache), _bits(att2.k_cache)) and torch.equal(_bits(att.v_cache), _bits(att2.v_cache))
+
+
+def test_attention_module_with_rope_on_the_distinct_layout(dev):
+    """kv_cache_layout == "distinct": the rotary embedding's launch also stores the block into that layout
+    (dfx_rope_kv_store), the attention launch then streams from it -- two launches, the same bits as rotating,
+    storing with store_kvcache_distinct_layout and attending in three."""
+    wl = make_workload("c3", num_seqs=5, ctx=(200, 800), seed=12).to(dev)
+    T, hq, hkv, hd = wl.q.shape[0], wl.num_q_heads, wl.num_kv_heads, wl.head_dim
+    g = torch.Generator("cpu").manual_seed(13)
+    qkv = torch.randn(T, (hq + 2 * hkv) * hd, generator=g).to(torch.bfloat16).to(dev)
+    q, k, v = qkv.split([hq * hd, hkv * hd, hkv * hd], dim=-1)
+    pos = torch.randint(0, MAXPOS, (T,), generator=g).to(dev)
+    rope = RotaryEmbedding(hd, hd, MAXPOS, BASE).to(dev)
+    pages, page = wl.k_cache.shape[0], wl.k_cache.shape[1]
+
+    def distinct(c):
+        return (c.view(pages, page, hkv, hd // 8, 8).permute(0, 2, 3, 1, 4).contiguous(), c.permute(0, 2, 3, 1).contiguous())
+    outs, caches = [], []
+    for one_call in (True, False):
+        att = dfx.Attention(hq, hd, wl.scale, hkv)
+        att.k_cache, att.v_cache = distinct(wl.k_cache)[0], distinct(wl.v_cache)[1]
+        md = metadata_for(wl, "static")
+        md.kv_cache_layout = "distinct"
+        md.need_kv_cache_store = True
+        dfx.set_fetch_fn_for_attn_metadata(lambda: md)
+        if one_call:
+            outs.append(att(q, k, v, rope=(rope, pos)))
+        else:
+            rq, rk = rope(pos, q, k)
+            outs.append(att(rq, rk, v))
+        caches.append((att.k_cache, att.v_cache))
+    torch.cuda.synchronize()
+    assert torch.equal(_bits(outs[0]), _bits(outs[1]))
+    assert torch.equal(_bits(caches[0][0]), _bits(caches[1][0])) and torch.equal(_bits(caches[0][1]), _bits(caches[1][1]))
+    tab = orot.cos_sin_cache(hd, MAXPOS, BASE)
+    c = wl.to("cpu")
+    c.q = orot.apply_rotary(q.contiguous().cpu(), pos.cpu(), tab, hd).view(T, hq, hd)
+    c.k_new = orot.apply_rotary(k.contiguous().cpu(), pos.cpu(), tab, hd).view(T, hkv, hd)
+    c.v_new = v.cpu().contiguous().view(T, hkv, hd)
+    assert max_abs_err(outs[0].view(T, hq, hd), oracle_fp32(c)) <= ATOL_BF16
 
 
 def test_rope_inside_the_launch_in_a_captured_graph(dev):

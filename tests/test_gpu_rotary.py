@@ -191,3 +191,37 @@ def test_layer_step_rope_store_attention_eager_and_in_a_graph(dev):
         eager = layer()
         torch.cuda.synchronize()
         assert torch.equal(got, eager), f"replay {rep}"
+
+
+@pytest.mark.parametrize("hd,h_q,h_kv,page", [(128, 28, 4, 256), (64, 8, 2, 32), (128, 4, 4, 16)])
+def test_rope_and_store_into_the_distinct_layout_bit_exact(dev, hd, h_q, h_kv, page):
+    """dfx_rope_kv_store writing the distinct cache layout (K [pages, H, hd / 8, page, 8], V [pages, H, hd, page]):
+    the rotated K and V land where the CPU restatement of the reference's distinct store puts them, bit for bit;
+    negative and out-of-range slots are skipped; the rest of the caches is untouched."""
+    from oracle import kv_cache as okv
+    g = torch.Generator("cpu").manual_seed(17)
+    pages = 7
+    T = min(300, pages * page - 8)
+    qkv = torch.randn(T, (h_q + 2 * h_kv) * hd, generator=g).to(torch.bfloat16)
+    q, k, v = qkv.split([h_q * hd, h_kv * hd, h_kv * hd], dim=-1)
+    pos = torch.randint(0, 4096, (T,), generator=g)
+    slots = torch.randperm(pages * page, generator=g)[:T].to(torch.int32)
+    slots[5] = -1
+    slots[9] = pages * page + 3
+    kd0 = torch.randn(pages, h_kv, hd // 8, page, 8, generator=g).to(torch.bfloat16)
+    vd0 = torch.randn(pages, h_kv, hd, page, generator=g).to(torch.bfloat16)
+    tab = orot.cos_sin_cache(hd, 4096, 1.0e6)
+    rk = orot.apply_rotary(k.contiguous(), pos, tab, hd)
+    want_k, want_v = kd0.clone(), vd0.clone()
+    ok = (slots >= 0) & (slots < pages * page)
+    okv.store_distinct(rk.view(T, h_kv, hd)[ok], v.reshape(T, h_kv, hd)[ok], want_k, want_v, slots[ok])
+    rope = RotaryEmbedding(hd, hd, 4096, 1.0e6).to(dev)
+    kd, vd = kd0.to(dev), vd0.to(dev)
+    d = qkv.to(dev)
+    dq, dk, dv = d.split([h_q * hd, h_kv * hd, h_kv * hd], dim=-1)
+    rq_got, rk_got = rope.forward_and_store(pos.to(dev), dq, dk, dv, kd, vd, slots.to(dev))
+    torch.cuda.synchronize()
+    assert torch.equal(rk_got.cpu().view(torch.int16), rk.view(torch.int16))
+    assert torch.equal(rq_got.cpu().view(torch.int16), orot.apply_rotary(q.contiguous(), pos, tab, hd).view(torch.int16))
+    assert torch.equal(kd.cpu().view(torch.int16), want_k.view(torch.int16))
+    assert torch.equal(vd.cpu().view(torch.int16), want_v.view(torch.int16))

@@ -196,13 +196,19 @@ def bench_rope(args, dev):
     pos = torch.randint(0, max_pos, (T,), generator=g).to(dev)
     pages, page = 64, 256
     slots = torch.randperm(pages * page, generator=g)[:T].to(torch.int32).to(dev)
+    distinct = args.layout == "distinct"
+    if distinct:
+        # a block of 32 tokens per sequence in consecutive slots of the sequence's page, as a decode step stores it
+        start = torch.randint(0, (page - 32) // 8 + 1, (pages,), generator=g) * 8 + torch.arange(pages) * page
+        slots = (start.repeat_interleave(32) + torch.arange(32).repeat(pages)).to(torch.int32).to(dev)
     sets = []
     for _ in range(n_sets):
         qkv = torch.randn(T, (hq + 2 * hkv) * hd, generator=g).to(torch.bfloat16).to(dev)
+        kc_shape, vc_shape = ((pages, hkv, hd // 8, page, 8), (pages, hkv, hd, page)) if distinct else ((pages, page, hkv, hd),) * 2
         sets.append((qkv, torch.empty(T, hq * hd, dtype=torch.bfloat16, device=dev),
                      torch.empty(T, hkv * hd, dtype=torch.bfloat16, device=dev),
-                     torch.zeros(pages, page, hkv, hd, dtype=torch.bfloat16, device=dev),
-                     torch.zeros(pages, page, hkv, hd, dtype=torch.bfloat16, device=dev)))
+                     torch.zeros(kc_shape, dtype=torch.bfloat16, device=dev),
+                     torch.zeros(vc_shape, dtype=torch.bfloat16, device=dev)))
     st = torch.cuda.current_stream().cuda_stream
     params = []
     for qkv, qo, ko, kc, vc in sets:
@@ -216,6 +222,10 @@ def bench_rope(args, dev):
         p.n_tokens, p.num_q_heads, p.num_kv_heads, p.head_dim = T, hq, hkv, hd
         p.kv_dtype, p.k_cache, p.v_cache = _lib.DFX_KV_BF16, kc.data_ptr(), vc.data_ptr()
         p.slot_mapping, p.slot_index_type, p.n_slots = slots.data_ptr(), _lib.DFX_INDEX_I32, pages * page
+        if distinct:
+            p.cache_layout, p.page_size = _lib.DFX_CACHE_DISTINCT, page
+            for i in range(3):
+                p.kc_stride[i], p.vc_stride[i] = kc.stride(i), vc.stride(i)
         params.append(p)
 
     def step(i):
@@ -241,10 +251,12 @@ def bench_rope(args, dev):
         "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
         "data": "synthetic",
         "config": {"workload": f"rope: {T} tokens, H_q={hq}, H_kv={hkv}, head_dim={hd}, rotated and stored into a "
-                               f"{pages}x{page}-slot bf16 cache in one launch", "spin_up_launches": n_spin},
+                               f"{pages}x{page}-slot bf16 cache in one launch"
+                               + (", distinct cache layout, 32 consecutive slots per sequence" if distinct else ""),
+                   "spin_up_launches": n_spin},
         "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS,
                      "traffic": None, "algorithmic_bytes": nbytes,
-                     "kernel": "rope_kv_store_kernel, duration = timed region / steps"},
+                     "kernel": ("rope_store_distinct_kernel" if distinct else "rope_kv_store_kernel") + ", duration = timed region / steps"},
     }))
 
 

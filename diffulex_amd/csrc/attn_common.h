@@ -159,7 +159,7 @@ struct TileInfo {
 template <int HD, int NB, int NW = kWaves, bool HIDDEN = false>
 struct AttnState {
     using S = Shape<HD, NB, NW>;
-    static_assert(!HIDDEN || (HD == 128 && NB == 1), "register map of attn_pipe_gen.h");
+    static_assert(!HIDDEN || ((HD == 128 || HD == 64) && NB == 1), "register map of attn_pipe_gen.h");
 
     const KArgs& a;
     const int tid, lane, wave, col, half;
@@ -222,7 +222,8 @@ struct AttnState {
                     for (int e = 0; e < 16; ++e) o[db][qb][e] = 0.0f;
             }
         }
-        if constexpr (HIDDEN) pipe_zero_outputs();
+        if constexpr (HIDDEN && HD == 128) pipe_zero_outputs();
+        if constexpr (HIDDEN && HD == 64) pipe64_zero_outputs();
     }
 
     // Q rows of row tile rt into B-operand registers (zeros for rows past G * q_len).
@@ -510,7 +511,8 @@ struct AttnState {
         int w = wave;
         asm volatile("" : "+v"(w));
         const uint8_t* p = reinterpret_cast<const uint8_t*>(slot_ptr(slot) + w * S::BLOCK_FLOATS) + lane_here() * 16;
-        pipe_request_partial(p, p + 3 * 1024, p + 6 * 1024);
+        if constexpr (HD == 128) pipe_request_partial(p, p + 3 * 1024, p + 6 * 1024);
+        else pipe64_request_partial(p, p + 4 * 1024);
     }
 
     // Merge one stored piece into the running state (l_run holds whole-row sums here): the piece in `slot`, or

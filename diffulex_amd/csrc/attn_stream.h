@@ -368,8 +368,9 @@ struct StreamAttn : TileMath<HD, NB, NW, HIDDEN> {
         if constexpr (HIDDEN && NW == 8 && KVB == 2) {
             // the common case, a full band of cached rows: offsets precomputed per lane, no vector arithmetic
             if (is_ctx && last >= C::ROWS_PER_WAVE - 1) {
-                pipe_issue_band(a.k_cache + off, a.v_cache + off,
-                                uniform(static_cast<int>(stages_lds + (static_cast<unsigned>(rel) % C::kStages) * C::STAGE_BYTES + wave * (C::IPW * 1024))));
+                const int dst = uniform(static_cast<int>(stages_lds + (static_cast<unsigned>(rel) % C::kStages) * C::STAGE_BYTES + wave * (C::IPW * 1024)));
+                if constexpr (HD == 128) pipe_issue_band(a.k_cache + off, a.v_cache + off, dst);
+                else pipe64_issue_band(a.k_cache + off, a.v_cache + off, dst);
                 return;
             }
         }
@@ -544,7 +545,9 @@ struct StreamAttn : TileMath<HD, NB, NW, HIDDEN> {
         // beyond the rows q has -- offsets rewritten in place after the plan was made -- reads row 0 of q)
         int row = uniform(d.q0) + i;
         row = row < a.n_q ? row : 0;
-        pipe_issue_queries(a.q + row * a.q_st + (uniform(d.kvh) * a.group + g) * a.q_sh + half * 8);
+        const uint16_t* qp = a.q + row * a.q_st + (uniform(d.kvh) * a.group + g) * a.q_sh + half * 8;
+        if constexpr (HD == 128) pipe_issue_queries(qp);
+        else pipe64_issue_queries(qp);
     }
     DFX_D void adopt_item(const UnitDesc& d) {
         this->s = uniform(d.s);
@@ -956,7 +959,8 @@ struct StreamAttn : TileMath<HD, NB, NW, HIDDEN> {
     bool queries_requested = false;     // ... which the planned start has requested (the first chunk's body resets it)
     template <typename Body>
     DFX_D void for_each_chunk_prefetched(Body&& body) {
-        static_assert(HIDDEN && KVB == 2 && C::LOADS_PER_UNIT == 4 && C::kPlanUnits * NW <= 2 * C::THREADS, "table shares and wait counts below");
+        static_assert(HIDDEN && KVB == 2 && C::kPlanUnits * NW <= 2 * C::THREADS, "table shares below");
+        constexpr int QL = C::S::NSLAB, UL = C::LOADS_PER_UNIT;  // loads of a lane's query row, of a wave's share of a unit
         bool planned = false;
         int64_t n_total = 0, n_first = 0, ubase = 0;
         int n_active = 0, plan_mode = 0, prefilled = 0;
@@ -1037,9 +1041,9 @@ struct StreamAttn : TileMath<HD, NB, NW, HIDDEN> {
                 }
                 // the tables are this wave's oldest loads: 8 of query rows and 4 per unit are younger
                 static_assert(kPrefill == 2, "wait counts");
-                if (prefilled == 2) wait_async_loads<8 + 8>();
-                else if (prefilled == 1) wait_async_loads<8 + 4>();
-                else wait_async_loads<8>();
+                if (prefilled == 2) wait_async_loads<QL + 2 * UL>();
+                else if (prefilled == 1) wait_async_loads<QL + UL>();
+                else wait_async_loads<QL>();
             }
         }
         if (!planned) {
@@ -1224,14 +1228,20 @@ __global__ void __launch_bounds__(64 * NW, 1) paged_attn_stream_fp8_kernel(const
 // PREFILL: the variant for launches without a cache.  Every tile
 // is one of fresh rows there, and its plain steps fetch full bands of those the way the other variant's
 // fetch bands of cached rows (which keeps its fresh tiles, one or two per item, on the general step).
-// The blocks of attn_pipe_gen.h for the tile layout of the kernel's cache.
-template <bool DISTINCT>
+// The blocks of attn_pipe_gen.h for the tile layout of the kernel's cache and its head_dim.
+template <bool DISTINCT, int HD = 128>
 struct PipeBlocks {
+    static_assert(HD == 128 || (HD == 64 && !DISTINCT), "families of blocks generated");
 #define DFX_PIPE_BLOCK(name, params, args)                     \
     DFX_D static void name params {                            \
         if constexpr (DISTINCT) pipe_d_##name args;            \
+        else if constexpr (HD == 64) pipe64_##name args;       \
         else pipe_##name args;                                 \
     }
+#define pipe64_mask_a_8 pipe_mask_a_8
+#define pipe64_mask_a_16 pipe_mask_a_16
+#define pipe64_mask_b_8 pipe_mask_b_8
+#define pipe64_mask_b_16 pipe_mask_b_16
     DFX_PIPE_BLOCK(first_scores, (uint32_t k, float& mx), (k, mx))
     DFX_PIPE_BLOCK(mask_a_8, (int thr, uint32_t holes, float& mx), (thr, holes, mx))
     DFX_PIPE_BLOCK(mask_a_16, (int thr, uint32_t holes, float& mx), (thr, holes, mx))
@@ -1245,21 +1255,31 @@ struct PipeBlocks {
     DFX_PIPE_BLOCK(last_a_y, (float c, float nm, float& l), (c, nm, l))
     DFX_PIPE_BLOCK(last_b_x, (uint32_t v, float c, float nm, float& l), (v, c, nm, l))
     DFX_PIPE_BLOCK(last_b_y, (float c, float nm, float& l), (c, nm, l))
+    DFX_D static void rescale_outputs(float alpha) {
+        if constexpr (HD == 64) pipe64_rescale_outputs(alpha);
+        else pipe_rescale_outputs(alpha);
+    }
+#undef pipe64_mask_a_8
+#undef pipe64_mask_a_16
+#undef pipe64_mask_b_8
+#undef pipe64_mask_b_16
 #undef DFX_PIPE_BLOCK
 };
 
 // DISTINCT: the cache is in the distinct layout (StreamAttn): the blocks read a chunk-major K tile and a d-major V
 // tile, a full tile of cached rows is fetched by pipe_d_issue_band, and the general step first does to its own
 // tile's V^T rows what the loads could not (transpose_fresh_v, clear_v_tail); no store, no rotary embedding.
-template <int NW, bool PREFILL = false, bool DISTINCT = false>
+// HD: 128, or 64 (unified layout, launches with a cache or without: the blocks pipe64_*; a wave fetches its 8 rows of
+// a tile with one load per matrix; no rotary embedding inside the launch).
+template <int NW, bool PREFILL = false, bool DISTINCT = false, int HD = 128>
 __global__ void __launch_bounds__(64 * NW, 1) __attribute__((amdgpu_num_vgpr(32)))
 paged_attn_pipe_kernel(const KArgs a) {
     static_assert(!(PREFILL && DISTINCT), "a launch without a cache has no cache layout");
+    static_assert(HD == 128 || !(PREFILL || DISTINCT), "head_dim 64: one kernel");
     extern __shared__ __attribute__((aligned(256))) uint8_t smem[];
-    constexpr int HD = 128;
     using C = StreamCfg<HD, 1, NW, false>;
     using SA = StreamAttn<HD, 1, NW, false, 2, true, DISTINCT>;
-    using PB = PipeBlocks<DISTINCT>;
+    using PB = PipeBlocks<DISTINCT, HD>;
     SA at(a, smem);
     pipe_reserve();
     if constexpr (DISTINCT) {
@@ -1271,6 +1291,10 @@ paged_attn_pipe_kernel(const KArgs a) {
             v[j] = static_cast<uint32_t>(d) * static_cast<uint32_t>(a.vd_sd * 2) + ((at.lane & 7) ^ ((d >> 1) & 7)) * 16;
         }
         pipe_d_set_load_offsets(at.lane * 16, v[0], v[1]);
+    } else if constexpr (HD == 64) {
+        const int r = at.lane / C::CPR;  // one load covers the wave's 8 rows
+        const int chunk = (at.lane % C::CPR) ^ C::swizzle(at.wave * C::ROWS_PER_WAVE + r);
+        pipe64_set_load_offsets(static_cast<uint32_t>(r) * static_cast<uint32_t>(a.c_st * 2) + chunk * 16);
     } else {
         uint32_t o[2];
 #pragma unroll
@@ -1298,7 +1322,7 @@ paged_attn_pipe_kernel(const KArgs a) {
             pipe_set_load_offsets(o[0], o[1]);
         }
     }
-    const bool rope = !PREFILL && !DISTINCT && a.rope_table != nullptr;  // (with it the store travels with the rotation of the fresh K rows)
+    const bool rope = !PREFILL && !DISTINCT && HD == 128 && a.rope_table != nullptr;  // (with it the store travels with the rotation of the fresh K rows)
     if constexpr (!DISTINCT) {
         if (!rope) store_fresh_rows<HD, false, 1>(a);
     }
@@ -1319,7 +1343,7 @@ paged_attn_pipe_kernel(const KArgs a) {
         // angles of the first item's query rows, requested behind the stores of those rows so that the two
         // trips to memory run together.
         bool rotate_first = false;
-        if constexpr (!PREFILL && !DISTINCT) {
+        if constexpr (!PREFILL && !DISTINCT && HD == 128) {
             if (rope) {
                 int64_t pos = 0;
                 if (opens) pos = at.rope_query_position(at.units[0]);
@@ -1343,7 +1367,9 @@ paged_attn_pipe_kernel(const KArgs a) {
             if (prefilled == 0) wait_async_loads<0>();
             else if (prefilled == 1) wait_async_loads<C::LOADS_PER_UNIT>();
             else wait_async_loads<2 * C::LOADS_PER_UNIT>();
-            if (rotate_first) pipe_rope_queries();
+            if constexpr (HD == 128) {
+                if (rotate_first) pipe_rope_queries();
+            }
             at.adopt_item(at.units[0]);
         }
         int issued = prefilled;  // ring fill: kStages - 1 units in flight
@@ -1421,7 +1447,7 @@ paged_attn_pipe_kernel(const KArgs a) {
                     if (__any(m_run != -INFINITY)) {
                         const float alpha = (m_new == -INFINITY) ? 1.0f : fast_exp2(m_run - m_new);
                         at.l_run[0] *= alpha;
-                        pipe_rescale_outputs(alpha);
+                        PB::rescale_outputs(alpha);
                     }
                     m_run = m_new;
                 }
@@ -1500,6 +1526,8 @@ paged_attn_pipe_kernel(const KArgs a) {
                         const int64_t page = (off >> 20) & 0xffffffffll, in_page = off & 0xfffff;
                         const uint8_t* kb = a.k_cache + (page * a.kd_sp + kvh * a.kd_sh + in_page * 8 + at.wave_s * 2 * a.kd_sc) * 2;
                         pipe_d_issue_band(kb, kb + a.kd_sc * 2, a.v_cache + (page * a.vd_sp + kvh * a.vd_sh + in_page) * 2, dst);
+                    } else if constexpr (HD == 64) {
+                        pipe64_issue_band(a.k_cache + off, a.v_cache + off, dst);
                     } else {
                         pipe_issue_band(a.k_cache + off, a.v_cache + off, dst);
                     }
@@ -1557,7 +1585,7 @@ paged_attn_pipe_kernel(const KArgs a) {
             if (next_opens) wait_async_loads<0>();  // the next item's query rows (and the tiles requested before them)
             at.finish_run(rel - 1, split);
             if (next_opens) {
-                if constexpr (!PREFILL) {
+                if constexpr (!PREFILL && HD == 128) {
                     if (rope) at.rope_queries(at.units[run_end]);
                 }
                 at.adopt_item(at.units[run_end]);

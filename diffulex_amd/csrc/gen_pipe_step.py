@@ -52,6 +52,16 @@ HD = 128
 ROWB = HD * 2
 NSLAB = HD // 16            # 8
 NDB = HD // 32              # 4
+
+
+def set_head_dim(hd):
+    """The blocks generated from here on are for this head_dim (128, or 64: half the contraction slabs of S^T, half
+    the d blocks of O^T -- a[32:63] -- and of the Q operand -- a[96:111]; a tile row is 128 bytes, a K or V tile 8 KiB)."""
+    global HD, ROWB, NSLAB, NDB, MAT_BYTES
+    HD, ROWB, NSLAB, NDB = hd, hd * 2, hd // 16, hd // 32
+    MAT_BYTES = 64 * ROWB
+
+
 COMPILER_REGS = 32          # v0..v31 and a0..a31 are the compiler's (amdgpu_num_vgpr(32))
 O_BASE, Q_BASE = 32, 96
 TMP, NTMP = 32, 11
@@ -82,6 +92,8 @@ def ar(base, n=1):
 
 
 def swizzle(row):
+    if HD == 64:  # (TileLayout<64>::swizzle: 128-byte rows, odd rows already sit 64 banks further)
+        return (((row >> 1) & 1) << 2) | ((row >> 2) & 3)
     return ((row & 3) << 2) | ((row >> 2) & 3)
 
 
@@ -263,16 +275,23 @@ def step_blocks(cur, nxt, has_next):
     bx.other("s_waitcnt lgkmcnt(0)")
     by = Block()
     by.other("s_waitcnt lgkmcnt(0)")
+    half, quarter = 2 * NDB, NDB  # of the 4 * NDB matrix instructions of phase Y (head_dim 128: 8 and 4)
     if has_next:
         phase_x(bx, nxt, sx, spread(len(sx), 2 * NSLAB))
         y2 = y2a + max_instrs(nxt)
-        qa = spread(len(y2a) + 4, 4)
+        qa = spread(len(y2a) + 4, quarter)
         sy = y1 + y2
-        phase_y(by, cur, sy, spread(len(y1), 8) + qa + spread(len(y2) - sum(qa), 4))
+        quotas = spread(len(y1), half) + qa + spread(len(y2) - sum(qa), quarter)
     else:
         emit_valu(bx, sx, len(sx))
         sy = y1 + y2a
-        phase_y(by, cur, sy, spread(len(y1), 8) + spread(len(y2a), 4) + [0, 0, 0, 0])
+        quotas = spread(len(y1), half) + spread(len(y2a), quarter) + [0] * quarter
+    # every pair is complete before the matrix instruction that reads it: instruction j (token block tb, slab sl)
+    # reads pairs 8 tb + 4 sl .. + 3; pairs 0..8 are done in phase X, pair p > 8 with instruction 7 (p - 8) of phase Y
+    for j in range(4 * NDB):
+        last_pair = 8 * (j // (2 * NDB)) + 4 * ((j // NDB) & 1) + 3
+        assert sum(quotas[:j]) >= 7 * max(0, last_pair - 8), (HD, j)
+    phase_y(by, cur, sy, quotas)
     assert not sx and not sy and not bx.lds_queue and not by.lds_queue
     return bx.text(), by.text()
 
@@ -405,6 +424,50 @@ def step_fns(name, cur, nxt, has_next, comment=None):
     fy = asm_fn(name + "_y", "float c, float neg_m, float& l_run" + (", float& mx" if has_next else ""), y,
                 ['[l] "+v"(l_run)'] + (['[mx] "=&v"(mx)'] if has_next else []), ['[c] "s"(c)', '[nm] "v"(neg_m)'], ["memory"])
     return fx + fy
+
+
+def head_dim_64_family():
+    """The blocks whose code depends on head_dim, once more for head_dim 64 (pipe64_*): same register map with
+    half the O^T accumulators (a[32:63]) and half the Q operand (a[96:111]); a wave fetches its 8 rows of a tile with
+    one load per matrix.  Masks, the accessors of the accumulators and of a requested piece are shared."""
+    global LAYOUT
+    LAYOUT = "u"
+    set_head_dim(64)
+    pre, what = "pipe64_", "  head_dim 64."
+    parts = []
+    parts.append(asm_fn(pre + "zero_outputs", "", join(f"v_accvgpr_write_b32 {ar(O_BASE + i)}, 0" for i in range(16 * NDB)),
+                        comment="O^T = 0." + what))
+    resc = list(MFMA_TO_VALU)
+    for g in range(0, 16 * NDB, 4):
+        resc += [f"v_accvgpr_read_b32 {vr(TMP + i - g)}, {ar(O_BASE + i)}" for i in range(g, g + 4)]
+        resc += [f"v_mul_f32 {vr(TMP + i - g)}, {vr(TMP + i - g)}, %[alpha]" for i in range(g, g + 4)]
+        resc += [f"v_accvgpr_write_b32 {ar(O_BASE + i)}, {vr(TMP + i - g)}" for i in range(g, g + 4)]
+    parts.append(asm_fn(pre + "rescale_outputs", "float alpha", join(resc), ins=['[alpha] "v"(alpha)'],
+                        comment="O^T *= alpha, behind the wait states for the matrix results." + what))
+    ql = [f"global_load_dwordx4 {ar(Q_BASE + 4 * s, 4)}, %[p], off offset:{s * 32}" for s in range(NSLAB)]
+    parts.append(asm_fn(pre + "issue_queries", "const void* row", join(ql), ins=['[p] "v"(row)'], clobbers=["memory"],
+                        comment="Q operand: requests the lane's half (slab s at byte 32 s) of the 128-byte query row at `row`." + what))
+    parts.append(asm_fn(pre + "set_load_offsets", "uint32_t o0", f"v_mov_b32 {vr(LOAD_OFF)}, %0", ins=['"v"(o0)'],
+                        comment="Once per kernel: the lane's byte offset (row * row stride + swizzled chunk * 16) for the one\n"
+                                "wave-wide load that fetches its wave's 8 rows (128 bytes each) of a tile of cached rows." + what))
+    issue = [f"s_add_u32 m0, %[d], 0", f"global_load_lds_dwordx4 {vr(LOAD_OFF)}, %[kb] nt",
+             f"s_add_u32 m0, %[d], {MAT_BYTES}", f"global_load_lds_dwordx4 {vr(LOAD_OFF)}, %[vb] nt"]
+    parts.append(asm_fn(pre + "issue_band", "const void* k_rows, const void* v_rows, uint32_t lds_dst", join(issue),
+                        ins=['[kb] "s"(k_rows)', '[vb] "s"(v_rows)', '[d] "s"(lds_dst)'], clobbers=["memory", "m0", "scc"],
+                        comment="The wave's two direct-to-LDS loads of a tile whose 8 rows of the wave are all cached rows." + what))
+    req = [f"global_load_dwordx4 {vr(SA + 4 * c, 4)}, %[p{c // 4}], off offset:{(c % 4) * 1024} sc1" for c in range(2 * NDB + 1)]
+    parts.append(asm_fn(pre + "request_partial", "const void* p0, const void* p1", join(req),
+                        ins=['[p0] "v"(p0)', '[p1] "v"(p1)'], clobbers=["memory"],
+                        comment="pipe_request_partial() for a block of four chunks and the statistics (p1: 4 KiB behind p0)." + what))
+    parts.append(asm_fn(pre + "first_scores", "uint32_t k_next, float& mx", first_scores_block(SA),
+                        ['[mx] "=&v"(mx)'], ['[k0] "v"(k_next)'], ["memory"],
+                        "S^T of a run's first tile into score set A, and the lane's maximum." + what))
+    parts.append(step_fns(pre + "step_ab", SA, SB, True, "One step, in two halves (_x then _y), as pipe_step_ab." + what))
+    parts.append(step_fns(pre + "step_ba", SB, SA, True))
+    parts.append(step_fns(pre + "last_a", SA, SB, False, "Last step of a run: no next tile." + what))
+    parts.append(step_fns(pre + "last_b", SB, SA, False))
+    set_head_dim(128)
+    return "".join(parts)
 
 
 def generate():
@@ -614,6 +677,7 @@ DFX_D void pipe_outputs_ready() { asm volatile("s_nop 15\\n\\ts_nop 1" ::: "memo
                         comment="The wave's four direct-to-LDS loads of a full tile of cached rows in the distinct layout: its two chunk\n"
                                 "columns of K (64 tokens of each at k_col0 / k_col1) and its 16 rows of V^T (v_rows: the tile's first token\n"
                                 "in row 0 of the (page, head)); lds_dst: the wave's place in the K tile of the ring stage."))
+    parts.append(head_dim_64_family())
     parts.append("}  // namespace dfx\n")
     return "".join(parts)
 

@@ -88,6 +88,9 @@ int make_plan(const dfx_attn_params* p, Plan& plan) {
     // at the C3 shape -17 %, 32 rows -1 to -15 %) while a workgroup has few items to open and close; with
     // four short items each the two workgroups per compute unit are ahead (64 rows: by 22 %, 32 rows: by
     // 7 %), and a launch cannot see lengths.
+    // (head_dim 64, whose tiles are half the bytes and the matrix work: 4 waves, two workgroups per compute unit, stay
+    // ahead up to the 128 rows they can hold -- 96 rows of the C4 kind: 150 us against 169 -- and the 8-wave pipelined
+    // kernel takes over from 129 rows on: 224 rows of the C3 kind 42.4 us against 47.3)
     if (plan.stream && plan.hd == 128 && !(p->flags & DFX_ATTN_NO_PIPELINE)) {
         const int64_t items = static_cast<int64_t>(p->num_seqs) * p->num_kv_heads;
         if (rows > 64 || items <= 2 * static_cast<int64_t>(device_cu_count())) plan.nb = 2;
@@ -96,7 +99,7 @@ int make_plan(const dfx_attn_params* p, Plan& plan) {
 
     // (8 waves only: with 4 waves a wave has twice the tile loads to address, and the 32 registers
     // the pipelined kernel leaves the compiler no longer hold that without spilling in the loop)
-    plan.pipelined = plan.stream && !plan.compact && plan.hd == 128 && plan.nb == 2 &&
+    plan.pipelined = plan.stream && !plan.compact && (plan.hd == 128 || !plan.fp8) && plan.nb == 2 &&
                      !(p->flags & DFX_ATTN_NO_PIPELINE);
     if (p->max_workgroups > 0) {
         plan.n_wg = p->max_workgroups;
@@ -191,6 +194,12 @@ int launch(const KArgs& ka, const Plan& plan, hipStream_t st, const PlanArgs* pa
                     }
                 }
             }
+            if constexpr (HD == 64 && NW == 8) {
+                if (plan.pipelined) {
+                    main_k = paged_attn_pipe_kernel<NW, false, false, 64>;
+                    slot = 34;
+                }
+            }
             lds = C::LDS_BYTES;
             plan_k = paged_attn_plan_kernel<C::RT>;
             plan_slot = C::RT == 256 ? 31 : 30;
@@ -277,7 +286,7 @@ int check_args(const dfx_attn_params* p, Plan& plan, bool& empty) {
     if (!(p->scale > 0.0f) || p->diffusion_block_size <= 0) return DFX_ERR_INVALID_ARG;
     if (p->mask_mode != DFX_MASK_FULL && p->mask_mode != DFX_MASK_BLOCK_CAUSAL) return DFX_ERR_INVALID_ARG;
     if (p->rope_cos_sin != nullptr) {
-        if (!plan.pipelined || !has_cache || plan.distinct) return DFX_ERR_UNSUPPORTED;
+        if (!plan.pipelined || !has_cache || plan.distinct || plan.hd != 128) return DFX_ERR_UNSUPPORTED;
         if (!p->rope_positions || !p->k_rotated || p->rope_max_position <= 0 || p->k_rotated == p->k_new) return DFX_ERR_INVALID_ARG;
         if (p->rope_position_index_type != DFX_INDEX_I32 && p->rope_position_index_type != DFX_INDEX_I64) return DFX_ERR_INVALID_ARG;
         if (p->kr_stride_token < 0 || p->kr_stride_token % 8 || p->kr_stride_head < 0 || p->kr_stride_head % 8) return DFX_ERR_INVALID_ARG;

@@ -988,6 +988,8 @@ PLAN_CASES = [
     ("c4", dict(num_seqs=3, ctx=(100, 500))),                # compact kernel, block-causal
     ("c5", dict(num_seqs=4, ctx=(200, 900))),                # FP8 streaming kernel
     ("c1", {}),                                              # head_dim 64
+    ("c3", dict(num_seqs=12, ctx=(50, 1200), hd=64)),        # head_dim 64 with 224 rows: the pipelined kernel's narrow variant, cut items
+    ("c3", dict(num_seqs=5, ctx=[0, 1, 63, 64, 700], hd=64, page=16)),
 ]
 
 

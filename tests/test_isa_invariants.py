@@ -81,8 +81,9 @@ def test_tile_loop_has_no_spills_and_no_compiler_waits(isa, kernel, max_waits):
     assert ops["global_load_lds_dwordx4"] in (2, 4, 8)   # a wave's share of the 64 * head_dim * elt * 2 bytes of a tile
 
 
-PIPE_KERNELS = ["_ZN3dfx22paged_attn_pipe_kernelILi8ELb0ELb0E", "_ZN3dfx22paged_attn_pipe_kernelILi8ELb1ELb0E",
-                "_ZN3dfx22paged_attn_pipe_kernelILi8ELb0ELb1E",   # the distinct cache layout
+PIPE_KERNELS = ["_ZN3dfx22paged_attn_pipe_kernelILi8ELb0ELb0ELi128E", "_ZN3dfx22paged_attn_pipe_kernelILi8ELb1ELb0ELi128E",
+                "_ZN3dfx22paged_attn_pipe_kernelILi8ELb0ELb1ELi128E",   # the distinct cache layout
+                "_ZN3dfx22paged_attn_pipe_kernelILi8ELb0ELb0ELi64E",    # head_dim 64
                 "_ZN3dfx26paged_attn_pipe_fp8_kernelILi8E"]
 
 
@@ -124,8 +125,8 @@ def test_pipelined_kernel_leaves_the_generated_blocks_registers_alone(isa, kerne
     assert int(re.search(r"\.amdhsa_accum_offset (\d+)", isa[i:i + 3000]).group(1)) == 128
     loop = _tile_loop(isa, kernel)
     ops = collections.Counter(l.split()[0] for l in loop)
-    # first tile of a run 16, two steps 32 each, two steps 32 + 16 each, two plain steps 32 each
-    assert ops["v_mfma_f32_32x32x16_bf16"] == 176
+    # first tile of a run 16, two steps 32 each, two steps 32 + 16 each, two plain steps 32 each (head_dim 64: half)
+    assert ops["v_mfma_f32_32x32x16_bf16"] == (88 if "ELi64E" in kernel else 176)
     # (the FP8 kernel carries more per-item state in scalar registers, some of which the compiler parks in
     # scratch until the item's rows are written: behind the steps, where no tile load is waited for by count)
     mfma = [i for i, l in enumerate(loop) if l.startswith("v_mfma")]

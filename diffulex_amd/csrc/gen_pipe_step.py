@@ -9,7 +9,10 @@ instruction stream alternates between them: a 32x32x16 matrix instruction occupi
 for 8 passes, in whose shadow the wave can issue four or five independent vector instructions.
 One step therefore computes S^T = K Q^T of the NEXT tile and O^T += V^T P^T of the CURRENT tile,
 with the softmax of the current tile (exp2, row sum, bf16 rounding) and the row maximum of the
-next one cut into pieces between the matrix instructions.  Left to the compiler, loop-carried
+next one cut into pieces between the matrix instructions.  Both waves of a SIMD reach the start of
+a phase together (behind the step's barrier), where the matrix unit would idle until the first
+operands have come from LDS: phase X does a dozen of its vector instructions there, and the first
+operands of phase Y are requested from the tail of phase X.  Left to the compiler, loop-carried
 matrix state around inline assembly is copied between registers (or spilled) at control-flow
 merges.  The kernel that uses these blocks is therefore compiled with amdgpu_num_vgpr(32): the
 compiler allocates v0..v31 and a0..a31 only, and the matrix state lives in the registers above,
@@ -80,6 +83,7 @@ MAT_BYTES = 64 * ROWB       # K tile; the V tile of a ring stage follows it
 LAYOUT = "u"
 CHUNK_COL_BYTES = 64 * 16
 NEG_INF = "0xff800000"
+FRONT_X = 12                # vector instructions of phase X ahead of its first matrix instruction
 MFMA_TO_VALU = ["s_nop 15", "s_nop 1"]  # 18 wait states: the longest the ISA asks for
 
 
@@ -89,6 +93,14 @@ def vr(base, n=1):
 
 def ar(base, n=1):
     return f"a{base}" if n == 1 else f"a[{base}:{base + n - 1}]"
+
+
+NBUF = 4                    # operand ring buffers (4 registers each): operands are read NBUF - 1 matrix instructions ahead
+
+
+def ring(n, cnt=4, sub=0):
+    """Registers sub .. sub + cnt - 1 of operand ring buffer n % NBUF."""
+    return vr(RING + 4 * (n % NBUF) + sub, cnt)
 
 
 def swizzle(row):
@@ -198,9 +210,13 @@ def emit_valu(b, stream, n):
             b.valu(text, defs)
 
 
-def phase_x(b, nxt, stream, quotas):
+def phase_x(b, nxt, stream, quotas, front=0, tail_read=None):
     """S^T of the next tile into set `nxt`: 16 matrix instructions (slab-major, token block minor),
-    K operands read three ahead through the ring, `quotas[i]` vector instructions behind the i-th.
+    K operands read three ahead through the ring, `front` vector instructions between the first
+    reads and the first matrix instruction (work for the time the reads take), `quotas[i]` behind the
+    i-th.  tail_read(j): issues operand read j (0..2) of the phase that follows, in the places of the
+    K reads the last three matrix instructions no longer need (the ring buffer each goes to was last
+    read by the matrix instruction issued just before, as with the K reads).
     (LDS instructions take their address when they issue, in program order: the address register
     may be rewritten for the next slab right behind the read.)"""
     n = 2 * NSLAB
@@ -208,50 +224,58 @@ def phase_x(b, nxt, stream, quotas):
     def read(i):
         slab, tb = i >> 1, i & 1
         if LAYOUT == "d":  # chunk column 2 slab + half, tokens 32 tb ..: every offset an immediate
-            b.lds_read(f"ds_read_b128 {vr(RING + 4 * (i % 4), 4)}, %[k0] offset:{slab * 2 * CHUNK_COL_BYTES + tb * 32 * 16}", ("k", i))
+            b.lds_read(f"ds_read_b128 {ring(i)}, %[k0] offset:{slab * 2 * CHUNK_COL_BYTES + tb * 32 * 16}", ("k", i))
             return
         if tb == 0 and slab > 0:
             b.valu(f"v_xor_b32 {vr(T_ADDR)}, {slab * 32:#x}, %[k0]", {T_ADDR})
         addr = "%[k0]" if slab == 0 else vr(T_ADDR)
-        b.lds_read(f"ds_read_b128 {vr(RING + 4 * (i % 4), 4)}, {addr} offset:{tb * 32 * ROWB}", ("k", i))
+        b.lds_read(f"ds_read_b128 {ring(i)}, {addr} offset:{tb * 32 * ROWB}", ("k", i))
 
-    for i in range(3):
+    A = NBUF - 1
+    for i in range(A):
         read(i)
+    emit_valu(b, stream, front)
     for i in range(n):
-        if i + 3 < n:
-            read(i + 3)
+        if i + A < n:
+            read(i + A)
+        elif tail_read is not None:
+            tail_read(i + A - n)
         b.wait_lds(("k", i))
         slab, tb = i >> 1, i & 1
         dst = vr(nxt + 16 * tb, 16)
-        b.mfma(dst, vr(RING + 4 * (i % 4), 4), ar(Q_BASE + 4 * slab, 4), "0" if slab == 0 else dst, reads=())
+        b.mfma(dst, ring(i), ar(Q_BASE + 4 * slab, 4), "0" if slab == 0 else dst, reads=())
         emit_valu(b, stream, quotas[i])
 
 
-def phase_y(b, cur, stream, quotas):
+def y_operand_read(b, j):
+    """Read of the V^T operand of matrix instruction j of phase Y into ring buffer j % 4."""
+    tb, sl, db = j // (2 * NDB), (j // NDB) & 1, j % NDB
+    if LAYOUT == "d":  # row 32 db + lane % 32 of V^T, the 8 tokens of the lane's half of the slab: one read
+        b.lds_read(f"ds_read_b128 {ring(j)}, {vr(T_VADDR + 2 * tb + sl)} offset:{db * 32 * 128}", ("v", j, 1))
+        return
+    for ii in range(2):
+        off = (tb * 32 + sl * 16 + ii * 8) * ROWB
+        b.lds_read(f"ds_read_b64_tr_b16 {ring(j, 2, 2 * ii)}, {vr(T_VADDR + 2 * db + ii)} offset:{off}",
+                   ("v", j, ii))
+
+
+def phase_y(b, cur, stream, quotas, hoisted=False):
     """O^T += V^T P^T of the current tile: 16 matrix instructions ordered (token block, 16-token
-    slab, d block), V^T operands (two transposing 8-byte reads each) two instructions ahead."""
+    slab, d block), V^T operands (two transposing 8-byte reads each) three instructions ahead; the
+    first three reads are in flight already if `hoisted` (phase X has issued them: b.lds_queue)."""
     n = 4 * NDB
-
-    def read(j):
-        tb, sl, db = j // (2 * NDB), (j // NDB) & 1, j % NDB
-        if LAYOUT == "d":  # row 32 db + lane % 32 of V^T, the 8 tokens of the lane's half of the slab: one read
-            b.lds_read(f"ds_read_b128 {vr(RING + 4 * (j % 4), 4)}, {vr(T_VADDR + 2 * tb + sl)} offset:{db * 32 * 128}", ("v", j, 1))
-            return
-        for ii in range(2):
-            off = (tb * 32 + sl * 16 + ii * 8) * ROWB
-            b.lds_read(f"ds_read_b64_tr_b16 {vr(RING + 4 * (j % 4) + 2 * ii, 2)}, {vr(T_VADDR + 2 * db + ii)} offset:{off}",
-                       ("v", j, ii))
-
-    read(0)
-    read(1)
+    A = NBUF - 1
+    if not hoisted:
+        for j in range(A):
+            y_operand_read(b, j)
     for j in range(n):
-        if j + 2 < n:
-            read(j + 2)
+        if j + A < n:
+            y_operand_read(b, j + A)
         b.wait_lds(("v", j, 1))
         tb, sl, db = j // (2 * NDB), (j // NDB) & 1, j % NDB
         acc = ar(O_BASE + 16 * db, 16)
         p = cur + 8 * tb + 4 * sl
-        b.mfma(acc, vr(RING + 4 * (j % 4), 4), vr(p, 4), acc, reads=range(p, p + 4))
+        b.mfma(acc, ring(j), vr(p, 4), acc, reads=range(p, p + 4))
         emit_valu(b, stream, quotas[j])
 
 
@@ -268,22 +292,28 @@ def step_blocks(cur, nxt, has_next):
     blocks so that a wave can issue its tile loads between them."""
     pairs = [pair_instrs(cur, pr) for pr in range(16)]
     flat = lambda ps: [ins for p in ps for ins in p]
-    sx = flat(pairs[:9]) + vaddr_instrs()
+    sx = vaddr_instrs() + flat(pairs[:9])  # (the addresses first: the tail of phase X reads with them)
     y1 = flat(pairs[9:14])
     y2a = flat(pairs[14:16])
     bx = Block()
     bx.other("s_waitcnt lgkmcnt(0)")
     by = Block()
-    by.other("s_waitcnt lgkmcnt(0)")
     half, quarter = 2 * NDB, NDB  # of the 4 * NDB matrix instructions of phase Y (head_dim 128: 8 and 4)
     if has_next:
-        phase_x(bx, nxt, sx, spread(len(sx), 2 * NSLAB))
+        # The matrix unit would idle while a phase's first operands travel from LDS (both waves of a SIMD reach
+        # that point together, behind the step's barrier).  Phase X therefore does FRONT_X of its vector
+        # instructions there, and phase Y's first three operands are requested from the tail of phase X.
+        phase_x(bx, nxt, sx, spread(len(sx) - FRONT_X, 2 * NSLAB), FRONT_X, lambda j: y_operand_read(bx, j))
+        # (phase Y starts with those reads in the queue and no wait of its own: whatever the compiler puts between
+        # the two blocks is younger than they are, and the queue returns in order)
+        by.lds_queue, bx.lds_queue = bx.lds_queue, []
         y2 = y2a + max_instrs(nxt)
         qa = spread(len(y2a) + 4, quarter)
         sy = y1 + y2
         quotas = spread(len(y1), half) + qa + spread(len(y2) - sum(qa), quarter)
     else:
         emit_valu(bx, sx, len(sx))
+        by.other("s_waitcnt lgkmcnt(0)")
         sy = y1 + y2a
         quotas = spread(len(y1), half) + spread(len(y2a), quarter) + [0] * quarter
     # every pair is complete before the matrix instruction that reads it: instruction j (token block tb, slab sl)
@@ -291,7 +321,7 @@ def step_blocks(cur, nxt, has_next):
     for j in range(4 * NDB):
         last_pair = 8 * (j // (2 * NDB)) + 4 * ((j // NDB) & 1) + 3
         assert sum(quotas[:j]) >= 7 * max(0, last_pair - 8), (HD, j)
-    phase_y(by, cur, sy, quotas)
+    phase_y(by, cur, sy, quotas, hoisted=has_next)
     assert not sx and not sy and not bx.lds_queue and not by.lds_queue
     return bx.text(), by.text()
 

@@ -21,6 +21,7 @@ PKG_DIR = Path(__file__).resolve().parent
 CSRC = PKG_DIR / "csrc"
 LIB_PATH = PKG_DIR / "libdiffulex_amd.so"
 OPS_PATH = PKG_DIR / "_torch_ops.so"
+STEP_BENCH_PATH = PKG_DIR / "build" / "step_bench"
 ARCH = "gfx950"
 
 # packed-fp32 instructions are kept out of the generated code on purpose
@@ -49,13 +50,34 @@ def _compile(src: Path, obj: Path) -> None:
         sys.stderr.write(err + "\n")
 
 
-def _generate() -> None:
-    """Run the source generators under csrc/ (the hand-scheduled tile step of the streaming kernel)."""
+def _generator():
     import importlib.util
     spec = importlib.util.spec_from_file_location("gen_pipe_step", CSRC / "gen_pipe_step.py")
     mod = importlib.util.module_from_spec(spec)
     spec.loader.exec_module(mod)
-    mod.main()
+    return mod
+
+
+def _generate() -> None:
+    """Run the source generators under csrc/ (the hand-scheduled tile step of the streaming kernel)."""
+    _generator().main()
+
+
+def build_step_bench(verbose: bool = True) -> Path:
+    """The microbenchmark of the generated tile step (csrc/step_bench.hip): an executable, with the
+    timing variants of the blocks it compares the step with generated into build/."""
+    obj_dir = PKG_DIR / "build"
+    obj_dir.mkdir(exist_ok=True)
+    gen = _generator()
+    for only in ("mfma", "valu", "lds"):
+        gen.main(out=str(obj_dir / f"step_only_{only}.h"), only=only, namespace=f"dfx_only_{only}")
+    cmd = [_hipcc(), *[f for f in HIP_FLAGS if f != "-fPIC"], f"-I{CSRC}", "-x", "hip", str(CSRC / "step_bench.hip"), "-o", str(STEP_BENCH_PATH)]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError(f"hipcc failed for step_bench.hip:\n{res.stderr[-4000:]}")
+    if verbose:
+        print(f"built {STEP_BENCH_PATH} ({STEP_BENCH_PATH.stat().st_size} bytes)")
+    return STEP_BENCH_PATH
 
 
 def build(verbose: bool = True) -> Path:
@@ -74,6 +96,7 @@ def build(verbose: bool = True) -> Path:
     if verbose:
         print(f"built {LIB_PATH} ({LIB_PATH.stat().st_size} bytes)")
     build_torch_ops(verbose)
+    build_step_bench(verbose)
     return LIB_PATH
 
 

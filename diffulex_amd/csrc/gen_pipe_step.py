@@ -85,6 +85,11 @@ CHUNK_COL_BYTES = 64 * 16
 NEG_INF = "0xff800000"
 FRONT_X = 12                # vector instructions of phase X ahead of its first matrix instruction
 MFMA_TO_VALU = ["s_nop 15", "s_nop 1"]  # 18 wait states: the longest the ISA asks for
+# Timing variants for step_bench.hip (never for the library): the step blocks with only one class of their
+# instructions -- "mfma", "valu" (the softmax arithmetic) or "lds" (the operand reads).  Their results are meaningless.
+ONLY = None
+NAMESPACE = "dfx"
+SOFTMAX_OPS = ("v_fma_f32", "v_exp_f32", "v_add_f32", "v_cvt_pk_bf16_f32", "v_max3_f32", "v_max_f32")
 
 
 def vr(base, n=1):
@@ -126,12 +131,16 @@ class Block:
         self.recent_valu_defs = (self.recent_valu_defs + [set(defs)])[-2:]
 
     def valu(self, text, defs):
+        if ONLY in ("mfma", "lds") and text.split()[0] in SOFTMAX_OPS:
+            return
         self._push(text, defs)
 
     def other(self, text):
         self._push(text)
 
     def lds_read(self, text, tag):
+        if ONLY in ("mfma", "valu"):
+            return
         self._push(text)
         self.lds_queue.append(tag)
 
@@ -145,6 +154,8 @@ class Block:
 
     def mfma(self, dst, a, b, c, reads):
         """reads: registers (numbers) of vector operands a/b/c written by the vector ALU."""
+        if ONLY in ("valu", "lds"):
+            return
         if any(set(reads) & d for d in self.recent_valu_defs):
             self._push("s_nop 1")
         self._push(f"v_mfma_f32_32x32x16_bf16 {dst}, {a}, {b}, {c}")
@@ -513,8 +524,8 @@ def generate():
 
 #include "dfx_common.h"
 
-namespace dfx {
-
+namespace ''' + NAMESPACE + ''' {
+''' + ("" if NAMESPACE == "dfx" else "using namespace ::dfx;\n") + '''
 ''']
     parts.append(asm_fn("pipe_reserve", "", "", clobbers=reserved,
                         comment="Makes the kernel's register count cover the registers of the blocks below (no instruction)."))
@@ -708,13 +719,20 @@ DFX_D void pipe_outputs_ready() { asm volatile("s_nop 15\\n\\ts_nop 1" ::: "memo
                                 "columns of K (64 tokens of each at k_col0 / k_col1) and its 16 rows of V^T (v_rows: the tile's first token\n"
                                 "in row 0 of the (page, head)); lds_dst: the wave's place in the K tile of the ring stage."))
     parts.append(head_dim_64_family())
-    parts.append("}  // namespace dfx\n")
+    parts.append(f"}}  // namespace {NAMESPACE}\n")
     return "".join(parts)
 
 
-def main():
-    out = os.path.join(HERE, "attn_pipe_gen.h")
-    text = generate()
+def main(out=None, only=None, namespace="dfx"):
+    """Writes the blocks to `out` (default: attn_pipe_gen.h beside this file, what the library is built from).
+    only / namespace: a timing variant for step_bench.hip in a namespace of its own."""
+    global ONLY, NAMESPACE
+    out = out or os.path.join(HERE, "attn_pipe_gen.h")
+    ONLY, NAMESPACE = only, namespace
+    try:
+        text = generate()
+    finally:
+        ONLY, NAMESPACE = None, "dfx"
     if not os.path.exists(out) or open(out).read() != text:
         with open(out, "w") as f:
             f.write(text)

@@ -1229,3 +1229,21 @@ def test_reordered_plan_with_sequences_of_no_or_few_tiles(dev, ctx):
         torch.cuda.synchronize()
         assert max_abs_err(got, want) <= ATOL_BF16
         assert max_abs_err(got, kept) <= 1e-2
+
+
+def test_step_microbenchmark_runs(dev):
+    """diffulex_amd/build/step_bench (csrc/step_bench.hip): the generated step on LDS-resident tiles.  A step holds
+    2048 cycles of matrix instructions per SIMD; whatever the schedule, it cannot be faster, and a step beyond
+    twice that would mean the blocks no longer overlap anything."""
+    import re
+    import subprocess
+    from diffulex_amd import build as dbuild
+    if not dbuild.STEP_BENCH_PATH.exists():
+        pytest.fail("diffulex_amd/build/step_bench has not been built (python -m diffulex_amd.build)")
+    out = subprocess.run([str(dbuild.STEP_BENCH_PATH), "200"], capture_output=True, text=True, timeout=100)
+    assert out.returncode == 0, out.stdout + out.stderr
+    rows = re.findall(r"^(.+?)\s+(\d+) workgroups\s+tile loads (\w+)\s+(\d+) cycles/step", out.stdout, re.M)
+    assert len(rows) == 10, out.stdout
+    for name, _, _, cycles in rows:
+        lo, hi = {"the step": (2048, 4096), "matrix instructions only": (2048, 3000)}.get(name.strip(), (500, 2500))
+        assert lo <= int(cycles) <= hi, (name, cycles)

@@ -146,3 +146,23 @@ def test_pipelined_kernel_leaves_the_generated_blocks_registers_alone(isa, kerne
         elif not in_asm and l.startswith("s_waitcnt") and "vmcnt" in l:
             waits += 1
     assert waits <= (6 if "fp8" in kernel else 0), waits
+
+
+def test_timing_variants_of_the_step_hold_one_class_of_instructions(tmp_path):
+    """csrc/step_bench.hip compares the step with variants of its blocks that hold the matrix instructions, the
+    softmax arithmetic or the operand reads alone (gen_pipe_step.main(only=...)): each in a namespace of its
+    own, and generating them leaves the library's header as it is."""
+    gen = dbuild._generator()
+    lib_header = (ROOT / "diffulex_amd" / "csrc" / "attn_pipe_gen.h").read_text()
+    counts = {}
+    for only in (None, "mfma", "valu", "lds"):
+        out = tmp_path / f"{only}.h"
+        gen.main(out=str(out), only=only, namespace="dfx" if only is None else f"dfx_only_{only}")
+        text = out.read_text()
+        step = text[text.index("void pipe_step_ab_x("):text.index("void pipe_step_ba_x(")]
+        counts[only] = (step.count("v_mfma_f32"), step.count("v_exp_f32"), step.count("ds_read_"))
+        assert (f"namespace dfx_only_{only} {{" in text) == (only is not None)
+    assert gen.main(out=str(tmp_path / "again.h")) and (tmp_path / "again.h").read_text() == lib_header == (tmp_path / "None.h").read_text()
+    mfma, exp2, reads = counts[None]
+    assert (mfma, exp2) == (32, 32) and reads == 16 + 32
+    assert counts["mfma"] == (mfma, 0, 0) and counts["valu"] == (0, exp2, 0) and counts["lds"] == (0, 0, reads)

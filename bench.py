@@ -303,7 +303,7 @@ def bench_prefill(args, dev):
                                f"block-causal mask, {dbs}-token blocks, no cache", "spin_up_launches": n_spin},
         "roofline": {"bound": "mfma", "achieved": tflops, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": tflops / MFMA_BF16_PEAK_TFLOPS, "traffic": None, "algorithmic_flops": nflops,
-                     "kernel": "paged_attn_pipe_kernel<8, true, false>, duration = timed region / steps"},
+                     "kernel": "paged_attn_pipe_kernel<8, true, false, 128>, duration = timed region / steps"},
     }))
 
 
@@ -458,8 +458,8 @@ def bench_layer(args, dev):
                    "tensor_sets_rotated": n_sets, "spin_up_launches": n_spin},
         "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS,
                      "traffic": None, "algorithmic_bytes": nbytes,
-                     "kernel": ("paged_attn_pipe_kernel<8, false, false> with the rotary embedding inside" if fused else
-                                "rope_kv_store_kernel + paged_attn_pipe_kernel<8, false, false>") +
+                     "kernel": ("paged_attn_pipe_kernel<8, false, false, 128> with the rotary embedding inside" if fused else
+                                "rope_kv_store_kernel + paged_attn_pipe_kernel<8, false, false, 128>") +
                                " (+ plan kernels once per graph), duration = graph replay / layers"},
     }))
 
@@ -529,7 +529,7 @@ def bench_d2f_small(args, dev):
                    "batches": rows, "host_wall_ms_per_step": worst["host_wall_ms_per_layer"]},
         "roofline": {"bound": "hbm", "achieved": worst["gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": worst["gbs"] / HBM_PEAK_GBS, "traffic": None, "algorithmic_bytes": worst["algorithmic_bytes"],
-                     "kernel": "paged_attn_pipe_kernel<8, false, false> (+ kv store), duration = max(GPU events, host issue) / layers"},
+                     "kernel": "paged_attn_pipe_kernel<8, false, false, 128> (+ kv store), duration = max(GPU events, host issue) / layers"},
     }))
 
 
@@ -663,8 +663,8 @@ def main():
     traffic, traffic_source = measured_traffic(args.workload, nbytes) if not over and args.layout == "unified" else (None, None)
     kernel = ("paged_attn_stream_kernel (head_dim 64: the compiler-scheduled step)" if wl.head_dim != 128 else
               "paged_attn_pipe_fp8_kernel<8>" if wl.kv_fp8 else
-              "paged_attn_pipe_kernel<8, false, false>" if args.layout == "unified" else
-              "paged_attn_pipe_kernel<8, false, true>")
+              "paged_attn_pipe_kernel<8, false, false, 128>" if args.layout == "unified" else
+              "paged_attn_pipe_kernel<8, false, true, 128>")
     result = {
         "metric": "attn query-tokens/sec + achieved HBM GB/s (% of peak), Dream-7B shape, 1 GPU",
         "value": wl.total_q_tokens / (ms * 1e-3), "unit": "query-tokens/s",

@@ -475,6 +475,24 @@ def test_full_size_c4_and_c5_on_sampled_sequences(dev):
         torch.cuda.empty_cache()
 
 
+def test_full_size_c3_with_head_dim_64_on_sampled_sequences(dev):
+    """The C3 shape with the head size of the reference's kernel tests (224 rows per item: the pipelined kernel's
+    head_dim 64 variant), without a plan and with the default one, against the oracle on sampled sequences and
+    against the compiler-scheduled step."""
+    wl = make_workload("c3", device=dev, hd=64)
+    seqs = [0, 21, 40, 63]
+    want = oracle_fp32(wl, seqs=seqs)
+    cu = wl.cu_seqlens_q.tolist()
+    cache = {}
+    outs = [_run(wl), _run(wl, plan_cache=cache), _run(wl, plan_cache=cache), _run(wl, flags=_lib.DFX_ATTN_NO_PIPELINE)]
+    for out in outs:
+        assert torch.isfinite(out.float()).all()
+        for s, w in zip(seqs, want):
+            assert max_abs_err(out[cu[s]:cu[s + 1]], w) <= ATOL_BF16, s
+    assert torch.equal(outs[1], outs[2])
+    assert max_abs_err(outs[0], outs[3]) <= 1e-2
+
+
 def test_the_planned_launch_the_benchmark_times_against_the_oracle(dev):
     """Full C3 with the default plan (cut points from the capacity sweep: plan mode 2), the launch the
     headline figure is measured on: against the oracle on sampled sequences, and the same bits from

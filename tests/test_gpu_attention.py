@@ -168,6 +168,7 @@ def test_fresh_k_and_v_with_different_strides(dev):
     ("c1", {}),                                          # head_dim 64, two workgroups per compute unit
     ("c5", dict(num_seqs=4, ctx=(200, 900))),            # FP8 cache: fresh rows fetched by the widening step
     ("c4", dict(num_seqs=3, ctx=(100, 500))),            # block-causal, 96 fresh rows per sequence
+    ("c3", dict(num_seqs=6, ctx=(100, 900), hd=64)),     # 8 waves, the pipelined tile loop for head_dim 64
 ])
 def test_fresh_v_sliced_out_of_the_projection(dev, name, over, flags):
     """What a decoder layer passes: K rotated into a buffer of its own, V still a column slice of
@@ -688,6 +689,7 @@ def test_graph_buffers_padded_the_way_the_reference_pads_them(dev, name, over, n
     ("c4", dict(num_seqs=3, ctx=(100, 500))),
     ("c5", dict(num_seqs=4, ctx=(200, 900))),
     ("c5", dict(num_seqs=3, ctx=[256, 0, 511], h_q=8, h_kv=2, hd=64, page=32)),
+    ("c3", dict(num_seqs=5, ctx=(100, 800), hd=64)),     # 224 rows, head_dim 64: the pipelined kernel's narrow variant
 ])
 def test_store_fused_into_the_attention_launch(dev, name, over, flags):
     """One launch that stores the fresh block and attends == the store launch followed by the

@@ -98,8 +98,12 @@ def test_attention_module_with_rope_takes_the_one_launch_path_and_matches_the_tw
     assert torch.equal(_bits(caches[0][0]), _bits(caches[1][0])) and torch.equal(_bits(caches[0][1]), _bits(caches[1][1]))
 
 
-def test_shapes_without_a_pipelined_kernel_refuse_the_rope_and_the_module_falls_back(dev):
-    wl = make_workload("c1", device=dev)                      # head_dim 64: no pipelined kernel
+@pytest.mark.parametrize("name,over", [
+    ("c1", {}),                                               # head_dim 64, 64 rows: no pipelined kernel
+    ("c3", dict(num_seqs=3, ctx=(100, 600), hd=64)),          # head_dim 64, 224 rows: its pipelined kernel does not rotate
+])
+def test_shapes_whose_kernel_does_not_rotate_refuse_the_rope_and_the_module_falls_back(dev, name, over):
+    wl = make_workload(name, device=dev, **over)
     T, hq, hkv, hd = wl.q.shape[0], wl.num_q_heads, wl.num_kv_heads, wl.head_dim
     rope = RotaryEmbedding(hd, hd, 512, 10000.0).to(dev)
     pos = torch.arange(T, device=dev) % 512

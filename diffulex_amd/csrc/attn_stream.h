@@ -604,23 +604,30 @@ struct StreamAttn : TileMath<HD, NB, NW, HIDDEN> {
         for (int64_t idx = thread_number_here(wave_s); idx < (n1 - n0) * 8; idx += C::THREADS) {
             const int64_t t = n0 + (idx >> 3);
             const int c = static_cast<int>(idx & 7);
+            // The slot first: its load travels with that of the position, and with a two-byte cache the V chunks
+            // then travel with the K chunks and the angles (two trips to memory instead of four).
+            int64_t slot = -1;
+            if (a.store_slots != nullptr)
+                slot = a.store_slots_i64 ? static_cast<const int64_t*>(a.store_slots)[t]
+                                         : static_cast<int64_t>(static_cast<const int32_t*>(a.store_slots)[t]);
+            const int64_t pos = rope_position(t);
+            const bool stored = slot >= 0 && slot < n_slots;
+            const int64_t page = a.page_shift >= 0 ? (slot >> a.page_shift) : slot / a.page_size;
+            const int64_t e = page * a.c_sp + (slot - page * a.page_size) * a.c_st + kv_head * a.c_sh + c * 8;  // elements
+            const uint16_t* vp = a.v_new + t * a.vn_st + kv_head * a.vn_sh + c * 8;
+            uint8_t* kc = const_cast<uint8_t*>(a.k_cache);
+            uint8_t* vc = const_cast<uint8_t*>(a.v_cache);
             uint32_t lo[4], hi[4];
-            pipe_rope_row(a.k_src + t * a.ks_st + kv_head * a.ks_sh + c * 8, a.rope_table + rope_position(t) * HD + c * 8, lo, hi);
+            const uint16_t* ksrc = a.k_src + t * a.ks_st + kv_head * a.ks_sh + c * 8;
+            if (!FP8 && stored) pipe_rope_row_with_v(ksrc, a.rope_table + pos * HD + c * 8, vp, vc + e * 2, lo, hi);
+            else pipe_rope_row(ksrc, a.rope_table + pos * HD + c * 8, lo, hi);
             const u32x4 o1 = {lo[0], lo[1], lo[2], lo[3]}, o2 = {hi[0], hi[1], hi[2], hi[3]};
             uint16_t* dst = const_cast<uint16_t*>(a.k_new) + t * a.kn_st + kv_head * a.kn_sh + c * 8;
             *reinterpret_cast<u32x4*>(dst) = o1;
             *reinterpret_cast<u32x4*>(dst + HD / 2) = o2;
-            if (a.store_slots == nullptr) continue;
-            int64_t slot = a.store_slots_i64 ? static_cast<const int64_t*>(a.store_slots)[t]
-                                             : static_cast<int64_t>(static_cast<const int32_t*>(a.store_slots)[t]);
-            if (slot < 0 || slot >= n_slots) continue;
-            const int64_t page = a.page_shift >= 0 ? (slot >> a.page_shift) : slot / a.page_size;
-            const int64_t e = page * a.c_sp + (slot - page * a.page_size) * a.c_st + kv_head * a.c_sh + c * 8;  // elements
-            const uint16_t* vp = a.v_new + t * a.vn_st + kv_head * a.vn_sh + c * 8;
-            const u32x4 v1 = *reinterpret_cast<const u32x4*>(vp), v2 = *reinterpret_cast<const u32x4*>(vp + HD / 2);
-            uint8_t* kc = const_cast<uint8_t*>(a.k_cache);
-            uint8_t* vc = const_cast<uint8_t*>(a.v_cache);
+            if (!stored) continue;
             if constexpr (FP8) {
+                const u32x4 v1 = *reinterpret_cast<const u32x4*>(vp), v2 = *reinterpret_cast<const u32x4*>(vp + HD / 2);
                 const float ks = a.k_scale[kv_head], vs = a.v_scale[kv_head];
                 *reinterpret_cast<u32x2*>(kc + e) = quantise8(o1, ks);
                 *reinterpret_cast<u32x2*>(kc + e + HD / 2) = quantise8(o2, ks);
@@ -629,8 +636,6 @@ struct StreamAttn : TileMath<HD, NB, NW, HIDDEN> {
             } else {
                 *reinterpret_cast<u32x4*>(kc + e * 2) = o1;
                 *reinterpret_cast<u32x4*>(kc + e * 2 + HD) = o2;
-                *reinterpret_cast<u32x4*>(vc + e * 2) = v1;
-                *reinterpret_cast<u32x4*>(vc + e * 2 + HD) = v2;
             }
         }
     }

@@ -417,25 +417,36 @@ def rope_queries_fns():
                            "angles, the query rows); the operand ring is free (between two items)."))
 
 
-def rope_row_fn():
+def rope_row_fn(with_v=False):
     """Rotary embedding of one pair of 16-byte chunks (c, c + 8) of a fresh K head row, in the blocks' registers:
-    the kernel's per-item rotation of the fresh K rows (the compiler's 32 registers would not hold it)."""
+    the kernel's per-item rotation of the fresh K rows (the compiler's 32 registers would not hold it).  with_v:
+    the same chunks of the V row travel with them, from v_chunk to v_dst (their cache slot, two-byte elements),
+    through registers of score set B: one trip to memory instead of two."""
     ins = [f"global_load_dwordx4 {vr(SA, 4)}, %[k], off", f"global_load_dwordx4 {vr(SA + 4, 4)}, %[k], off offset:{HD}",
            f"global_load_dwordx4 {vr(SA + 8, 4)}, %[t], off", f"global_load_dwordx4 {vr(SA + 12, 4)}, %[t], off offset:16",
            f"global_load_dwordx4 {vr(SA + 16, 4)}, %[t], off offset:{HD * 2}",
-           f"global_load_dwordx4 {vr(SA + 20, 4)}, %[t], off offset:{HD * 2 + 16}",
-           "s_waitcnt vmcnt(0)"]
+           f"global_load_dwordx4 {vr(SA + 20, 4)}, %[t], off offset:{HD * 2 + 16}"]
+    if with_v:
+        ins += [f"global_load_dwordx4 {vr(SB, 4)}, %[v], off", f"global_load_dwordx4 {vr(SB + 4, 4)}, %[v], off offset:{HD}"]
+    ins.append("s_waitcnt vmcnt(0)")
+    if with_v:
+        ins += [f"global_store_dwordx4 %[vd], {vr(SB, 4)}, off", f"global_store_dwordx4 %[vd], {vr(SB + 4, 4)}, off offset:{HD}"]
     for j in range(4):
         rotate_pairs(ins, SA + j, SA + 4 + j, SA + 8 + 2 * j, SA + 16 + 2 * j, SA + 24 + j, SA + 28 + j, TMP)
     ins += [f"v_mov_b32 %{j}, {vr(SA + 24 + j)}" for j in range(8)]
     outs = [f'"=v"(lo[{j}])' for j in range(4)] + [f'"=v"(hi[{j}])' for j in range(4)]
+    name = "pipe_rope_row_with_v" if with_v else "pipe_rope_row"
+    args = ", const void* v_chunk, void* v_dst" if with_v else ""
+    extra_ins = ', [v] "v"(v_chunk), [vd] "v"(v_dst)' if with_v else ""
+    extra_doc = ("\n// The same chunks of the V row go from v_chunk to v_dst (16 bytes each, HD bytes apart on both sides) in the same\n"
+                 "// trip to memory, through score set B." if with_v else "")
     return f'''// Rotates chunks c and c + 8 (16 bytes each, HD bytes apart) of the head row at `k_chunk` by the angles of
 // the table row at `table_chunk` (the position's row plus 8 c floats): the arithmetic of dfx_rope_kv_store, bit
-// for bit.  Uses score set A; waits for every load of the wave in flight.
-DFX_D void pipe_rope_row(const void* k_chunk, const void* table_chunk, uint32_t (&lo)[4], uint32_t (&hi)[4]) {{
+// for bit.  Uses score set A; waits for every load of the wave in flight.{extra_doc}
+DFX_D void {name}(const void* k_chunk, const void* table_chunk{args}, uint32_t (&lo)[4], uint32_t (&hi)[4]) {{
     asm volatile("{join(ins)}"
                  : {", ".join(outs)}
-                 : [k] "v"(k_chunk), [t] "v"(table_chunk)
+                 : [k] "v"(k_chunk), [t] "v"(table_chunk){extra_ins}
                  : "memory");
 }}
 
@@ -640,6 +651,7 @@ DFX_D u32x4 pipe_partial_chunk(int c) {
 ''')
     parts.append(rope_queries_fns())
     parts.append(rope_row_fn())
+    parts.append(rope_row_fn(with_v=True))
     for d in range(NDB):
         outs = [f'"=v"(x[{e}])' for e in range(16)]
         body = join(f"v_accvgpr_read_b32 %{e}, {ar(O_BASE + 16 * d + e)}" for e in range(16))

@@ -752,6 +752,25 @@ struct StreamAttn : TileMath<HD, NB, NW, HIDDEN> {
         asm volatile("" : "+s"(dbs));
         return (first_pos / dbs + 1) * dbs;
     }
+    // The same for the 32 rows of this wave alone (row_of(rt, 0) over its lanes), which is what decides whether
+    // the wave masks a tile: never below clear_limit() of the whole tile.  Negative (minus the limit) if the
+    // wave's rows do not all see the same keys -- with a diffusion block of 32 positions or a multiple and
+    // items that begin on a block boundary they do: every lane's visible_limit() is this value then, a tile
+    // is masked with one threshold for the wave, and the waves of a row tile that spans several blocks each
+    // mask only the tile their own block ends in.  A wave without rows: never masks.
+    DFX_D int wave_clear_limit(int rt, int q_len) const {
+        const int n_rows = a.group * q_len;
+        const int r_lo = rt * C::RT + wave * 32;
+        if (r_lo >= n_rows) return 0x7fffffff;
+        const int g_lo = r_lo / q_len;
+        const int p_lo = r_lo - g_lo * q_len;
+        const int p_hi = p_lo + min(31, n_rows - 1 - r_lo);  // in the head of the first row, if it is below q_len
+        int dbs = a.dbs;
+        asm volatile("" : "+s"(dbs));
+        if (p_hi >= q_len) return -dbs;  // several heads: position 0 is among the rows
+        const int clear = (p_lo / dbs + 1) * dbs;
+        return p_hi < clear ? clear : -clear;
+    }
     // Both at once, waiting for every outstanding load of the wave.
     DFX_D void begin_item_hidden(const UnitDesc& d) {
         request_queries(d);
@@ -1377,8 +1396,26 @@ paged_attn_pipe_kernel(const KArgs a) {
             }
             at.adopt_item(at.units[0]);
         }
+        // The wave's loads of unit u.  Without a cache every band is one of fresh rows, and a full one is fetched by
+        // the block the plain steps use (offsets per lane worked out once) instead of the general code.
+        auto issue_unit = [&](int u) {
+            if constexpr (PREFILL) {
+                const BandDesc& b = at.bands[u * NW + at.wave];
+                const int tag = uniform(b.is_ctx);
+                if (tag <= 0 && uniform(b.last) >= C::ROWS_PER_WAVE - 1) {
+                    const int64_t off = (static_cast<int64_t>(uniform(static_cast<int>(b.off >> 32))) << 32) |
+                                        static_cast<uint32_t>(uniform(static_cast<int>(b.off)));
+                    const int dst = uniform(static_cast<int>(at.stages_lds + (static_cast<unsigned>(u) % C::kStages) * C::STAGE_BYTES +
+                                                             at.wave * (C::IPW * 1024)));
+                    pipe_issue_band_fresh(reinterpret_cast<const uint8_t*>(a.k_new) + off,
+                                          reinterpret_cast<const uint8_t*>(a.v_new) + off + static_cast<int64_t>(-1 - tag) * a.v_fresh_delta, dst);
+                    return;
+                }
+            }
+            at.issue_unit(u);
+        };
         int issued = prefilled;  // ring fill: kStages - 1 units in flight
-        for (; issued < C::kStages - 1 && issued < n_units; ++issued) at.issue_unit(issued);
+        for (; issued < C::kStages - 1 && issued < n_units; ++issued) issue_unit(issued);
 
         auto tile_of = [&](int r) { return smem + C::STAGES_OFF + (static_cast<unsigned>(r) % C::kStages) * C::STAGE_BYTES; };
         // Unit r must have landed: only younger units may still be outstanding.  Behind the barrier
@@ -1399,14 +1436,21 @@ paged_attn_pipe_kernel(const KArgs a) {
         // Under the block-causal mask: the fresh key position up to which every query row of the current
         // run's row tile sees everything (set where a run begins).  A fresh tile that ends at or below it
         // needs no mask; in a prefill those are all of a row tile's tiles but the last few.
+        // That limit for the rows of this wave (wave_clear_limit(): negative if its rows differ in what they see).
         int bc_clear = 0;
         // Mask of the score set that holds unit r, if that tile needs one; updates the lane maximum.
         auto mask = [&](int r, bool set_a, float& mx_lane) {
             const TileInfo t = at.tile_info_of(r);
-            const bool bc = !t.is_ctx && a.mask_mode == DFX_MASK_BLOCK_CAUSAL && t.base + C::TN > bc_clear;
+            const int clear = bc_clear < 0 ? -bc_clear : bc_clear;
+            const bool bc = !t.is_ctx && a.mask_mode == DFX_MASK_BLOCK_CAUSAL && t.base + C::TN > clear;
             if (!(t.base + C::TN > t.limit || t.holes != 0 || bc)) return;
             int lim = t.limit;
-            if (bc) lim = min(lim, at.visible_limit(at.units[r]));
+            if (bc) lim = min(lim, bc_clear > 0 ? clear : at.visible_limit(at.units[r]));
+            if (bc && bc_clear > 0 && lim <= t.base) {  // the wave's rows see nothing of this tile
+                if (set_a) pipe_hide_a(mx_lane);
+                else pipe_hide_b(mx_lane);
+                return;
+            }
             const int thr = lim - t.base - (DISTINCT ? 8 : 4) * at.half;
             const uint32_t holes = static_cast<uint32_t>(t.holes);
             if (set_a) {
@@ -1424,10 +1468,10 @@ paged_attn_pipe_kernel(const KArgs a) {
             const UnitDesc d = at.units[rel];
             const int run_end = min(rel + uniform(d.run), n_units);
             // (an item that opens inside the chunk was adopted when the run before it ended)
-            if (a.mask_mode == DFX_MASK_BLOCK_CAUSAL) bc_clear = uniform(at.clear_limit(uniform(d.rt), uniform(d.q_len)));
+            if (a.mask_mode == DFX_MASK_BLOCK_CAUSAL) bc_clear = uniform(at.wave_clear_limit(uniform(d.rt), uniform(d.q_len)));
 
             // S^T of the run's first tile (into score set A), with nothing to overlap it with
-            if (admit(rel, rel)) at.issue_unit(issued++);
+            if (admit(rel, rel)) issue_unit(issued++);
             // For the plain steps behind the run's first step (below), read now, with the first tile's
             // matrix work between the reads and their use: how many there are, and the band offset
             // of the unit the first of them fetches (in steady state, which is checked there, step
@@ -1485,7 +1529,7 @@ paged_attn_pipe_kernel(const KArgs a) {
                 const bool ask_queries = next_opens && r + 2 == run_end;
                 queries_asked = queries_asked || ask_queries;
                 if (!compute_first || !busy) {
-                    if (fetch) at.issue_unit(issued);
+                    if (fetch) issue_unit(issued);
                     if (busy) prepare();
                 }
                 if (!busy && ask_queries) at.request_queries(at.units[run_end]);
@@ -1513,7 +1557,7 @@ paged_attn_pipe_kernel(const KArgs a) {
                         }
                     }
                     if (compute_first) {
-                        if (fetch) at.issue_unit(issued);
+                        if (fetch) issue_unit(issued);
                         if (has_next) prepare();
                     }
                 }

@@ -697,6 +697,11 @@ DFX_D void pipe_set_output(int db, const f32x16& v) {
 DFX_D void pipe_outputs_ready() { asm volatile("s_nop 15\\n\\ts_nop 1" ::: "memory"); }
 
 ''')
+    for nm, s in (("a", SA), ("b", SB)):
+        hide = [f"v_mov_b32 {vr(s)}, {NEG_INF}"] + [f"v_mov_b32 {vr(s + j)}, {vr(s)}" for j in range(1, 32)] + [f"v_mov_b32 %[mx], {vr(s)}"]
+        parts.append(asm_fn(f"pipe_hide_{nm}", "float& mx", join(hide), ['[mx] "=&v"(mx)'], [], [],
+                            f"Score set {nm.upper()} of a tile the wave's rows see nothing of: every score and the lane's maximum -inf (what the\n"
+                            "mask blocks make of such a tile; any tile layout and head_dim).  The set's matrix results are ready."))
     global LAYOUT
     for LAYOUT, pre, what in (("u", "pipe_", ""), ("d", "pipe_d_", "  Tiles of a cache in the distinct layout.")):
         parts.append(asm_fn(pre + "first_scores", "uint32_t k_next, float& mx", first_scores_block(SA),

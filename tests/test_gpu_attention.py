@@ -879,6 +879,39 @@ def test_block_causal_prefill_without_a_cache(dev):
         assert max_abs_err(got, want) <= ATOL_BF16
 
 
+@pytest.mark.parametrize("case", [
+    # (lengths, query heads, KV heads, head_dim, diffusion block size)
+    ((40, 100, 333), 14, 2, 128, 8),      # lengths that are no multiple of a wave's 32 rows: waves whose rows span two heads
+    ((96, 200), 8, 2, 128, 48),           # blocks of 48 positions: waves whose rows span two blocks
+    ((64, 512, 31), 8, 1, 128, 16),       # two blocks per wave
+    ((300,), 28, 4, 128, 96),
+    ((640, 1024), 14, 2, 128, 32),        # a block per wave, row tiles of eight blocks: waves that see nothing of a tile
+    ((640, 130), 8, 2, 128, 64),          # two waves per block
+    ((200, 577), 16, 2, 64, 32),
+    ((100, 72), 8, 2, 64, 24),
+])
+def test_block_causal_prefill_where_the_waves_of_a_row_tile_see_different_keys(dev, case):
+    """The pipelined kernel decides per wave whether a tile needs the block-causal mask, masks with one threshold
+    where all of a wave's rows see the same keys and row by row where they do not: block sizes below, at and
+    above a wave's 32 rows, lengths that put the rows of two heads or two blocks into one wave."""
+    from oracle import attention as oat
+    lengths, hq, hkv, hd, dbs = case
+    T = sum(lengths)
+    g = torch.Generator().manual_seed(T + dbs)
+    q = torch.randn(T, hq, hd, generator=g).to(torch.bfloat16)
+    k = torch.randn(T, hkv, hd, generator=g).to(torch.bfloat16)
+    v = torch.randn(T, hkv, hd, generator=g).to(torch.bfloat16)
+    cu = torch.tensor([0] + list(np.cumsum(lengths)), dtype=torch.int32)
+    want = oat.paged_attention_fp32(q, k, v, None, None, None, None, cu, cu, hd ** -0.5, mask_mode=MASK_BLOCK_CAUSAL, dbs=dbs)
+    for max_wg in (0, 5):
+        got = dfx.paged_attention(q.to(dev), k.to(dev), v.to(dev), None, None, hd ** -0.5, block_tables=None, context_lens=None,
+                                  cu_seqlens_q=cu.to(dev), cu_seqlens_new=cu.to(dev), max_seqlen_q=max(lengths),
+                                  mask_mode=MASK_BLOCK_CAUSAL, diffusion_block_size=dbs, max_workgroups=max_wg)
+        torch.cuda.synchronize()
+        assert torch.isfinite(got.float()).all()
+        assert max_abs_err(got, want) <= ATOL_BF16
+
+
 @pytest.mark.parametrize("mask", [MASK_FULL, MASK_BLOCK_CAUSAL])
 def test_prefill_with_v_sliced_out_of_the_projection(dev, mask):
     """A prefill as a decoder layer issues it: K rotated into a buffer of its own, V still a column slice of the

@@ -1436,20 +1436,28 @@ paged_attn_pipe_kernel(const KArgs a) {
         // Under the block-causal mask: the fresh key position up to which every query row of the current
         // run's row tile sees everything (set where a run begins).  A fresh tile that ends at or below it
         // needs no mask; in a prefill those are all of a row tile's tiles but the last few.
-        // That limit for the rows of this wave (wave_clear_limit(): negative if its rows differ in what they see).
+        // Without a cache (where the staircases are: row tiles of eight diffusion blocks) that limit is the one of
+        // this wave's rows (wave_clear_limit(): negative if its rows differ in what they see): one threshold for the
+        // wave where they agree, and no mask block for a tile it sees nothing of.  The other variants keep the limit of
+        // the row tile and the row-by-row threshold: the second way to the limit costs their tile loop scalar
+        // registers, which the compiler then keeps in vector lanes (C3, which masks nothing, +0.7 %).
         int bc_clear = 0;
         // Mask of the score set that holds unit r, if that tile needs one; updates the lane maximum.
         auto mask = [&](int r, bool set_a, float& mx_lane) {
             const TileInfo t = at.tile_info_of(r);
-            const int clear = bc_clear < 0 ? -bc_clear : bc_clear;
+            const int clear = PREFILL && bc_clear < 0 ? -bc_clear : bc_clear;
             const bool bc = !t.is_ctx && a.mask_mode == DFX_MASK_BLOCK_CAUSAL && t.base + C::TN > clear;
             if (!(t.base + C::TN > t.limit || t.holes != 0 || bc)) return;
             int lim = t.limit;
-            if (bc) lim = min(lim, bc_clear > 0 ? clear : at.visible_limit(at.units[r]));
-            if (bc && bc_clear > 0 && lim <= t.base) {  // the wave's rows see nothing of this tile
-                if (set_a) pipe_hide_a(mx_lane);
-                else pipe_hide_b(mx_lane);
-                return;
+            if constexpr (PREFILL) {
+                if (bc) lim = min(lim, bc_clear > 0 ? clear : at.visible_limit(at.units[r]));
+                if (bc && bc_clear > 0 && lim <= t.base) {  // the wave's rows see nothing of this tile
+                    if (set_a) pipe_hide_a(mx_lane);
+                    else pipe_hide_b(mx_lane);
+                    return;
+                }
+            } else {
+                if (bc) lim = min(lim, at.visible_limit(at.units[r]));
             }
             const int thr = lim - t.base - (DISTINCT ? 8 : 4) * at.half;
             const uint32_t holes = static_cast<uint32_t>(t.holes);
@@ -1468,7 +1476,8 @@ paged_attn_pipe_kernel(const KArgs a) {
             const UnitDesc d = at.units[rel];
             const int run_end = min(rel + uniform(d.run), n_units);
             // (an item that opens inside the chunk was adopted when the run before it ended)
-            if (a.mask_mode == DFX_MASK_BLOCK_CAUSAL) bc_clear = uniform(at.wave_clear_limit(uniform(d.rt), uniform(d.q_len)));
+            if (a.mask_mode == DFX_MASK_BLOCK_CAUSAL)
+                bc_clear = uniform(PREFILL ? at.wave_clear_limit(uniform(d.rt), uniform(d.q_len)) : at.clear_limit(uniform(d.rt), uniform(d.q_len)));
 
             // S^T of the run's first tile (into score set A), with nothing to overlap it with
             if (admit(rel, rel)) issue_unit(issued++);
